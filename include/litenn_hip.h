@@ -1,0 +1,213 @@
+/*
+ * litenn_hip.h -- C ABI of the MI355X (gfx950) device backend for LiteNN's
+ * GGUF-quantised LLaMA path.
+ *
+ * The first group of entry points is what a DeviceTraits<HIP> specialisation
+ * binds, one call per static member of the reference's Device concept
+ * (src/LiteNN/Device.h:17-69), modelled on DeviceTraits<CUDA>
+ * (src/LiteNN/Device/CUDA.h:98-165).  The second group are extensions the
+ * reference has no counterpart for, because it dequantises GGUF blocks to f32
+ * on the host at lowering time (tools/gguf/LLaMABuilder.cpp:66-162): they
+ * consume the raw block payload exactly as the importer stores it
+ * (tools/gguf/GGUFImporter.cpp:478-491).  The third group is the decoder
+ * runtime that replaces "lower a static graph per (sequenceLength,
+ * pastLength) and interpret it" (tools/gguf/LLaMABuilder.cpp:826-872,
+ * src/LiteNN/Runtime/Interpreter.h:35-43).
+ *
+ * Conventions
+ *  - every function returns 0 on success and a non-zero status otherwise;
+ *    litenn_hip_last_error() then holds "<action> failed: <message>" for the
+ *    calling thread (the reference throws std::runtime_error with that text,
+ *    src/LiteNN/Device/CUDA.cpp:89-95).
+ *  - `dtype` uses DataType's positional values (src/LiteNN/DType.h:17-30),
+ *    `fmt` uses QuantizedBlockFormat's (src/LiteNN/Quantization.h:31-62).
+ *  - sizes are ELEMENT counts, never bytes (src/LiteNN/Device.h:28-31).
+ *  - tensors are row-major and contiguous.
+ *  - `opts` mirrors CUDAExecutionOptions (src/LiteNN/Device/CUDA.h:70-74):
+ *    NULL means stream 0 and synchronise before returning.
+ *  - all entry points are thread-safe; each call selects `dev` for its own
+ *    duration (cf. CUDADeviceGuard, src/LiteNN/Device/CUDA.cpp:734-761).
+ */
+#ifndef LITENN_HIP_H
+#define LITENN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* DataType, src/LiteNN/DType.h:17-30 */
+enum litenn_dtype {
+	LITENN_F32 = 0, LITENN_F64 = 1, LITENN_I32 = 2, LITENN_I64 = 3, LITENN_BOOL = 4, LITENN_F16 = 5,
+	LITENN_BF16 = 6, LITENN_F8E4M3 = 7, LITENN_F8E5M2 = 8, LITENN_I8 = 9, LITENN_U8 = 10,
+};
+
+/* QuantizedBlockFormat, src/LiteNN/Quantization.h:31-62 (only the members this backend executes) */
+enum litenn_block_format {
+	LITENN_FMT_Q4_0 = 1, LITENN_FMT_Q8_0 = 5, LITENN_FMT_Q4_K = 9, LITENN_FMT_Q6_K = 11,
+	LITENN_FMT_F16 = 25, LITENN_FMT_F32 = 27,
+};
+
+/* UnaryOp / BinaryOp / ReduceOp, src/LiteNN/Operators.h:12-51,237-242 */
+enum litenn_unary_op {
+	LITENN_UN_NEGATE = 0, LITENN_UN_ABS, LITENN_UN_SQRT, LITENN_UN_EXP, LITENN_UN_LOG, LITENN_UN_SIN, LITENN_UN_COS,
+	LITENN_UN_TAN, LITENN_UN_ARCSIN, LITENN_UN_ARCCOS, LITENN_UN_ARCTAN, LITENN_UN_TRANSPOSE,
+	LITENN_UN_LOGICAL_NEGATION, LITENN_UN_ERF,
+};
+enum litenn_binary_op {
+	LITENN_BIN_ADD = 0, LITENN_BIN_SUBTRACT, LITENN_BIN_MULTIPLY, LITENN_BIN_DIVIDE, LITENN_BIN_MATMUL, LITENN_BIN_POW,
+	LITENN_BIN_MAX, LITENN_BIN_MIN, LITENN_BIN_LESS, LITENN_BIN_GREATER, LITENN_BIN_EQUAL,
+};
+enum litenn_reduce_op { LITENN_RED_SUM = 0, LITENN_RED_MEAN = 1, LITENN_RED_MAX = 2 };
+
+/* CUDAExecutionOptions, src/LiteNN/Device/CUDA.h:70-74 */
+typedef struct litenn_hip_exec {
+	void* stream;    /* hipStream_t, NULL = null stream */
+	int synchronize; /* non-zero: hipStreamSynchronize before returning */
+} litenn_hip_exec;
+
+const char* litenn_hip_last_error(void);
+
+/* ---- group 1: the Device concept ------------------------------------- */
+
+/* CUDADeviceCount, src/LiteNN/Device/CUDA.cpp:1400-1416.  Never fails; 0 when no GPU. */
+int litenn_hip_device_count(void);
+/* DeviceTraits<CUDA>::Info, src/LiteNN/Device/CUDA.cpp:1735-1751 */
+int litenn_hip_device_info(int dev, char* buf, size_t buf_len);
+/* Allocate / Deallocate / ZeroFill, src/LiteNN/Device.h:28-34, CUDA.cpp:1753-1777.
+ * Memory is uninitialised; the caller frees with the same (dtype, n). */
+int litenn_hip_alloc(int dev, int dtype, size_t n, void** out);
+int litenn_hip_free(int dev, void* ptr, int dtype, size_t n);
+int litenn_hip_zero(int dev, void* ptr, int dtype, size_t n);
+/* CopyToCPU / CopyFromCPU / ConvertTo, src/LiteNN/Device.h:35-39, CUDA.cpp:1785-1892.
+ * Synchronous on return unless opts says otherwise; dtype may change. */
+int litenn_hip_copy_to_host(int dev, int src_dtype, const void* src, size_t n, int dst_dtype, void* dst,
+                            const litenn_hip_exec* opts);
+int litenn_hip_copy_from_host(int dev, int dst_dtype, void* dst, int src_dtype, const void* src, size_t n,
+                              const litenn_hip_exec* opts);
+int litenn_hip_convert(int dev, int src_dtype, const void* src, size_t n, int dst_dtype, void* dst,
+                       const litenn_hip_exec* opts);
+/* DoUnaryOp, src/LiteNN/Device.h:42-44 (CPU semantics :393-511) */
+int litenn_hip_unary(int dev, int op, void* dst, int dtype, const size_t* shape, size_t rank, const void* src,
+                     const litenn_hip_exec* opts);
+/* DoBinaryOp, src/LiteNN/Device.h:45-49 (CPU semantics :513-689; MatMul :628-660).
+ * Broadcast aligns LEADING dimensions (src/LiteNN/Operators.h:173-188). */
+int litenn_hip_binary(int dev, int op, void* dst, int dtype1, const size_t* shape1, size_t rank1, const void* src1,
+                      int dtype2, const size_t* shape2, size_t rank2, const void* src2, const litenn_hip_exec* opts);
+/* DoReduceOp, src/LiteNN/Device.h:50-52 (:691-759) */
+int litenn_hip_reduce(int dev, int op, void* dst, int dtype, const size_t* shape, size_t rank, const void* src,
+                      size_t axis, const litenn_hip_exec* opts);
+/* DoConcatOp, src/LiteNN/Device.h:53-58 (:761-792).  shapes is input_count rows of `rank` extents. */
+int litenn_hip_concat(int dev, void* dst, int dtype, const void* const* srcs, const size_t* shapes, size_t rank,
+                      size_t input_count, size_t axis, const litenn_hip_exec* opts);
+/* DoSliceOp, src/LiteNN/Device.h:59-60 (:794-823) */
+int litenn_hip_slice(int dev, void* dst, int dtype, const size_t* src_shape, size_t rank, const void* src, size_t axis,
+                     size_t start, size_t length, const litenn_hip_exec* opts);
+/* DoGetRowsOp, src/LiteNN/Device.h:61-64 (:825-883).  index_dtype is I32 or I64; an
+ * out-of-range index fails with "GetRows index out of range". */
+int litenn_hip_get_rows(int dev, void* dst, int dtype, const size_t* data_shape, size_t data_rank, const void* data,
+                        int index_dtype, const size_t* index_shape, size_t index_rank, const void* indices,
+                        const litenn_hip_exec* opts);
+/* DoPermuteOp, src/LiteNN/Device.h:65-68 (:885-966).  perm[d] = input axis of output axis d. */
+int litenn_hip_permute(int dev, void* dst, int dtype, const size_t* src_shape, size_t rank, const void* src,
+                       const size_t* perm, const litenn_hip_exec* opts);
+
+/* ---- group 2: quantised extensions (no reference counterpart) -------- */
+
+/* y[m, n] (f32) = x[m, k] . deq(wq)[n, k]^T with f32 accumulation, i.e. the value
+ * AddLinear produces after the lowering's dequantise + transpose
+ * (tools/gguf/LLaMABuilder.cpp:144-150,225-230; src/LiteNN/Layer/Linear.h:67-95).
+ * wq is the raw GGUF payload: n rows of k/block blocks.  x_dtype is F32.
+ * residual (f32 [m, n]) may be NULL; when given, y = residual + x.W
+ * (the Add at tools/gguf/LLaMABuilder.cpp:652-653,661-663).  residual may alias y.
+ * m == 1..15 runs the streaming GEMV; m >= 16 runs the MFMA GEMM unless
+ * LITENN_HIP_MATMUL_PRECISE is set in `flags`, which keeps f32 activations. */
+#define LITENN_HIP_MATMUL_PRECISE 1u
+int litenn_hip_mul_mat_q(int dev, int fmt, const void* wq, size_t n, size_t k, const void* x, int x_dtype, size_t m,
+                         void* y, const void* residual, unsigned flags, const litenn_hip_exec* opts);
+/* f32 [rows, k] = dequantised rows of wq (ggml to_float as called at
+ * tools/gguf/LLaMABuilder.cpp:144-150). */
+int litenn_hip_dequantize(int dev, int fmt, const void* wq, size_t rows, size_t k, void* dst,
+                          const litenn_hip_exec* opts);
+/* out[i, :] = deq(table)[ids[i], :]; ids are I32 on the device
+ * (AddLLaMATokenEmbedding, tools/gguf/LLaMABuilder.cpp:738-759). */
+int litenn_hip_get_rows_q(int dev, int fmt, const void* table, size_t rows, size_t k, const void* ids, size_t n_ids,
+                          void* out, const litenn_hip_exec* opts);
+/* RMSNorm over the last axis with f64 accumulation: y = x / sqrt(mean(x^2) + eps) * w
+ * (src/LiteNN/Layer/RMSNorm.h:41-57, src/LiteNN/ComputePrimitives.h:792-817).  w may be NULL. */
+int litenn_hip_rmsnorm(int dev, const void* x, const void* w, double eps, size_t m, size_t d, void* y,
+                       const litenn_hip_exec* opts);
+/* Interleaved-pair RoPE on x[m, n_heads, head_dim] (f32) at positions pos_offset + row,
+ * first rope_dims features of every head, tail copied
+ * (src/LiteNN/Layer/RoPE.h:24-117, tools/gguf/LLaMABuilder.cpp:311-348). */
+int litenn_hip_rope_interleaved(int dev, const void* x, void* y, size_t m, size_t n_heads, size_t head_dim,
+                                size_t rope_dims, double base, double freq_scale, size_t pos_offset,
+                                const litenn_hip_exec* opts);
+/* cache[past + i, :] = convert(cur[i, :]) for i < m; cache dtype F16 or F32
+ * (AddKVCacheAppend, src/LiteNN/Layer/KVCache.h:87-104; f32 -> Float16 rounding of
+ * src/LiteNN/DType.h:63-110). */
+int litenn_hip_kv_append(int dev, void* cache, int cache_dtype, size_t past, const void* cur, size_t m, size_t width,
+                         const litenn_hip_exec* opts);
+/* Causal attention of m query rows at positions past..past+m-1 against a cache holding
+ * past+m rows: q [m, n_head, head_dim] f32 (already rotated), k/v cache
+ * [>= past+m, n_kv_head, head_dim] F16 or F32, out [m, n_head, head_dim] f32; scale
+ * 1/sqrt(head_dim); query head h reads kv head h / (n_head / n_kv_head)
+ * (tools/gguf/LLaMABuilder.cpp:624-645, src/LiteNN/Layer/FlashAttnExt.h:126-228). */
+int litenn_hip_attn_decode(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
+                           size_t past, size_t n_head, size_t n_kv_head, size_t head_dim, void* out,
+                           const litenn_hip_exec* opts);
+/* y = silu(gate) * up (src/LiteNN/Layer/SwiGLU.h:59-69, Activation.h:22-63) */
+int litenn_hip_silu_mul(int dev, const void* gate, const void* up, void* y, size_t n, const litenn_hip_exec* opts);
+/* out_index[row] (I32) = first maximal index of x[row, :] (f32); ties pick the lowest index
+ * (cf. the stable sort at src/LiteNN/Runtime/Interpreter.h:134-163). */
+int litenn_hip_argmax(int dev, const void* x, size_t rows, size_t n, void* out_index, const litenn_hip_exec* opts);
+
+/* ---- group 3: LLaMA decoder runtime ----------------------------------- */
+
+typedef struct litenn_hip_llama litenn_hip_llama;
+
+/* tensor ids for litenn_hip_llama_set_tensor; shapes are GGUF [n, k] = [out, in] */
+enum litenn_llama_tensor {
+	LITENN_T_TOKEN_EMBD = 0, LITENN_T_OUTPUT = 1, LITENN_T_ATTN_Q = 2, LITENN_T_ATTN_K = 3, LITENN_T_ATTN_V = 4,
+	LITENN_T_ATTN_OUTPUT = 5, LITENN_T_FFN_GATE = 6, LITENN_T_FFN_UP = 7, LITENN_T_FFN_DOWN = 8,
+	LITENN_T_OUTPUT_NORM = 9, LITENN_T_ATTN_NORM = 10, LITENN_T_FFN_NORM = 11,
+};
+
+/* Hyper-parameters as ParseLLaMAHyperparameters yields them
+ * (tools/gguf/GGUFImporter.cpp:505-642).  kv_dtype is F16 or F32. */
+typedef struct litenn_hip_llama_params {
+	int32_t block_count, embedding_length, head_count, head_count_kv, feed_forward_length, vocab_size,
+	    context_length, rope_dimension_count;
+	double rms_norm_epsilon, rope_freq_base, rope_freq_scale;
+	int32_t kv_dtype;
+} litenn_hip_llama_params;
+
+int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* params, litenn_hip_llama** out);
+int litenn_hip_llama_free(litenn_hip_llama* model);
+/* `data` is DEVICE memory holding the raw payload (or f32 for the norm weights); it is
+ * referenced, not copied, and must outlive the model.  LITENN_T_OUTPUT may be left unset:
+ * the head is then tied to token_embd (tools/gguf/LLaMABuilder.cpp:719-733). */
+int litenn_hip_llama_set_tensor(litenn_hip_llama* model, int which, int layer, int fmt, const void* data, size_t n,
+                                size_t k);
+int litenn_hip_llama_reset(litenn_hip_llama* model);
+int litenn_hip_llama_past(const litenn_hip_llama* model);
+/* LowerLLaMACausalLMDecode(sequenceLength = m, pastLength = positionOffset = past) executed
+ * against the cache the model holds (tools/gguf/LLaMABuilder.cpp:826-872); tokens are host
+ * I32.  logits (host f32 [m, vocab]) and last_logits (host f32 [vocab]) may be NULL.
+ * flags: LITENN_HIP_MATMUL_PRECISE keeps f32 activations for m >= 16. */
+int litenn_hip_llama_eval(litenn_hip_llama* model, const int32_t* tokens, size_t m, float* logits, float* last_logits,
+                          unsigned flags);
+/* Greedy loop kept on the device: eval(prompt), then n_new times argmax -> eval of that
+ * token.  out_tokens is host I32 [n_new].  decode_ms (may be NULL) receives the
+ * device time of the n_new - 1 single-token steps. */
+int litenn_hip_llama_generate(litenn_hip_llama* model, const int32_t* prompt, size_t n_prompt, size_t n_new,
+                              int32_t* out_tokens, unsigned flags, double* prefill_ms, double* decode_ms);
+/* Copies the first `past` cache rows of one layer to host as f32 [past, n_kv_head*head_dim]. */
+int litenn_hip_llama_get_kv(litenn_hip_llama* model, int layer, float* k, float* v);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,65 @@
+"""Compiles the HIP sources of this package into lib/liblitenn_hip.so for gfx950."""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_DIR = os.path.join(HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "liblitenn_hip.so")
+
+SOURCES = ["api.hip", "gemv.hip", "gemm.hip", "glue.hip", "primitives.hip", "llama.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    # packed-FP32 instruction selection is switched off for every device function
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
+]
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; the HIP backend cannot be built")
+    return exe
+
+
+def build(verbose: bool = True, jobs: int = 6) -> str:
+    """Compile every source (always, even if a library is already present) and link."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    obj_dir = os.path.join(HERE, "build")
+    os.makedirs(obj_dir, exist_ok=True)
+    procs, objs = [], []
+    for src in SOURCES:
+        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
+        objs.append(obj)
+        cmd = [hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        while sum(p.poll() is None for _, p in procs) >= jobs:
+            procs[0][1].wait()
+    failed = False
+    for src, p in procs:
+        out, _ = p.communicate()
+        out = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l and l.strip())
+        if p.returncode != 0:
+            failed = True
+            print(f"--- {src} failed ---\n{out}", file=sys.stderr)
+        elif verbose and out:
+            print(out)
+    if failed:
+        raise RuntimeError("hipcc failed")
+    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", LIB_PATH]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build()

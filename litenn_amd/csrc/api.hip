@@ -1,0 +1,749 @@
+// C ABI: error state, device management, memory, dtype conversion, and the quantised
+// extension entry points.  Host-side validation lives here so that no kernel is ever
+// launched on operands whose shapes it does not expect.
+#include "common.hpp"
+
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+namespace litenn_hip
+{
+	// launchers defined in gemv.hip / gemm.hip / glue.hip
+	int launch_gemv(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
+	                const float* residual, hipStream_t stream);
+	int launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
+	                const float* residual, hipStream_t stream);
+	void launch_dequantize(int fmt, const void* wq, size_t rows, size_t k, float* dst, hipStream_t stream);
+	void launch_get_rows_q(int fmt, const void* table, size_t rows, size_t k, const int32_t* ids, size_t n_ids,
+	                       float* out, int* err_flag, hipStream_t stream);
+	void launch_rmsnorm(const float* x, const float* w, double eps, size_t m, size_t d, float* y, hipStream_t s);
+	void launch_rope_table(float* cos_t, float* sin_t, size_t positions, size_t half, double base, double freq_scale,
+	                       size_t pos_offset, hipStream_t s);
+	void launch_rope(const float* x, float* y, size_t m, size_t n_heads, size_t head_dim, size_t rope_dims,
+	                 const float* cos_t, const float* sin_t, hipStream_t s);
+	void launch_kv_append(void* cache, int cache_dtype, size_t past_elems, const float* cur, size_t count,
+	                      hipStream_t s);
+	void launch_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
+	                        const int* past_dev, size_t past_host, size_t max_len, size_t n_head, size_t n_kv_head,
+	                        size_t head_dim, float* out, hipStream_t s);
+	void launch_silu_mul(const float* gate, const float* up, float* y, size_t n, hipStream_t s);
+	void launch_argmax(const float* x, size_t rows, size_t n, int32_t* out, hipStream_t s);
+
+	// ---- error state -----------------------------------------------------------------------
+	static thread_local std::string g_error;
+
+	void set_error(const std::string& message) { g_error = message; }
+
+	int fail(const char* action, const std::string& message)
+	{
+		// same text shape as the reference's ThrowCUDAError (Device/CUDA.cpp:89-95)
+		g_error = std::string(action) + " failed: " + message;
+		return 1;
+	}
+
+	int fail_hip(const char* action, hipError_t err)
+	{
+		(void)hipGetLastError(); // clear the sticky launch error so the next call starts clean
+		return fail(action, hipGetErrorString(err));
+	}
+
+	DeviceGuard::DeviceGuard(int dev)
+	{
+		int count = 0;
+		err_ = hipGetDeviceCount(&count);
+		if (err_ != hipSuccess)
+		{
+			return;
+		}
+		if (dev < 0 || dev >= count)
+		{
+			err_ = hipErrorInvalidDevice;
+			return;
+		}
+		err_ = hipGetDevice(&previous_);
+		if (err_ != hipSuccess)
+		{
+			return;
+		}
+		if (previous_ != dev)
+		{
+			err_ = hipSetDevice(dev);
+			if (err_ != hipSuccess)
+			{
+				return;
+			}
+		}
+		else
+		{
+			previous_ = -1; // nothing to restore
+		}
+		ok_ = true;
+	}
+
+	DeviceGuard::~DeviceGuard()
+	{
+		if (ok_ && previous_ >= 0)
+		{
+			(void)hipSetDevice(previous_);
+		}
+	}
+
+	int finish(const char* action, const litenn_hip_exec* opts)
+	{
+		LITENN_HIP_TRY(action, hipGetLastError());
+		if (!opts || opts->synchronize)
+		{
+			LITENN_HIP_TRY(action, hipStreamSynchronize(stream_of(opts)));
+		}
+		return 0;
+	}
+
+	size_t dtype_size(int dtype)
+	{
+		switch (dtype)
+		{
+		case LITENN_F32:
+		case LITENN_I32:
+			return 4;
+		case LITENN_F64:
+		case LITENN_I64:
+			return 8;
+		case LITENN_F16:
+		case LITENN_BF16:
+			return 2;
+		case LITENN_BOOL:
+		case LITENN_F8E4M3:
+		case LITENN_F8E5M2:
+		case LITENN_I8:
+		case LITENN_U8:
+			return 1;
+		default:
+			return 0;
+		}
+	}
+
+	int block_elements(int fmt)
+	{
+		switch (fmt)
+		{
+		case LITENN_FMT_Q4_0:
+		case LITENN_FMT_Q8_0:
+			return 32;
+		case LITENN_FMT_Q4_K:
+		case LITENN_FMT_Q6_K:
+			return 256;
+		case LITENN_FMT_F16:
+		case LITENN_FMT_F32:
+			return 1;
+		default:
+			return 0;
+		}
+	}
+
+	int block_bytes(int fmt)
+	{
+		switch (fmt)
+		{
+		case LITENN_FMT_Q4_0:
+			return 18;
+		case LITENN_FMT_Q8_0:
+			return 34;
+		case LITENN_FMT_Q4_K:
+			return 144;
+		case LITENN_FMT_Q6_K:
+			return 210;
+		case LITENN_FMT_F16:
+			return 2;
+		case LITENN_FMT_F32:
+			return 4;
+		default:
+			return 0;
+		}
+	}
+
+	size_t row_bytes(int fmt, size_t k)
+	{
+		const int be = block_elements(fmt);
+		if (be == 0 || k % static_cast<size_t>(be) != 0)
+		{
+			return 0;
+		}
+		return k / static_cast<size_t>(be) * static_cast<size_t>(block_bytes(fmt));
+	}
+
+	// ---- dtype conversion --------------------------------------------------------------------
+	namespace
+	{
+		struct F16 { uint16_t bits; };
+		struct BF16 { uint16_t bits; };
+
+		template <typename T>
+		__device__ __forceinline__ double load_as_double(const T* p, size_t i) { return static_cast<double>(p[i]); }
+		template <>
+		__device__ __forceinline__ double load_as_double<F16>(const F16* p, size_t i)
+		{
+			return static_cast<double>(f16_bits_to_f32(p[i].bits));
+		}
+		template <>
+		__device__ __forceinline__ double load_as_double<BF16>(const BF16* p, size_t i)
+		{
+			return static_cast<double>(__uint_as_float(static_cast<uint32_t>(p[i].bits) << 16));
+		}
+
+		template <typename S>
+		struct IsInt { static constexpr bool value = false; };
+		template <> struct IsInt<int32_t> { static constexpr bool value = true; };
+		template <> struct IsInt<int64_t> { static constexpr bool value = true; };
+		template <> struct IsInt<int8_t> { static constexpr bool value = true; };
+		template <> struct IsInt<uint8_t> { static constexpr bool value = true; };
+		template <> struct IsInt<bool> { static constexpr bool value = true; };
+
+		// static_cast<Dst>(src) for every pair, with LiteNN's own Float16 / BFloat16 constructors
+		// (via float; DType.h:63-110, :136-141).
+		template <typename S, typename D>
+		__device__ __forceinline__ void convert_one(const S* src, D* dst, size_t i)
+		{
+			if constexpr (IsInt<S>::value && IsInt<D>::value)
+			{
+				dst[i] = static_cast<D>(src[i]);
+			}
+			else
+			{
+				dst[i] = static_cast<D>(load_as_double<S>(src, i));
+			}
+		}
+		template <typename S>
+		__device__ __forceinline__ void convert_one(const S* src, F16* dst, size_t i)
+		{
+			dst[i].bits = f32_to_f16_bits_litenn(static_cast<float>(load_as_double<S>(src, i)));
+		}
+		template <typename S>
+		__device__ __forceinline__ void convert_one(const S* src, BF16* dst, size_t i)
+		{
+			const uint32_t bits = __float_as_uint(static_cast<float>(load_as_double<S>(src, i)));
+			const uint32_t lsb = (bits >> 16) & 1u;
+			dst[i].bits = static_cast<uint16_t>((bits + 0x7fffu + lsb) >> 16);
+		}
+
+		template <typename S, typename D>
+		__global__ void convert_kernel(const S* __restrict__ src, D* __restrict__ dst, size_t n)
+		{
+			const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+			if (i < n)
+			{
+				convert_one(src, dst, i);
+			}
+		}
+
+		template <typename S>
+		bool convert_from(const void* src, int dst_dtype, void* dst, size_t n, hipStream_t s)
+		{
+			const dim3 grid((n + 255) / 256), block(256);
+			const S* sp = static_cast<const S*>(src);
+			switch (dst_dtype)
+			{
+			case LITENN_F32: convert_kernel<S, float><<<grid, block, 0, s>>>(sp, static_cast<float*>(dst), n); return true;
+			case LITENN_F64: convert_kernel<S, double><<<grid, block, 0, s>>>(sp, static_cast<double*>(dst), n); return true;
+			case LITENN_I32: convert_kernel<S, int32_t><<<grid, block, 0, s>>>(sp, static_cast<int32_t*>(dst), n); return true;
+			case LITENN_I64: convert_kernel<S, int64_t><<<grid, block, 0, s>>>(sp, static_cast<int64_t*>(dst), n); return true;
+			case LITENN_BOOL: convert_kernel<S, bool><<<grid, block, 0, s>>>(sp, static_cast<bool*>(dst), n); return true;
+			case LITENN_F16: convert_kernel<S, F16><<<grid, block, 0, s>>>(sp, static_cast<F16*>(dst), n); return true;
+			case LITENN_BF16: convert_kernel<S, BF16><<<grid, block, 0, s>>>(sp, static_cast<BF16*>(dst), n); return true;
+			case LITENN_I8: convert_kernel<S, int8_t><<<grid, block, 0, s>>>(sp, static_cast<int8_t*>(dst), n); return true;
+			case LITENN_U8: convert_kernel<S, uint8_t><<<grid, block, 0, s>>>(sp, static_cast<uint8_t*>(dst), n); return true;
+			default: return false;
+			}
+		}
+	} // namespace
+
+	// device -> device conversion; false when a dtype is not executed by this backend (fp8)
+	bool launch_convert(int src_dtype, const void* src, size_t n, int dst_dtype, void* dst, hipStream_t s)
+	{
+		if (n == 0)
+		{
+			return true;
+		}
+		switch (src_dtype)
+		{
+		case LITENN_F32: return convert_from<float>(src, dst_dtype, dst, n, s);
+		case LITENN_F64: return convert_from<double>(src, dst_dtype, dst, n, s);
+		case LITENN_I32: return convert_from<int32_t>(src, dst_dtype, dst, n, s);
+		case LITENN_I64: return convert_from<int64_t>(src, dst_dtype, dst, n, s);
+		case LITENN_BOOL: return convert_from<bool>(src, dst_dtype, dst, n, s);
+		case LITENN_F16: return convert_from<F16>(src, dst_dtype, dst, n, s);
+		case LITENN_BF16: return convert_from<BF16>(src, dst_dtype, dst, n, s);
+		case LITENN_I8: return convert_from<int8_t>(src, dst_dtype, dst, n, s);
+		case LITENN_U8: return convert_from<uint8_t>(src, dst_dtype, dst, n, s);
+		default: return false;
+		}
+	}
+} // namespace litenn_hip
+
+using namespace litenn_hip;
+
+#define GUARD(action, dev)                                                                                             \
+	DeviceGuard guard_(dev);                                                                                           \
+	if (!guard_.ok())                                                                                                  \
+	{                                                                                                                  \
+		return fail_hip(action, guard_.error());                                                                       \
+	}
+
+extern "C" const char* litenn_hip_last_error(void)
+{
+	return g_error.c_str();
+}
+
+extern "C" int litenn_hip_device_count(void)
+{
+	int count = 0;
+	if (hipGetDeviceCount(&count) != hipSuccess)
+	{
+		(void)hipGetLastError();
+		return 0;
+	}
+	return count;
+}
+
+extern "C" int litenn_hip_device_info(int dev, char* buf, size_t buf_len)
+{
+	GUARD("HIP device query", dev);
+	hipDeviceProp_t prop;
+	LITENN_HIP_TRY("HIP device query", hipGetDeviceProperties(&prop, dev));
+	if (buf && buf_len)
+	{
+		snprintf(buf, buf_len, "HIP device %d: %s (%s, %d CUs, %.1f GiB)", dev, prop.name, prop.gcnArchName,
+		         prop.multiProcessorCount, static_cast<double>(prop.totalGlobalMem) / (1024.0 * 1024.0 * 1024.0));
+	}
+	return 0;
+}
+
+extern "C" int litenn_hip_alloc(int dev, int dtype, size_t n, void** out)
+{
+	const size_t es = dtype_size(dtype);
+	if (!out || es == 0)
+	{
+		return fail("HIP allocate", "bad dtype or null output pointer");
+	}
+	GUARD("HIP allocate", dev);
+	*out = nullptr;
+	// zero-element tensors still get a distinct, freeable pointer
+	LITENN_HIP_TRY("HIP allocate", hipMalloc(out, n * es ? n * es : 1));
+	return 0;
+}
+
+extern "C" int litenn_hip_free(int dev, void* ptr, int dtype, size_t n)
+{
+	(void)dtype;
+	(void)n;
+	if (!ptr)
+	{
+		return 0;
+	}
+	GUARD("HIP deallocate", dev);
+	LITENN_HIP_TRY("HIP deallocate", hipFree(ptr));
+	return 0;
+}
+
+extern "C" int litenn_hip_zero(int dev, void* ptr, int dtype, size_t n)
+{
+	const size_t es = dtype_size(dtype);
+	if (es == 0)
+	{
+		return fail("HIP zero fill", "bad dtype");
+	}
+	if (n == 0)
+	{
+		return 0;
+	}
+	GUARD("HIP zero fill", dev);
+	LITENN_HIP_TRY("HIP zero fill", hipMemset(ptr, 0, n * es));
+	return 0;
+}
+
+extern "C" int litenn_hip_convert(int dev, int src_dtype, const void* src, size_t n, int dst_dtype, void* dst,
+                                  const litenn_hip_exec* opts)
+{
+	if (dtype_size(src_dtype) == 0 || dtype_size(dst_dtype) == 0)
+	{
+		return fail("HIP convert", "bad dtype");
+	}
+	GUARD("HIP convert", dev);
+	if (src_dtype == dst_dtype)
+	{
+		if (n)
+		{
+			LITENN_HIP_TRY("HIP convert", hipMemcpyAsync(dst, src, n * dtype_size(src_dtype), hipMemcpyDeviceToDevice,
+			                                             stream_of(opts)));
+		}
+	}
+	else if (!launch_convert(src_dtype, src, n, dst_dtype, dst, stream_of(opts)))
+	{
+		return fail("HIP convert", "dtype pair is not supported on the device");
+	}
+	return finish("HIP convert", opts);
+}
+
+extern "C" int litenn_hip_copy_to_host(int dev, int src_dtype, const void* src, size_t n, int dst_dtype, void* dst,
+                                       const litenn_hip_exec* opts)
+{
+	if (dtype_size(src_dtype) == 0 || dtype_size(dst_dtype) == 0)
+	{
+		return fail("HIP copy to host", "bad dtype");
+	}
+	if (n == 0)
+	{
+		return 0;
+	}
+	GUARD("HIP copy to host", dev);
+	hipStream_t s = stream_of(opts);
+	if (src_dtype == dst_dtype)
+	{
+		LITENN_HIP_TRY("HIP copy to host", hipMemcpyAsync(dst, src, n * dtype_size(src_dtype), hipMemcpyDeviceToHost, s));
+		return finish("HIP copy to host", opts);
+	}
+	// convert on the device, then one copy; the staging buffer forces a synchronous finish
+	void* tmp = nullptr;
+	LITENN_HIP_TRY("HIP copy to host", hipMalloc(&tmp, n * dtype_size(dst_dtype)));
+	int rc = 0;
+	if (!launch_convert(src_dtype, src, n, dst_dtype, tmp, s))
+	{
+		rc = fail("HIP copy to host", "dtype pair is not supported on the device");
+	}
+	else
+	{
+		const hipError_t e = hipMemcpyAsync(dst, tmp, n * dtype_size(dst_dtype), hipMemcpyDeviceToHost, s);
+		const hipError_t e2 = hipStreamSynchronize(s);
+		if (e != hipSuccess || e2 != hipSuccess)
+		{
+			rc = fail_hip("HIP copy to host", e != hipSuccess ? e : e2);
+		}
+	}
+	(void)hipFree(tmp);
+	return rc;
+}
+
+extern "C" int litenn_hip_copy_from_host(int dev, int dst_dtype, void* dst, int src_dtype, const void* src, size_t n,
+                                         const litenn_hip_exec* opts)
+{
+	if (dtype_size(src_dtype) == 0 || dtype_size(dst_dtype) == 0)
+	{
+		return fail("HIP copy from host", "bad dtype");
+	}
+	if (n == 0)
+	{
+		return 0;
+	}
+	GUARD("HIP copy from host", dev);
+	hipStream_t s = stream_of(opts);
+	if (src_dtype == dst_dtype)
+	{
+		LITENN_HIP_TRY("HIP copy from host",
+		               hipMemcpyAsync(dst, src, n * dtype_size(src_dtype), hipMemcpyHostToDevice, s));
+		return finish("HIP copy from host", opts);
+	}
+	void* tmp = nullptr;
+	LITENN_HIP_TRY("HIP copy from host", hipMalloc(&tmp, n * dtype_size(src_dtype)));
+	int rc = 0;
+	const hipError_t e = hipMemcpyAsync(tmp, src, n * dtype_size(src_dtype), hipMemcpyHostToDevice, s);
+	if (e != hipSuccess)
+	{
+		rc = fail_hip("HIP copy from host", e);
+	}
+	else if (!launch_convert(src_dtype, tmp, n, dst_dtype, dst, s))
+	{
+		rc = fail("HIP copy from host", "dtype pair is not supported on the device");
+	}
+	const hipError_t e2 = hipStreamSynchronize(s);
+	if (rc == 0 && e2 != hipSuccess)
+	{
+		rc = fail_hip("HIP copy from host", e2);
+	}
+	(void)hipFree(tmp);
+	return rc;
+}
+
+// ---- group 2: quantised extensions ------------------------------------------------------------
+
+static bool is_weight_format(int fmt)
+{
+	return block_elements(fmt) != 0;
+}
+
+extern "C" int litenn_hip_mul_mat_q(int dev, int fmt, const void* wq, size_t n, size_t k, const void* x, int x_dtype,
+                                    size_t m, void* y, const void* residual, unsigned flags,
+                                    const litenn_hip_exec* opts)
+{
+	const char* action = "HIP quantized matmul";
+	if (!is_weight_format(fmt))
+	{
+		return fail(action, "unsupported block format");
+	}
+	if (x_dtype != LITENN_F32)
+	{
+		return fail(action, "activations must be Float32");
+	}
+	if (row_bytes(fmt, k) == 0)
+	{
+		return fail(action, "row width is incompatible with the block size of the format");
+	}
+	if (n > 0x7fffffffu || k > 0x7fffffffu || m > 0x7fffffffu)
+	{
+		return fail(action, "dimension exceeds 2^31-1");
+	}
+	if (n == 0 || m == 0)
+	{
+		return 0;
+	}
+	if (k == 0)
+	{
+		return fail(action, "inner dimension must be positive");
+	}
+	if (!wq || !x || !y)
+	{
+		return fail(action, "null operand");
+	}
+	GUARD(action, dev);
+	hipStream_t s = stream_of(opts);
+	const float* xf = static_cast<const float*>(x);
+	float* yf = static_cast<float*>(y);
+	const float* rf = static_cast<const float*>(residual);
+	const bool quant = fmt != LITENN_FMT_F16 && fmt != LITENN_FMT_F32;
+	if (m >= 16 && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && k % 256 == 0)
+	{
+		if (launch_gemm(fmt, wq, n, k, xf, m, yf, rf, s) != 0)
+		{
+			return 1;
+		}
+	}
+	else
+	{
+		launch_gemv(fmt, wq, n, k, xf, m, yf, rf, s);
+	}
+	return finish(action, opts);
+}
+
+extern "C" int litenn_hip_dequantize(int dev, int fmt, const void* wq, size_t rows, size_t k, void* dst,
+                                     const litenn_hip_exec* opts)
+{
+	const char* action = "HIP dequantize";
+	if (!is_weight_format(fmt) || row_bytes(fmt, k) == 0)
+	{
+		return fail(action, "unsupported block format or row width");
+	}
+	if (rows == 0 || k == 0)
+	{
+		return 0;
+	}
+	if (k > 0x7fffffffu || rows > 0x7fffffffu)
+	{
+		return fail(action, "dimension exceeds 2^31-1");
+	}
+	GUARD(action, dev);
+	launch_dequantize(fmt, wq, rows, k, static_cast<float*>(dst), stream_of(opts));
+	return finish(action, opts);
+}
+
+extern "C" int litenn_hip_get_rows_q(int dev, int fmt, const void* table, size_t rows, size_t k, const void* ids,
+                                     size_t n_ids, void* out, const litenn_hip_exec* opts)
+{
+	const char* action = "HIP GetRows";
+	if (!is_weight_format(fmt) || row_bytes(fmt, k) == 0)
+	{
+		return fail(action, "unsupported block format or row width");
+	}
+	if (n_ids == 0)
+	{
+		return 0;
+	}
+	if (k > 0x7fffffffu || rows > 0x7fffffffu || n_ids > 0x7fffffffu)
+	{
+		return fail(action, "dimension exceeds 2^31-1");
+	}
+	GUARD(action, dev);
+	hipStream_t s = stream_of(opts);
+	// the range check runs on the device; its flag is read back, which makes this call blocking
+	int* flag = nullptr;
+	LITENN_HIP_TRY(action, hipMalloc(reinterpret_cast<void**>(&flag), sizeof(int)));
+	int host_flag = 0;
+	hipError_t e = hipMemcpyAsync(flag, &host_flag, sizeof(int), hipMemcpyHostToDevice, s);
+	if (e == hipSuccess)
+	{
+		launch_get_rows_q(fmt, table, rows, k, static_cast<const int32_t*>(ids), n_ids, static_cast<float*>(out), flag,
+		                  s);
+		e = hipGetLastError();
+	}
+	if (e == hipSuccess)
+	{
+		e = hipMemcpyAsync(&host_flag, flag, sizeof(int), hipMemcpyDeviceToHost, s);
+	}
+	if (e == hipSuccess)
+	{
+		e = hipStreamSynchronize(s);
+	}
+	(void)hipFree(flag);
+	if (e != hipSuccess)
+	{
+		return fail_hip(action, e);
+	}
+	if (host_flag)
+	{
+		return fail(action, "GetRows index out of range");
+	}
+	return 0;
+}
+
+extern "C" int litenn_hip_rmsnorm(int dev, const void* x, const void* w, double eps, size_t m, size_t d, void* y,
+                                  const litenn_hip_exec* opts)
+{
+	const char* action = "HIP RMSNorm";
+	if (m == 0 || d == 0)
+	{
+		return 0;
+	}
+	if (d > 0x7fffffffu || m > 0x7fffffffu)
+	{
+		return fail(action, "dimension exceeds 2^31-1");
+	}
+	GUARD(action, dev);
+	launch_rmsnorm(static_cast<const float*>(x), static_cast<const float*>(w), eps, m, d, static_cast<float*>(y),
+	               stream_of(opts));
+	return finish(action, opts);
+}
+
+extern "C" int litenn_hip_rope_interleaved(int dev, const void* x, void* y, size_t m, size_t n_heads, size_t head_dim,
+                                           size_t rope_dims, double base, double freq_scale, size_t pos_offset,
+                                           const litenn_hip_exec* opts)
+{
+	const char* action = "HIP RoPE";
+	if (head_dim % 2 != 0)
+	{
+		return fail(action, "RoPE featureSize must be even");
+	}
+	if (rope_dims > head_dim || rope_dims % 2 != 0)
+	{
+		return fail(action, "rope dimension count must be even and no larger than headDim");
+	}
+	if (!(base > 0.0) || !(freq_scale > 0.0))
+	{
+		return fail(action, "RoPE base and frequencyScale must be finite and greater than zero");
+	}
+	if (m == 0 || n_heads == 0 || head_dim == 0)
+	{
+		return 0;
+	}
+	if (m * n_heads * head_dim > 0x7fffffffu)
+	{
+		return fail(action, "tensor too large");
+	}
+	GUARD(action, dev);
+	hipStream_t s = stream_of(opts);
+	const size_t half = rope_dims / 2;
+	float* tables = nullptr;
+	if (half)
+	{
+		LITENN_HIP_TRY(action, hipMalloc(reinterpret_cast<void**>(&tables), sizeof(float) * 2 * m * half));
+		launch_rope_table(tables, tables + m * half, m, half, base, freq_scale, pos_offset, s);
+	}
+	launch_rope(static_cast<const float*>(x), static_cast<float*>(y), m, n_heads, head_dim, rope_dims, tables,
+	            tables ? tables + m * half : nullptr, s);
+	// the angle tables are private to this call, so it always completes before returning
+	hipError_t e = hipGetLastError();
+	if (e == hipSuccess)
+	{
+		e = hipStreamSynchronize(s);
+	}
+	if (tables)
+	{
+		(void)hipFree(tables);
+	}
+	if (e != hipSuccess)
+	{
+		return fail_hip(action, e);
+	}
+	return 0;
+}
+
+extern "C" int litenn_hip_kv_append(int dev, void* cache, int cache_dtype, size_t past, const void* cur, size_t m,
+                                    size_t width, const litenn_hip_exec* opts)
+{
+	const char* action = "HIP KV append";
+	if (cache_dtype != LITENN_F16 && cache_dtype != LITENN_F32)
+	{
+		return fail(action, "cache dtype must be Float16 or Float32");
+	}
+	if (m == 0 || width == 0)
+	{
+		return 0;
+	}
+	GUARD(action, dev);
+	launch_kv_append(cache, cache_dtype, past * width, static_cast<const float*>(cur), m * width, stream_of(opts));
+	return finish(action, opts);
+}
+
+extern "C" int litenn_hip_attn_decode(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype,
+                                      size_t m, size_t past, size_t n_head, size_t n_kv_head, size_t head_dim,
+                                      void* out, const litenn_hip_exec* opts)
+{
+	const char* action = "HIP attention";
+	if (cache_dtype != LITENN_F16 && cache_dtype != LITENN_F32)
+	{
+		return fail(action, "cache dtype must be Float16 or Float32");
+	}
+	if (n_head == 0 || n_kv_head == 0 || n_head % n_kv_head != 0)
+	{
+		return fail(action, "head count must be a positive multiple of the KV head count");
+	}
+	if (head_dim == 0 || head_dim > 256)
+	{
+		return fail(action, "head dimension must be in [1, 256]");
+	}
+	if (m == 0)
+	{
+		return 0;
+	}
+	if (past + m > 15360)
+	{
+		return fail(action, "key length exceeds the 15360 positions the score buffer holds");
+	}
+	if (m > 65535)
+	{
+		return fail(action, "too many query rows");
+	}
+	GUARD(action, dev);
+	launch_attn_decode(static_cast<const float*>(q), kcache, vcache, cache_dtype, m, nullptr, past, past + m, n_head,
+	                   n_kv_head, head_dim, static_cast<float*>(out), stream_of(opts));
+	return finish(action, opts);
+}
+
+extern "C" int litenn_hip_silu_mul(int dev, const void* gate, const void* up, void* y, size_t n,
+                                   const litenn_hip_exec* opts)
+{
+	const char* action = "HIP SiLU";
+	if (n == 0)
+	{
+		return 0;
+	}
+	GUARD(action, dev);
+	launch_silu_mul(static_cast<const float*>(gate), static_cast<const float*>(up), static_cast<float*>(y), n,
+	                stream_of(opts));
+	return finish(action, opts);
+}
+
+extern "C" int litenn_hip_argmax(int dev, const void* x, size_t rows, size_t n, void* out_index,
+                                 const litenn_hip_exec* opts)
+{
+	const char* action = "HIP argmax";
+	if (rows == 0)
+	{
+		return 0;
+	}
+	if (n == 0 || n > 0x7fffffffu)
+	{
+		return fail(action, "row length must be in [1, 2^31-1]");
+	}
+	GUARD(action, dev);
+	launch_argmax(static_cast<const float*>(x), rows, n, static_cast<int32_t*>(out_index), stream_of(opts));
+	return finish(action, opts);
+}

@@ -1,0 +1,151 @@
+// Shared host/device helpers of the gfx950 backend.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "../../include/litenn_hip.h"
+
+namespace litenn_hip
+{
+	// ---- error reporting: status code + thread-local message ---------------
+	void set_error(const std::string& message);
+	int fail(const char* action, const std::string& message);
+	int fail_hip(const char* action, hipError_t err);
+
+#define LITENN_HIP_TRY(action, expr)                                                                                   \
+	do                                                                                                                 \
+	{                                                                                                                  \
+		const hipError_t litenn_err_ = (expr);                                                                         \
+		if (litenn_err_ != hipSuccess)                                                                                 \
+		{                                                                                                              \
+			return ::litenn_hip::fail_hip(action, litenn_err_);                                                        \
+		}                                                                                                              \
+	} while (0)
+
+	// Selects `dev` for the lifetime of the guard and restores the caller's device.
+	class DeviceGuard
+	{
+	public:
+		explicit DeviceGuard(int dev);
+		~DeviceGuard();
+		bool ok() const { return ok_; }
+		hipError_t error() const { return err_; }
+
+	private:
+		int previous_ = -1;
+		bool ok_ = false;
+		hipError_t err_ = hipSuccess;
+	};
+
+	inline hipStream_t stream_of(const litenn_hip_exec* opts)
+	{
+		return opts ? static_cast<hipStream_t>(opts->stream) : nullptr;
+	}
+
+	// Applies the synchronize flag of the execution options and reports launch errors.
+	int finish(const char* action, const litenn_hip_exec* opts);
+
+	size_t dtype_size(int dtype);
+	int block_elements(int fmt);
+	int block_bytes(int fmt);
+	// bytes of one row of k elements, 0 when k is not a whole number of blocks
+	size_t row_bytes(int fmt, size_t k);
+
+	constexpr int kWave = 64;
+} // namespace litenn_hip
+
+// ---- device-side helpers ---------------------------------------------------
+#if defined(__HIPCC__)
+namespace litenn_hip
+{
+	__device__ __forceinline__ float f16_bits_to_f32(uint32_t bits)
+	{
+		return __half2float(__ushort_as_half(static_cast<unsigned short>(bits & 0xffffu)));
+	}
+
+	// LiteNN's Float32 -> Float16 conversion (src/LiteNN/DType.h:63-110): nearest, ties UP in
+	// magnitude (only the first dropped bit is examined), subnormals and overflow handled the
+	// same way.  Not IEEE round-to-nearest-even, so the hardware converter is not used.
+	__device__ __forceinline__ uint16_t f32_to_f16_bits_litenn(float value)
+	{
+		const uint32_t bits = __float_as_uint(value);
+		const uint32_t sign = (bits >> 16) & 0x8000u;
+		const int exponent = static_cast<int>((bits >> 23) & 0xffu) - 127;
+		uint32_t mantissa = bits & 0x7fffffu;
+		if ((bits & 0x7fffffffu) == 0)
+		{
+			return static_cast<uint16_t>(sign);
+		}
+		if (((bits >> 23) & 0xffu) == 0xffu)
+		{
+			return static_cast<uint16_t>(sign | 0x7c00u | (mantissa ? 0x0200u : 0u));
+		}
+		if (exponent > 15)
+		{
+			return static_cast<uint16_t>(sign | 0x7c00u);
+		}
+		if (exponent < -14)
+		{
+			if (exponent < -24)
+			{
+				return static_cast<uint16_t>(sign);
+			}
+			mantissa |= 0x800000u;
+			const uint32_t shift = static_cast<uint32_t>(-exponent - 1);
+			uint32_t half_mantissa = mantissa >> shift;
+			half_mantissa += (mantissa >> (shift - 1)) & 1u;
+			return static_cast<uint16_t>(sign | half_mantissa);
+		}
+		// adding the rounding bit carries into the exponent exactly as the reference's
+		// explicit mantissa-overflow branch does, and saturates at infinity (0x7c00)
+		uint32_t half = (static_cast<uint32_t>(exponent + 15) << 10) | (mantissa >> 13);
+		half += (mantissa >> 12) & 1u;
+		return static_cast<uint16_t>(sign | half);
+	}
+
+	template <int Ctrl, int RowMask = 0xF, int BankMask = 0xF>
+	__device__ __forceinline__ float dpp_f32(float v)
+	{
+		return __int_as_float(
+		    __builtin_amdgcn_update_dpp(0, __float_as_int(v), Ctrl, RowMask, BankMask, false));
+	}
+
+	// Sum over the 64 lanes of a wavefront with DPP only (no LDS traffic); the total is
+	// returned in every lane.
+	__device__ __forceinline__ float wave_sum(float v)
+	{
+		v += dpp_f32<0xB1>(v);  // quad_perm [1,0,3,2]
+		v += dpp_f32<0x4E>(v);  // quad_perm [2,3,0,1]
+		v += dpp_f32<0x141>(v); // row_half_mirror
+		v += dpp_f32<0x140>(v); // row_mirror: every lane holds its 16-lane row total
+		v += dpp_f32<0x142, 0xA>(v); // row_bcast15 into rows 1 and 3
+		v += dpp_f32<0x143, 0xC>(v); // row_bcast31 into rows 2 and 3: lane 63 holds the total
+		return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+	}
+
+	// Sum within aligned groups of 16 lanes; every lane of the group holds the result.
+	__device__ __forceinline__ float row16_sum(float v)
+	{
+		v += dpp_f32<0xB1>(v);
+		v += dpp_f32<0x4E>(v);
+		v += dpp_f32<0x141>(v);
+		v += dpp_f32<0x140>(v);
+		return v;
+	}
+
+	__device__ __forceinline__ float wave_max(float v)
+	{
+		for (int off = 32; off > 0; off >>= 1)
+		{
+			v = fmaxf(v, __shfl_xor(v, off, 64));
+		}
+		return v;
+	}
+} // namespace litenn_hip
+#endif

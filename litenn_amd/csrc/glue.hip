@@ -1,0 +1,470 @@
+// The small kernels that surround the quantised matmuls in the LLaMA decoder:
+// RMSNorm, interleaved RoPE, KV-cache append, causal single-row attention over an
+// fp16/f32 cache, SiLU*up, arg-max.  All of them are bandwidth-trivial next to the
+// weight stream; they are written to keep f32 (f64 for the norm) semantics of the
+// reference chains and to read every operand once.
+#include "common.hpp"
+
+namespace litenn_hip
+{
+	namespace
+	{
+		// ---------------- RMSNorm (f64 accumulate, ComputePrimitives.h:792-817) -------------
+		__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x,
+		                                                       const float* __restrict__ w, double eps, int d,
+		                                                       float* __restrict__ y)
+		{
+			__shared__ double red[4];
+			const float* xr = x + static_cast<size_t>(blockIdx.x) * d;
+			float* yr = y + static_cast<size_t>(blockIdx.x) * d;
+			double acc = 0.0;
+			for (int i = threadIdx.x; i < d; i += blockDim.x)
+			{
+				const double v = static_cast<double>(xr[i]);
+				acc += v * v;
+			}
+			for (int off = 32; off > 0; off >>= 1)
+			{
+				acc += __shfl_xor(acc, off, 64);
+			}
+			if ((threadIdx.x & 63) == 0)
+			{
+				red[threadIdx.x >> 6] = acc;
+			}
+			__syncthreads();
+			double total = 0.0;
+			for (int i = 0; i < static_cast<int>(blockDim.x >> 6); ++i)
+			{
+				total += red[i];
+			}
+			const double denom = sqrt(total / static_cast<double>(d) + eps);
+			for (int i = threadIdx.x; i < d; i += blockDim.x)
+			{
+				double v = static_cast<double>(xr[i]) / denom;
+				if (w)
+				{
+					v *= static_cast<double>(w[i]);
+				}
+				yr[i] = static_cast<float>(v);
+			}
+		}
+
+		// ---------------- RoPE -------------------------------------------------------------
+		// Angle tables exactly as MakeRoPEAngleTable builds them (RoPE.h:24-41): f64 maths,
+		// stored as f32.  table[pos * half + dim] for pos in [0, positions).
+		__global__ void rope_table_kernel(float* __restrict__ cos_t, float* __restrict__ sin_t, int positions, int half,
+		                                  double base, double freq_scale, int pos_offset)
+		{
+			const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+			if (idx >= positions * half)
+			{
+				return;
+			}
+			const int pos = idx / half, dim = idx % half;
+			const double exponent = -2.0 * static_cast<double>(dim) / static_cast<double>(half * 2);
+			const double inv_freq = pow(base, exponent);
+			const double angle = static_cast<double>(pos_offset + pos) * inv_freq * freq_scale;
+			cos_t[idx] = static_cast<float>(cos(angle));
+			sin_t[idx] = static_cast<float>(sin(angle));
+		}
+
+		// f32 rotation with separately rounded products (RoPE.h:93-111): the fused forms are
+		// avoided on purpose so the four multiplies round like the reference's Multiply nodes.
+		__device__ __forceinline__ void rotate(float a, float b, float c, float s, float& o0, float& o1)
+		{
+			o0 = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, s));
+			o1 = __fadd_rn(__fmul_rn(a, s), __fmul_rn(b, c));
+		}
+
+		// x,y [m, n_heads, head_dim]; tables indexed by row (positions start at the table's origin)
+		__global__ void rope_kernel(const float* __restrict__ x, float* __restrict__ y, int m, int n_heads, int head_dim,
+		                            int rope_dims, const float* __restrict__ cos_t, const float* __restrict__ sin_t)
+		{
+			const int half_all = head_dim / 2;
+			const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+			const size_t total = static_cast<size_t>(m) * n_heads * half_all;
+			if (idx >= total)
+			{
+				return;
+			}
+			const int p = idx % half_all;
+			const size_t rh = idx / half_all; // row * n_heads + head
+			const int row = rh / n_heads;
+			const size_t base = rh * head_dim + 2 * p;
+			const float a = x[base], b = x[base + 1];
+			if (2 * p < rope_dims)
+			{
+				const int half = rope_dims / 2;
+				float o0, o1;
+				rotate(a, b, cos_t[row * half + p], sin_t[row * half + p], o0, o1);
+				y[base] = o0;
+				y[base + 1] = o1;
+			}
+			else
+			{
+				y[base] = a;
+				y[base + 1] = b;
+			}
+		}
+
+		template <typename KV>
+		__device__ __forceinline__ void store_kv(KV* dst, float v);
+		template <>
+		__device__ __forceinline__ void store_kv<float>(float* dst, float v) { *dst = v; }
+		template <>
+		__device__ __forceinline__ void store_kv<uint16_t>(uint16_t* dst, float v) { *dst = f32_to_f16_bits_litenn(v); }
+
+		template <typename KV>
+		__device__ __forceinline__ float load_kv(const KV* src);
+		template <>
+		__device__ __forceinline__ float load_kv<float>(const float* src) { return *src; }
+		template <>
+		__device__ __forceinline__ float load_kv<uint16_t>(const uint16_t* src) { return f16_bits_to_f32(*src); }
+
+		template <typename KV>
+		__global__ void kv_append_kernel(KV* __restrict__ cache, size_t past, const float* __restrict__ cur, size_t count)
+		{
+			const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+			if (idx < count)
+			{
+				store_kv<KV>(cache + past + idx, cur[idx]);
+			}
+		}
+
+		// Decoder step glue: rotate q in place, rotate k and append it and v to the caches
+		// (tools/gguf/LLaMABuilder.cpp:596-622,640-645).  Position of row i is *past + i.
+		// tables are [ctx, rope_dims/2].
+		template <typename KV>
+		__global__ void rope_qkv_append_kernel(float* __restrict__ q, const float* __restrict__ k,
+		                                       const float* __restrict__ v, KV* __restrict__ kcache,
+		                                       KV* __restrict__ vcache, const int* __restrict__ past_dev, int m,
+		                                       int n_head, int n_kv_head, int head_dim, int rope_dims,
+		                                       const float* __restrict__ cos_t, const float* __restrict__ sin_t)
+		{
+			const int half_all = head_dim / 2;
+			const int half = rope_dims / 2;
+			const int past = *past_dev;
+			const int heads = n_head + 2 * n_kv_head; // q heads, k heads, v heads
+			const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+			const size_t total = static_cast<size_t>(m) * heads * half_all;
+			if (idx >= total)
+			{
+				return;
+			}
+			const int p = idx % half_all;
+			const size_t rh = idx / half_all;
+			const int row = rh / heads;
+			const int h = rh % heads;
+			const int pos = past + row;
+			const size_t kvw = static_cast<size_t>(n_kv_head) * head_dim;
+			if (h < n_head)
+			{
+				float* base = q + (static_cast<size_t>(row) * n_head + h) * head_dim + 2 * p;
+				if (2 * p < rope_dims)
+				{
+					float o0, o1;
+					rotate(base[0], base[1], cos_t[static_cast<size_t>(pos) * half + p],
+					       sin_t[static_cast<size_t>(pos) * half + p], o0, o1);
+					base[0] = o0;
+					base[1] = o1;
+				}
+			}
+			else if (h < n_head + n_kv_head)
+			{
+				const int kh = h - n_head;
+				const float* src = k + static_cast<size_t>(row) * kvw + kh * head_dim + 2 * p;
+				KV* dst = kcache + static_cast<size_t>(pos) * kvw + kh * head_dim + 2 * p;
+				float o0 = src[0], o1 = src[1];
+				if (2 * p < rope_dims)
+				{
+					rotate(src[0], src[1], cos_t[static_cast<size_t>(pos) * half + p],
+					       sin_t[static_cast<size_t>(pos) * half + p], o0, o1);
+				}
+				store_kv<KV>(dst, o0);
+				store_kv<KV>(dst + 1, o1);
+			}
+			else
+			{
+				const int vh = h - n_head - n_kv_head;
+				const float* src = v + static_cast<size_t>(row) * kvw + vh * head_dim + 2 * p;
+				KV* dst = vcache + static_cast<size_t>(pos) * kvw + vh * head_dim + 2 * p;
+				store_kv<KV>(dst, src[0]);
+				store_kv<KV>(dst + 1, src[1]);
+			}
+		}
+
+		// ---------------- attention of one query row against the cache -----------------------
+		// grid (n_head, m); block 256.  Query row i sits at position past + i and sees keys
+		// 0 .. past + i (the additive -1e9 causal constant of CausalMask.h:16-34 turns every later
+		// key into an exact zero after exp in f32, so those keys are simply not visited).
+		// Scores live in LDS (max_len floats).  head_dim <= 256.
+		template <typename KV>
+		__global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q,
+		                                                           const KV* __restrict__ kcache,
+		                                                           const KV* __restrict__ vcache,
+		                                                           float* __restrict__ out,
+		                                                           const int* __restrict__ past_dev, int past_host,
+		                                                           int n_head, int n_kv_head, int head_dim,
+		                                                           float scale)
+		{
+			extern __shared__ float smem[];
+			__shared__ float red[8];
+			__shared__ float part_o[256];
+			const int h = blockIdx.x;
+			const int row = blockIdx.y;
+			const int past = past_dev ? *past_dev : past_host;
+			const int len = past + row + 1;
+			const int kvh = h / (n_head / n_kv_head);
+			const size_t kvw = static_cast<size_t>(n_kv_head) * head_dim;
+			const float* qr = q + (static_cast<size_t>(row) * n_head + h) * head_dim;
+			const KV* kbase = kcache + static_cast<size_t>(kvh) * head_dim;
+			const KV* vbase = vcache + static_cast<size_t>(kvh) * head_dim;
+			float* scores = smem;
+
+			// scores: 16 lanes per key, head_dim/16 elements per lane
+			const int sub = threadIdx.x & 15;
+			const int grp = threadIdx.x >> 4; // 16 key groups per block
+			const int per = (head_dim + 15) >> 4;
+			float qv[16];
+#pragma unroll
+			for (int e = 0; e < 16; ++e)
+			{
+				qv[e] = (e < per && sub * per + e < head_dim) ? qr[sub * per + e] : 0.0f;
+			}
+			for (int t0 = 0; t0 < len; t0 += 16)
+			{
+				const int t = t0 + grp;
+				float acc = 0.0f;
+				if (t < len)
+				{
+					const KV* kr = kbase + static_cast<size_t>(t) * kvw + sub * per;
+#pragma unroll
+					for (int e = 0; e < 16; ++e)
+					{
+						if (e < per && sub * per + e < head_dim)
+						{
+							acc = fmaf(qv[e], load_kv<KV>(kr + e), acc);
+						}
+					}
+				}
+				acc = row16_sum(acc);
+				if (t < len && sub == 0)
+				{
+					scores[t] = acc * scale;
+				}
+			}
+			__syncthreads();
+			float mx = -INFINITY;
+			for (int t = threadIdx.x; t < len; t += blockDim.x)
+			{
+				mx = fmaxf(mx, scores[t]);
+			}
+			mx = wave_max(mx);
+			if ((threadIdx.x & 63) == 0)
+			{
+				red[threadIdx.x >> 6] = mx;
+			}
+			__syncthreads();
+			mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+			float sum = 0.0f;
+			for (int t = threadIdx.x; t < len; t += blockDim.x)
+			{
+				const float e = expf(scores[t] - mx);
+				scores[t] = e;
+				sum += e;
+			}
+			sum = wave_sum(sum);
+			if ((threadIdx.x & 63) == 0)
+			{
+				red[4 + (threadIdx.x >> 6)] = sum;
+			}
+			__syncthreads();
+			const float denom = (red[4] + red[5]) + (red[6] + red[7]);
+
+			// output: thread (part, c) accumulates keys t = part, part + parts, ...
+			const int parts = 256 / head_dim > 0 ? 256 / head_dim : 1;
+			const int c = threadIdx.x % head_dim;
+			const int part = threadIdx.x / head_dim;
+			float o = 0.0f;
+			if (part < parts)
+			{
+				for (int t = part; t < len; t += parts)
+				{
+					o = fmaf(scores[t], load_kv<KV>(vbase + static_cast<size_t>(t) * kvw + c), o);
+				}
+			}
+			part_o[threadIdx.x] = o;
+			__syncthreads();
+			if (threadIdx.x < head_dim)
+			{
+				float total = 0.0f;
+				for (int pp = 0; pp < parts; ++pp)
+				{
+					total += part_o[pp * head_dim + threadIdx.x];
+				}
+				out[(static_cast<size_t>(row) * n_head + h) * head_dim + threadIdx.x] = total / denom;
+			}
+		}
+
+		// ---------------- SiLU(gate) * up (Activation.h:22-35,56-63; SwiGLU.h:63-66) ---------
+		__global__ void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+		                                float* __restrict__ y, size_t n)
+		{
+			const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+			if (i < n)
+			{
+				const float g = gate[i];
+				const float sig = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf(-g)));
+				y[i] = __fmul_rn(__fmul_rn(g, sig), up[i]);
+			}
+		}
+
+		// ---------------- arg-max: first maximal index ---------------------------------------
+		__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ x, int n,
+		                                                       int32_t* __restrict__ out)
+		{
+			__shared__ float bv[16];
+			__shared__ int bi[16];
+			const float* xr = x + static_cast<size_t>(blockIdx.x) * n;
+			float best = -INFINITY;
+			int best_i = 0x7fffffff;
+			for (int i = threadIdx.x; i < n; i += blockDim.x)
+			{
+				const float v = xr[i];
+				if (v > best || best_i == 0x7fffffff)
+				{
+					best = v;
+					best_i = i;
+				}
+			}
+			for (int off = 32; off > 0; off >>= 1)
+			{
+				const float ov = __shfl_xor(best, off, 64);
+				const int oi = __shfl_xor(best_i, off, 64);
+				if (ov > best || (ov == best && oi < best_i))
+				{
+					best = ov;
+					best_i = oi;
+				}
+			}
+			if ((threadIdx.x & 63) == 0)
+			{
+				bv[threadIdx.x >> 6] = best;
+				bi[threadIdx.x >> 6] = best_i;
+			}
+			__syncthreads();
+			if (threadIdx.x == 0)
+			{
+				for (int wv = 1; wv < static_cast<int>(blockDim.x >> 6); ++wv)
+				{
+					if (bv[wv] > best || (bv[wv] == best && bi[wv] < best_i))
+					{
+						best = bv[wv];
+						best_i = bi[wv];
+					}
+				}
+				out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
+			}
+		}
+
+		__global__ void add_int_kernel(int* p, int v) { *p += v; }
+		__global__ void set_int_kernel(int* p, int v) { *p = v; }
+	} // namespace
+
+	// ---- launchers used by the C ABI and by the decoder runtime ---------------------------
+	void launch_rmsnorm(const float* x, const float* w, double eps, size_t m, size_t d, float* y, hipStream_t s)
+	{
+		rmsnorm_kernel<<<dim3(m), dim3(256), 0, s>>>(x, w, eps, static_cast<int>(d), y);
+	}
+
+	void launch_rope_table(float* cos_t, float* sin_t, size_t positions, size_t half, double base, double freq_scale,
+	                       size_t pos_offset, hipStream_t s)
+	{
+		const size_t total = positions * half;
+		rope_table_kernel<<<dim3((total + 255) / 256), dim3(256), 0, s>>>(cos_t, sin_t, static_cast<int>(positions),
+		                                                                   static_cast<int>(half), base, freq_scale,
+		                                                                   static_cast<int>(pos_offset));
+	}
+
+	void launch_rope(const float* x, float* y, size_t m, size_t n_heads, size_t head_dim, size_t rope_dims,
+	                 const float* cos_t, const float* sin_t, hipStream_t s)
+	{
+		const size_t total = m * n_heads * (head_dim / 2);
+		rope_kernel<<<dim3((total + 255) / 256), dim3(256), 0, s>>>(x, y, static_cast<int>(m),
+		                                                             static_cast<int>(n_heads),
+		                                                             static_cast<int>(head_dim),
+		                                                             static_cast<int>(rope_dims), cos_t, sin_t);
+	}
+
+	void launch_kv_append(void* cache, int cache_dtype, size_t past_elems, const float* cur, size_t count, hipStream_t s)
+	{
+		const dim3 grid((count + 255) / 256), block(256);
+		if (cache_dtype == LITENN_F16)
+		{
+			kv_append_kernel<uint16_t><<<grid, block, 0, s>>>(static_cast<uint16_t*>(cache), past_elems, cur, count);
+		}
+		else
+		{
+			kv_append_kernel<float><<<grid, block, 0, s>>>(static_cast<float*>(cache), past_elems, cur, count);
+		}
+	}
+
+	void launch_rope_qkv_append(float* q, const float* k, const float* v, void* kcache, void* vcache, int cache_dtype,
+	                            const int* past_dev, size_t m, size_t n_head, size_t n_kv_head, size_t head_dim,
+	                            size_t rope_dims, const float* cos_t, const float* sin_t, hipStream_t s)
+	{
+		const size_t total = m * (n_head + 2 * n_kv_head) * (head_dim / 2);
+		const dim3 grid((total + 255) / 256), block(256);
+		if (cache_dtype == LITENN_F16)
+		{
+			rope_qkv_append_kernel<uint16_t><<<grid, block, 0, s>>>(
+			    q, k, v, static_cast<uint16_t*>(kcache), static_cast<uint16_t*>(vcache), past_dev, static_cast<int>(m),
+			    static_cast<int>(n_head), static_cast<int>(n_kv_head), static_cast<int>(head_dim),
+			    static_cast<int>(rope_dims), cos_t, sin_t);
+		}
+		else
+		{
+			rope_qkv_append_kernel<float><<<grid, block, 0, s>>>(
+			    q, k, v, static_cast<float*>(kcache), static_cast<float*>(vcache), past_dev, static_cast<int>(m),
+			    static_cast<int>(n_head), static_cast<int>(n_kv_head), static_cast<int>(head_dim),
+			    static_cast<int>(rope_dims), cos_t, sin_t);
+		}
+	}
+
+	// max_len: upper bound of past + m (sizes the LDS score buffer)
+	void launch_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
+	                        const int* past_dev, size_t past_host, size_t max_len, size_t n_head, size_t n_kv_head,
+	                        size_t head_dim, float* out, hipStream_t s)
+	{
+		const dim3 grid(n_head, m), block(256);
+		const size_t lds = sizeof(float) * max_len;
+		const float scale = static_cast<float>(1.0 / sqrt(static_cast<double>(head_dim)));
+		if (cache_dtype == LITENN_F16)
+		{
+			attn_decode_kernel<uint16_t><<<grid, block, lds, s>>>(
+			    q, static_cast<const uint16_t*>(kcache), static_cast<const uint16_t*>(vcache), out, past_dev,
+			    static_cast<int>(past_host), static_cast<int>(n_head), static_cast<int>(n_kv_head),
+			    static_cast<int>(head_dim), scale);
+		}
+		else
+		{
+			attn_decode_kernel<float><<<grid, block, lds, s>>>(
+			    q, static_cast<const float*>(kcache), static_cast<const float*>(vcache), out, past_dev,
+			    static_cast<int>(past_host), static_cast<int>(n_head), static_cast<int>(n_kv_head),
+			    static_cast<int>(head_dim), scale);
+		}
+	}
+
+	void launch_silu_mul(const float* gate, const float* up, float* y, size_t n, hipStream_t s)
+	{
+		silu_mul_kernel<<<dim3((n + 255) / 256), dim3(256), 0, s>>>(gate, up, y, n);
+	}
+
+	void launch_argmax(const float* x, size_t rows, size_t n, int32_t* out, hipStream_t s)
+	{
+		argmax_kernel<<<dim3(rows), dim3(1024), 0, s>>>(x, static_cast<int>(n), out);
+	}
+
+	void launch_add_int(int* p, int v, hipStream_t s) { add_int_kernel<<<1, 1, 0, s>>>(p, v); }
+	void launch_set_int(int* p, int v, hipStream_t s) { set_int_kernel<<<1, 1, 0, s>>>(p, v); }
+} // namespace litenn_hip

@@ -1,0 +1,731 @@
+// LLaMA decoder runtime on one GPU.
+//
+// The reference lowers a new static graph for every (sequenceLength, pastLength) pair and
+// interprets it node by node, re-dequantising every weight to f32 each time
+// (tools/gguf/LLaMABuilder.cpp:826-872, src/LiteNN/Runtime/Interpreter.h:89-104,325-329).
+// Here the same operator sequence (LLaMABuilder.cpp:568-668,774-800) runs as a fixed list of
+// kernel launches over weights that stay in their .gguf block layout in HBM, with a
+// preallocated KV cache, the current length kept in device memory, and the single-token
+// step captured once into a HIP graph so that a greedy loop never returns to the host.
+#include "common.hpp"
+
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+namespace litenn_hip
+{
+	int launch_gemv(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
+	                const float* residual, hipStream_t stream);
+	int launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
+	                const float* residual, hipStream_t stream);
+	void launch_get_rows_q(int fmt, const void* table, size_t rows, size_t k, const int32_t* ids, size_t n_ids,
+	                       float* out, int* err_flag, hipStream_t stream);
+	void launch_rmsnorm(const float* x, const float* w, double eps, size_t m, size_t d, float* y, hipStream_t s);
+	void launch_rope_qkv_append(float* q, const float* k, const float* v, void* kcache, void* vcache, int cache_dtype,
+	                            const int* past_dev, size_t m, size_t n_head, size_t n_kv_head, size_t head_dim,
+	                            size_t rope_dims, const float* cos_t, const float* sin_t, hipStream_t s);
+	void launch_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
+	                        const int* past_dev, size_t past_host, size_t max_len, size_t n_head, size_t n_kv_head,
+	                        size_t head_dim, float* out, hipStream_t s);
+	void launch_silu_mul(const float* gate, const float* up, float* y, size_t n, hipStream_t s);
+	void launch_argmax(const float* x, size_t rows, size_t n, int32_t* out, hipStream_t s);
+	bool launch_convert(int src_dtype, const void* src, size_t n, int dst_dtype, void* dst, hipStream_t s);
+
+	namespace
+	{
+		// counters[0] = past length, counters[1] = tokens emitted so far
+		__global__ void advance_kernel(int* counters, int past_inc, const int32_t* next, int32_t* out)
+		{
+			if (out)
+			{
+				out[counters[1]] = *next;
+				counters[1] += 1;
+			}
+			counters[0] += past_inc;
+		}
+
+		__global__ void set_counters_kernel(int* counters, int past, int emitted)
+		{
+			counters[0] = past;
+			counters[1] = emitted;
+		}
+
+		struct Weight
+		{
+			int fmt = 0;
+			const void* data = nullptr;
+			size_t n = 0, k = 0;
+		};
+
+		struct Layer
+		{
+			Weight wq, wk, wv, wo, gate, up, down;
+			const float* attn_norm = nullptr;
+			const float* ffn_norm = nullptr;
+			void* kcache = nullptr;
+			void* vcache = nullptr;
+		};
+	} // namespace
+} // namespace litenn_hip
+
+using namespace litenn_hip;
+
+struct litenn_hip_llama
+{
+	int dev = 0;
+	litenn_hip_llama_params p{};
+	int head_dim = 0;
+	Weight tok_embd, output;
+	const float* output_norm = nullptr;
+	std::vector<Layer> layers;
+	hipStream_t stream = nullptr;
+	float* cos_t = nullptr; // [context_length, rope_dims/2]
+	float* sin_t = nullptr;
+	// activations for `cap_rows` rows
+	size_t cap_rows = 0, cap_logit_rows = 0;
+	float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *gate = nullptr,
+	      *up = nullptr, *logits = nullptr;
+	int32_t* d_tokens = nullptr;
+	int32_t* d_next = nullptr; // token produced by the last arg-max
+	int32_t* d_out = nullptr;  // generated tokens
+	size_t cap_out = 0;
+	int* d_counters = nullptr; // {past, emitted}
+	int* d_err = nullptr;
+	int past = 0;
+	hipGraphExec_t step_exec = nullptr;
+	hipGraph_t step_graph = nullptr;
+};
+
+namespace
+{
+	const char* kAction = "HIP LLaMA";
+
+	void free_scratch(litenn_hip_llama* m)
+	{
+		float** bufs[] = { &m->x, &m->xn, &m->q, &m->k, &m->v, &m->attn, &m->gate, &m->up };
+		for (float** b : bufs)
+		{
+			if (*b)
+			{
+				(void)hipFree(*b);
+				*b = nullptr;
+			}
+		}
+		if (m->d_tokens)
+		{
+			(void)hipFree(m->d_tokens);
+			m->d_tokens = nullptr;
+		}
+		m->cap_rows = 0;
+	}
+
+	void drop_graph(litenn_hip_llama* m)
+	{
+		if (m->step_exec)
+		{
+			(void)hipGraphExecDestroy(m->step_exec);
+			m->step_exec = nullptr;
+		}
+		if (m->step_graph)
+		{
+			(void)hipGraphDestroy(m->step_graph);
+			m->step_graph = nullptr;
+		}
+	}
+
+	int ensure_rows(litenn_hip_llama* m, size_t rows, size_t logit_rows)
+	{
+		const size_t d = m->p.embedding_length;
+		const size_t qw = static_cast<size_t>(m->p.head_count) * m->head_dim;
+		const size_t kvw = static_cast<size_t>(m->p.head_count_kv) * m->head_dim;
+		const size_t ff = m->p.feed_forward_length;
+		if (rows > m->cap_rows)
+		{
+			drop_graph(m); // the captured step references the old buffers
+			free_scratch(m);
+			struct { float** p; size_t n; } bufs[] = { { &m->x, d }, { &m->xn, d }, { &m->q, qw }, { &m->k, kvw },
+				                                        { &m->v, kvw }, { &m->attn, qw }, { &m->gate, ff }, { &m->up, ff } };
+			for (auto& b : bufs)
+			{
+				LITENN_HIP_TRY(kAction, hipMalloc(reinterpret_cast<void**>(b.p), sizeof(float) * rows * b.n));
+			}
+			LITENN_HIP_TRY(kAction, hipMalloc(reinterpret_cast<void**>(&m->d_tokens), sizeof(int32_t) * rows));
+			m->cap_rows = rows;
+		}
+		if (logit_rows > m->cap_logit_rows)
+		{
+			drop_graph(m);
+			if (m->logits)
+			{
+				(void)hipFree(m->logits);
+				m->logits = nullptr;
+			}
+			LITENN_HIP_TRY(kAction, hipMalloc(reinterpret_cast<void**>(&m->logits),
+			                                  sizeof(float) * logit_rows * static_cast<size_t>(m->p.vocab_size)));
+			m->cap_logit_rows = logit_rows;
+		}
+		return 0;
+	}
+
+	int check_complete(const litenn_hip_llama* m)
+	{
+		if (!m->tok_embd.data || !m->output_norm)
+		{
+			return fail(kAction, "Missing GGUF tensor 'token_embd.weight' or 'output_norm.weight'");
+		}
+		for (const Layer& L : m->layers)
+		{
+			if (!L.wq.data || !L.wk.data || !L.wv.data || !L.wo.data || !L.gate.data || !L.up.data || !L.down.data ||
+			    !L.attn_norm || !L.ffn_norm)
+			{
+				return fail(kAction, "Missing GGUF tensor in a decoder block");
+			}
+		}
+		return 0;
+	}
+
+	void matmul(const Weight& w, const float* x, size_t rows, float* y, const float* residual, unsigned flags,
+	            hipStream_t s)
+	{
+		const bool quant = w.fmt != LITENN_FMT_F16 && w.fmt != LITENN_FMT_F32;
+		if (rows >= 16 && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && w.k % 256 == 0)
+		{
+			launch_gemm(w.fmt, w.data, w.n, w.k, x, rows, y, residual, s);
+		}
+		else
+		{
+			launch_gemv(w.fmt, w.data, w.n, w.k, x, rows, y, residual, s);
+		}
+	}
+
+	// Enqueues the decoder over `rows` tokens whose ids are at `ids` (device); positions start at
+	// counters[0].  Logits are produced for the last `logit_rows` rows into m->logits.
+	void forward(litenn_hip_llama* m, const int32_t* ids, size_t rows, size_t logit_rows, unsigned flags)
+	{
+		hipStream_t s = m->stream;
+		const size_t d = m->p.embedding_length;
+		const size_t H = m->p.head_count, KH = m->p.head_count_kv, hd = m->head_dim;
+		const size_t ff = m->p.feed_forward_length;
+		const int* past_dev = m->d_counters;
+		launch_get_rows_q(m->tok_embd.fmt, m->tok_embd.data, m->tok_embd.n, d, ids, rows, m->x, m->d_err, s);
+		for (Layer& L : m->layers)
+		{
+			launch_rmsnorm(m->x, L.attn_norm, m->p.rms_norm_epsilon, rows, d, m->xn, s);
+			matmul(L.wq, m->xn, rows, m->q, nullptr, flags, s);
+			matmul(L.wk, m->xn, rows, m->k, nullptr, flags, s);
+			matmul(L.wv, m->xn, rows, m->v, nullptr, flags, s);
+			launch_rope_qkv_append(m->q, m->k, m->v, L.kcache, L.vcache, m->p.kv_dtype, past_dev, rows, H, KH, hd,
+			                       m->p.rope_dimension_count, m->cos_t, m->sin_t, s);
+			launch_attn_decode(m->q, L.kcache, L.vcache, m->p.kv_dtype, rows, past_dev, 0, m->p.context_length, H, KH,
+			                   hd, m->attn, s);
+			matmul(L.wo, m->attn, rows, m->x, m->x, flags, s); // x = x + attn . Wo
+			launch_rmsnorm(m->x, L.ffn_norm, m->p.rms_norm_epsilon, rows, d, m->xn, s);
+			matmul(L.gate, m->xn, rows, m->gate, nullptr, flags, s);
+			matmul(L.up, m->xn, rows, m->up, nullptr, flags, s);
+			launch_silu_mul(m->gate, m->up, m->gate, rows * ff, s);
+			matmul(L.down, m->gate, rows, m->x, m->x, flags, s); // x = x + mlp
+		}
+		const size_t first = rows - logit_rows;
+		launch_rmsnorm(m->x + first * d, m->output_norm, m->p.rms_norm_epsilon, logit_rows, d, m->xn, s);
+		const Weight& head = m->output.data ? m->output : m->tok_embd;
+		matmul(head, m->xn, logit_rows, m->logits, nullptr, flags, s);
+	}
+
+	int check_error_flag(litenn_hip_llama* m)
+	{
+		int flag = 0;
+		LITENN_HIP_TRY(kAction, hipMemcpyAsync(&flag, m->d_err, sizeof(int), hipMemcpyDeviceToHost, m->stream));
+		LITENN_HIP_TRY(kAction, hipStreamSynchronize(m->stream));
+		if (flag)
+		{
+			const int zero = 0;
+			(void)hipMemcpy(m->d_err, &zero, sizeof(int), hipMemcpyHostToDevice);
+			return fail(kAction, "GetRows index out of range");
+		}
+		return 0;
+	}
+} // namespace
+
+extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* params, litenn_hip_llama** out)
+{
+	if (!params || !out)
+	{
+		return fail(kAction, "null argument");
+	}
+	const litenn_hip_llama_params& p = *params;
+	// the checks of ParseLLaMAHyperparameters (tools/gguf/GGUFImporter.cpp:603-640)
+	if (p.context_length <= 0 || p.embedding_length <= 0 || p.block_count <= 0 || p.feed_forward_length <= 0 ||
+	    p.vocab_size <= 0)
+	{
+		return fail(kAction, "LLaMA hyperparameters must be greater than zero");
+	}
+	if (p.head_count <= 0 || p.head_count_kv <= 0 || p.embedding_length % p.head_count != 0 ||
+	    p.head_count % p.head_count_kv != 0)
+	{
+		return fail(kAction, "LLaMA head counts must divide the embedding length and each other");
+	}
+	if (!(p.rms_norm_epsilon > 0.0))
+	{
+		return fail(kAction, "LLaMA attention.layer_norm_rms_epsilon must be greater than zero");
+	}
+	if (!(p.rope_freq_base > 0.0) || !(p.rope_freq_scale > 0.0))
+	{
+		return fail(kAction, "LLaMA rope.freq_base and rope.freq_scale must be greater than zero");
+	}
+	const int head_dim = p.embedding_length / p.head_count;
+	int rope_dims = p.rope_dimension_count == 0 ? head_dim : p.rope_dimension_count;
+	if (rope_dims > head_dim || rope_dims % 2 != 0 || rope_dims < 0)
+	{
+		return fail(kAction, "LLaMA rope.dimension_count must be an even value in [2, headDim]");
+	}
+	if (head_dim > 256 || head_dim % 2 != 0)
+	{
+		return fail(kAction, "head dimension must be even and at most 256");
+	}
+	if (p.context_length > 15360)
+	{
+		return fail(kAction, "context length exceeds the 15360 positions the attention score buffer holds");
+	}
+	if (p.kv_dtype != LITENN_F16 && p.kv_dtype != LITENN_F32)
+	{
+		return fail(kAction, "KV cache dtype must be Float16 or Float32");
+	}
+	DeviceGuard guard(dev);
+	if (!guard.ok())
+	{
+		return fail_hip(kAction, guard.error());
+	}
+	auto* m = new litenn_hip_llama();
+	m->dev = dev;
+	m->p = p;
+	m->p.rope_dimension_count = rope_dims;
+	m->head_dim = head_dim;
+	m->layers.resize(static_cast<size_t>(p.block_count));
+	auto bail = [&](hipError_t e) {
+		litenn_hip_llama_free(m);
+		return fail_hip(kAction, e);
+	};
+	hipError_t e = hipStreamCreate(&m->stream);
+	if (e != hipSuccess)
+	{
+		m->stream = nullptr;
+		return bail(e);
+	}
+	const size_t kv_bytes = static_cast<size_t>(p.context_length) * p.head_count_kv * head_dim * dtype_size(p.kv_dtype);
+	for (Layer& L : m->layers)
+	{
+		if ((e = hipMalloc(&L.kcache, kv_bytes)) != hipSuccess || (e = hipMalloc(&L.vcache, kv_bytes)) != hipSuccess)
+		{
+			return bail(e);
+		}
+	}
+	// angle tables in f64 on the host, stored as f32: MakeRoPEAngleTable (Layer/RoPE.h:24-41)
+	const size_t half = static_cast<size_t>(rope_dims) / 2;
+	if (half)
+	{
+		std::vector<float> c(static_cast<size_t>(p.context_length) * half), s(c.size());
+		for (size_t pos = 0; pos < static_cast<size_t>(p.context_length); ++pos)
+		{
+			for (size_t dim = 0; dim < half; ++dim)
+			{
+				const double exponent = -2.0 * static_cast<double>(dim) / static_cast<double>(half * 2);
+				const double inv_freq = std::pow(p.rope_freq_base, exponent);
+				const double angle = static_cast<double>(pos) * inv_freq * p.rope_freq_scale;
+				c[pos * half + dim] = static_cast<float>(std::cos(angle));
+				s[pos * half + dim] = static_cast<float>(std::sin(angle));
+			}
+		}
+		if ((e = hipMalloc(reinterpret_cast<void**>(&m->cos_t), sizeof(float) * c.size())) != hipSuccess ||
+		    (e = hipMalloc(reinterpret_cast<void**>(&m->sin_t), sizeof(float) * c.size())) != hipSuccess ||
+		    (e = hipMemcpy(m->cos_t, c.data(), sizeof(float) * c.size(), hipMemcpyHostToDevice)) != hipSuccess ||
+		    (e = hipMemcpy(m->sin_t, s.data(), sizeof(float) * s.size(), hipMemcpyHostToDevice)) != hipSuccess)
+		{
+			return bail(e);
+		}
+	}
+	if ((e = hipMalloc(reinterpret_cast<void**>(&m->d_counters), 2 * sizeof(int))) != hipSuccess ||
+	    (e = hipMalloc(reinterpret_cast<void**>(&m->d_err), sizeof(int))) != hipSuccess ||
+	    (e = hipMalloc(reinterpret_cast<void**>(&m->d_next), sizeof(int32_t))) != hipSuccess ||
+	    (e = hipMemset(m->d_counters, 0, 2 * sizeof(int))) != hipSuccess ||
+	    (e = hipMemset(m->d_err, 0, sizeof(int))) != hipSuccess ||
+	    (e = hipMemset(m->d_next, 0, sizeof(int32_t))) != hipSuccess)
+	{
+		return bail(e);
+	}
+	*out = m;
+	return 0;
+}
+
+extern "C" int litenn_hip_llama_free(litenn_hip_llama* m)
+{
+	if (!m)
+	{
+		return 0;
+	}
+	DeviceGuard guard(m->dev);
+	if (m->stream)
+	{
+		(void)hipStreamSynchronize(m->stream);
+	}
+	drop_graph(m);
+	free_scratch(m);
+	for (Layer& L : m->layers)
+	{
+		if (L.kcache)
+		{
+			(void)hipFree(L.kcache);
+		}
+		if (L.vcache)
+		{
+			(void)hipFree(L.vcache);
+		}
+	}
+	void* singles[] = { m->cos_t, m->sin_t, m->logits, m->d_next, m->d_out, m->d_counters, m->d_err };
+	for (void* ptr : singles)
+	{
+		if (ptr)
+		{
+			(void)hipFree(ptr);
+		}
+	}
+	if (m->stream)
+	{
+		(void)hipStreamDestroy(m->stream);
+	}
+	delete m;
+	return 0;
+}
+
+extern "C" int litenn_hip_llama_set_tensor(litenn_hip_llama* m, int which, int layer, int fmt, const void* data,
+                                           size_t n, size_t k)
+{
+	if (!m || !data)
+	{
+		return fail(kAction, "null argument");
+	}
+	const size_t d = m->p.embedding_length, hd = m->head_dim;
+	const size_t qw = m->p.head_count * hd, kvw = m->p.head_count_kv * hd, ff = m->p.feed_forward_length;
+	const size_t vocab = m->p.vocab_size;
+	const bool per_layer = which >= LITENN_T_ATTN_Q && which != LITENN_T_OUTPUT_NORM;
+	if (per_layer && (layer < 0 || layer >= m->p.block_count))
+	{
+		return fail(kAction, "layer index out of range");
+	}
+	Layer* L = per_layer ? &m->layers[static_cast<size_t>(layer)] : nullptr;
+	Weight* target = nullptr;
+	size_t want_n = 0, want_k = 0;
+	switch (which)
+	{
+	case LITENN_T_TOKEN_EMBD: target = &m->tok_embd; want_n = vocab; want_k = d; break;
+	case LITENN_T_OUTPUT: target = &m->output; want_n = vocab; want_k = d; break;
+	case LITENN_T_ATTN_Q: target = &L->wq; want_n = qw; want_k = d; break;
+	case LITENN_T_ATTN_K: target = &L->wk; want_n = kvw; want_k = d; break;
+	case LITENN_T_ATTN_V: target = &L->wv; want_n = kvw; want_k = d; break;
+	case LITENN_T_ATTN_OUTPUT: target = &L->wo; want_n = d; want_k = qw; break;
+	case LITENN_T_FFN_GATE: target = &L->gate; want_n = ff; want_k = d; break;
+	case LITENN_T_FFN_UP: target = &L->up; want_n = ff; want_k = d; break;
+	case LITENN_T_FFN_DOWN: target = &L->down; want_n = d; want_k = ff; break;
+	case LITENN_T_OUTPUT_NORM:
+	case LITENN_T_ATTN_NORM:
+	case LITENN_T_FFN_NORM:
+		if (fmt != LITENN_FMT_F32 || n * k != d)
+		{
+			return fail(kAction, "norm weight must be Float32 with shape [embedding_length] or [1, embedding_length]");
+		}
+		if (which == LITENN_T_OUTPUT_NORM)
+		{
+			m->output_norm = static_cast<const float*>(data);
+		}
+		else if (which == LITENN_T_ATTN_NORM)
+		{
+			L->attn_norm = static_cast<const float*>(data);
+		}
+		else
+		{
+			L->ffn_norm = static_cast<const float*>(data);
+		}
+		drop_graph(m);
+		return 0;
+	default:
+		return fail(kAction, "unknown tensor id");
+	}
+	if (n != want_n || k != want_k)
+	{
+		return fail(kAction, "tensor shape does not match the hyper-parameters");
+	}
+	if (row_bytes(fmt, k) == 0)
+	{
+		return fail(kAction, "unsupported block format or row width");
+	}
+	target->fmt = fmt;
+	target->data = data;
+	target->n = n;
+	target->k = k;
+	drop_graph(m);
+	return 0;
+}
+
+extern "C" int litenn_hip_llama_reset(litenn_hip_llama* m)
+{
+	if (!m)
+	{
+		return fail(kAction, "null argument");
+	}
+	m->past = 0;
+	return 0;
+}
+
+extern "C" int litenn_hip_llama_past(const litenn_hip_llama* m)
+{
+	return m ? m->past : -1;
+}
+
+extern "C" int litenn_hip_llama_eval(litenn_hip_llama* m, const int32_t* tokens, size_t rows, float* logits,
+                                     float* last_logits, unsigned flags)
+{
+	if (!m || !tokens)
+	{
+		return fail(kAction, "null argument");
+	}
+	if (rows == 0)
+	{
+		return fail(kAction, "sequence length must be positive");
+	}
+	if (static_cast<size_t>(m->past) + rows > static_cast<size_t>(m->p.context_length))
+	{
+		return fail(kAction, "context length exceeded");
+	}
+	if (check_complete(m) != 0)
+	{
+		return 1;
+	}
+	for (size_t i = 0; i < rows; ++i)
+	{
+		if (tokens[i] < 0 || tokens[i] >= m->p.vocab_size)
+		{
+			return fail(kAction, "GetRows index out of range"); // Device.h:868-871
+		}
+	}
+	DeviceGuard guard(m->dev);
+	if (!guard.ok())
+	{
+		return fail_hip(kAction, guard.error());
+	}
+	const size_t logit_rows = logits ? rows : 1;
+	if (ensure_rows(m, rows, logit_rows) != 0)
+	{
+		return 1;
+	}
+	hipStream_t s = m->stream;
+	LITENN_HIP_TRY(kAction, hipMemcpyAsync(m->d_tokens, tokens, sizeof(int32_t) * rows, hipMemcpyHostToDevice, s));
+	set_counters_kernel<<<1, 1, 0, s>>>(m->d_counters, m->past, 0);
+	forward(m, m->d_tokens, rows, logit_rows, flags);
+	LITENN_HIP_TRY(kAction, hipGetLastError());
+	const size_t vocab = m->p.vocab_size;
+	if (logits)
+	{
+		LITENN_HIP_TRY(kAction, hipMemcpyAsync(logits, m->logits, sizeof(float) * rows * vocab, hipMemcpyDeviceToHost, s));
+	}
+	if (last_logits)
+	{
+		LITENN_HIP_TRY(kAction, hipMemcpyAsync(last_logits, m->logits + (logit_rows - 1) * vocab, sizeof(float) * vocab,
+		                                       hipMemcpyDeviceToHost, s));
+	}
+	if (check_error_flag(m) != 0)
+	{
+		return 1;
+	}
+	m->past += static_cast<int>(rows);
+	return 0;
+}
+
+extern "C" int litenn_hip_llama_generate(litenn_hip_llama* m, const int32_t* prompt, size_t n_prompt, size_t n_new,
+                                         int32_t* out_tokens, unsigned flags, double* prefill_ms, double* decode_ms)
+{
+	if (!m || !prompt || !out_tokens)
+	{
+		return fail(kAction, "null argument");
+	}
+	if (n_prompt == 0 || n_new == 0)
+	{
+		return fail(kAction, "prompt and generation lengths must be positive");
+	}
+	if (static_cast<size_t>(m->past) + n_prompt + n_new - 1 > static_cast<size_t>(m->p.context_length))
+	{
+		return fail(kAction, "context length exceeded");
+	}
+	if (check_complete(m) != 0)
+	{
+		return 1;
+	}
+	for (size_t i = 0; i < n_prompt; ++i)
+	{
+		if (prompt[i] < 0 || prompt[i] >= m->p.vocab_size)
+		{
+			return fail(kAction, "GetRows index out of range");
+		}
+	}
+	DeviceGuard guard(m->dev);
+	if (!guard.ok())
+	{
+		return fail_hip(kAction, guard.error());
+	}
+	if (ensure_rows(m, n_prompt, 1) != 0)
+	{
+		return 1;
+	}
+	if (n_new > m->cap_out)
+	{
+		drop_graph(m);
+		if (m->d_out)
+		{
+			(void)hipFree(m->d_out);
+			m->d_out = nullptr;
+		}
+		LITENN_HIP_TRY(kAction, hipMalloc(reinterpret_cast<void**>(&m->d_out), sizeof(int32_t) * n_new));
+		m->cap_out = n_new;
+	}
+	hipStream_t s = m->stream;
+	hipEvent_t ev[3];
+	for (hipEvent_t& e : ev)
+	{
+		LITENN_HIP_TRY(kAction, hipEventCreate(&e));
+	}
+	int rc = 0;
+	auto cleanup = [&]() {
+		for (hipEvent_t& e : ev)
+		{
+			(void)hipEventDestroy(e);
+		}
+	};
+#define GEN_TRY(expr)                                                                                                  \
+	do                                                                                                                 \
+	{                                                                                                                  \
+		const hipError_t e_ = (expr);                                                                                  \
+		if (e_ != hipSuccess)                                                                                          \
+		{                                                                                                              \
+			cleanup();                                                                                                 \
+			return fail_hip(kAction, e_);                                                                              \
+		}                                                                                                              \
+	} while (0)
+
+	// prompt: one pass over n_prompt rows, logits of the last row only, first token from its arg-max
+	GEN_TRY(hipMemcpyAsync(m->d_tokens, prompt, sizeof(int32_t) * n_prompt, hipMemcpyHostToDevice, s));
+	set_counters_kernel<<<1, 1, 0, s>>>(m->d_counters, m->past, 0);
+	GEN_TRY(hipEventRecord(ev[0], s));
+	forward(m, m->d_tokens, n_prompt, 1, flags);
+	launch_argmax(m->logits, 1, m->p.vocab_size, m->d_next, s);
+	advance_kernel<<<1, 1, 0, s>>>(m->d_counters, static_cast<int>(n_prompt), m->d_next, m->d_out);
+	GEN_TRY(hipEventRecord(ev[1], s));
+	GEN_TRY(hipGetLastError());
+
+	// single-token steps: embed d_next at position counters[0], arg-max, append.  The step is
+	// captured once; every replay reads its position from device memory.
+	const char* graph_env = getenv("LITENN_HIP_GRAPH");
+	const bool use_graph = !(graph_env && graph_env[0] == '0');
+	if (n_new > 1)
+	{
+		if (use_graph && !m->step_exec)
+		{
+			GEN_TRY(hipStreamSynchronize(s));
+			hipError_t ce = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
+			if (ce == hipSuccess)
+			{
+				forward(m, m->d_next, 1, 1, flags);
+				launch_argmax(m->logits, 1, m->p.vocab_size, m->d_next, s);
+				advance_kernel<<<1, 1, 0, s>>>(m->d_counters, 1, m->d_next, m->d_out);
+				ce = hipStreamEndCapture(s, &m->step_graph);
+			}
+			if (ce == hipSuccess)
+			{
+				ce = hipGraphInstantiate(&m->step_exec, m->step_graph, nullptr, nullptr, 0);
+			}
+			if (ce != hipSuccess)
+			{
+				drop_graph(m);
+				cleanup();
+				return fail_hip(kAction, ce);
+			}
+		}
+		for (size_t i = 1; i < n_new; ++i)
+		{
+			if (use_graph)
+			{
+				GEN_TRY(hipGraphLaunch(m->step_exec, s));
+			}
+			else
+			{
+				forward(m, m->d_next, 1, 1, flags);
+				launch_argmax(m->logits, 1, m->p.vocab_size, m->d_next, s);
+				advance_kernel<<<1, 1, 0, s>>>(m->d_counters, 1, m->d_next, m->d_out);
+			}
+		}
+	}
+	GEN_TRY(hipEventRecord(ev[2], s));
+	GEN_TRY(hipGetLastError());
+	GEN_TRY(hipMemcpyAsync(out_tokens, m->d_out, sizeof(int32_t) * n_new, hipMemcpyDeviceToHost, s));
+	GEN_TRY(hipStreamSynchronize(s));
+	float ms = 0.0f;
+	if (prefill_ms)
+	{
+		GEN_TRY(hipEventElapsedTime(&ms, ev[0], ev[1]));
+		*prefill_ms = ms;
+	}
+	if (decode_ms)
+	{
+		GEN_TRY(hipEventElapsedTime(&ms, ev[1], ev[2]));
+		*decode_ms = ms;
+	}
+	cleanup();
+#undef GEN_TRY
+	// the last emitted token has not been fed back: the cache holds prompt + (n_new - 1) rows
+	m->past += static_cast<int>(n_prompt + n_new - 1);
+	return rc;
+}
+
+extern "C" int litenn_hip_llama_get_kv(litenn_hip_llama* m, int layer, float* k, float* v)
+{
+	if (!m || layer < 0 || layer >= m->p.block_count)
+	{
+		return fail(kAction, "layer index out of range");
+	}
+	DeviceGuard guard(m->dev);
+	if (!guard.ok())
+	{
+		return fail_hip(kAction, guard.error());
+	}
+	const size_t count = static_cast<size_t>(m->past) * m->p.head_count_kv * m->head_dim;
+	if (count == 0)
+	{
+		return 0;
+	}
+	LITENN_HIP_TRY(kAction, hipStreamSynchronize(m->stream));
+	float* tmp = nullptr;
+	LITENN_HIP_TRY(kAction, hipMalloc(reinterpret_cast<void**>(&tmp), sizeof(float) * count));
+	int rc = 0;
+	const Layer& L = m->layers[static_cast<size_t>(layer)];
+	const void* caches[2] = { L.kcache, L.vcache };
+	float* outs[2] = { k, v };
+	for (int i = 0; i < 2 && rc == 0; ++i)
+	{
+		if (!launch_convert(m->p.kv_dtype, caches[i], count, LITENN_F32, tmp, m->stream))
+		{
+			rc = fail(kAction, "cache conversion failed");
+			break;
+		}
+		const void* src = tmp;
+		hipError_t e = hipMemcpyAsync(outs[i], src, sizeof(float) * count, hipMemcpyDeviceToHost, m->stream);
+		if (e == hipSuccess)
+		{
+			e = hipStreamSynchronize(m->stream);
+		}
+		if (e != hipSuccess)
+		{
+			rc = fail_hip(kAction, e);
+		}
+	}
+	(void)hipFree(tmp);
+	return rc;
+}

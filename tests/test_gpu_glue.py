@@ -1,0 +1,123 @@
+"""Parity of the decoder's small kernels (through the C ABI) with the CPU checker and with the
+reference's own test vectors."""
+import math
+
+import numpy as np
+import pytest
+
+from conftest import rel_l2
+from litenn_amd.formats import DT_F16, DT_F32
+
+pytestmark = pytest.mark.gpu
+
+
+def T(hip, a, dtype=np.float32):
+    return hip.Tensor.from_numpy(np.ascontiguousarray(a, dtype))
+
+
+def test_rmsnorm(hip, oracle, golden):
+    rng = np.random.default_rng(1)
+    for m, d in [(1, 4096), (3, 257), (16, 11008)]:
+        x = (rng.standard_normal((m, d)) * 7).astype(np.float32)
+        w = rng.standard_normal(d).astype(np.float32)
+        eps = float(np.float32(1e-5))
+        got = hip.rmsnorm(T(hip, x), T(hip, w), eps).numpy()
+        want = oracle.rmsnorm(x, w, eps)
+        # f64 accumulation on both sides: at most one f32 ulp apart
+        assert np.max(np.abs(got.view(np.int32) - want.view(np.int32))) <= 1
+        assert np.array_equal(hip.rmsnorm(T(hip, x), None, eps).numpy(), oracle.rmsnorm(x, None, eps)) or \
+            rel_l2(hip.rmsnorm(T(hip, x), None, eps).numpy(), oracle.rmsnorm(x, None, eps)) < 1e-7
+    c = golden["rmsnorm"][2]
+    got = hip.rmsnorm(T(hip, c["x"]), T(hip, c["w"]), c["eps"]).numpy()[0]
+    denom = math.sqrt(14.0 / 3.0 + 1e-6)
+    assert np.allclose(got, [2 * v / denom for v in (1, 2, 3)], atol=c["tol"])
+    zero = golden["rmsnorm"][1]
+    assert np.all(hip.rmsnorm(T(hip, zero["x"]), T(hip, zero["w"]), zero["eps"]).numpy() == 0)
+
+
+def test_rope(hip, oracle, golden):
+    rng = np.random.default_rng(2)
+    for m, heads, hd, base, off, rd in [(1, 32, 128, 1e4, 0, None), (5, 8, 128, 5e5, 1000, None),
+                                         (3, 2, 64, 1e4, 17, 32), (2, 1, 4, 1.0, 1, None)]:
+        x = rng.standard_normal((m, heads * hd)).astype(np.float32)
+        got = hip.rope_interleaved(T(hip, x), heads, hd, base, off, rope_dims=rd).numpy()
+        want = np.concatenate([oracle.rope(x[:, h * hd:(h + 1) * hd].copy(), base, off, rope_dims=rd)
+                               for h in range(heads)], axis=1)
+        # device f64 cos/sin may differ from the host's by an ulp before rounding to f32
+        assert np.allclose(got, want, rtol=0, atol=2e-6 * max(1.0, float(np.abs(x).max())))
+    c = golden["rope"][1]
+    y = hip.rope_interleaved(T(hip, c["x"]), 1, 4, c["base"], c["pos_offset"]).numpy()
+    assert np.allclose(y[1], [math.cos(1), math.sin(1), -math.sin(1), math.cos(1)], atol=c["tol"])
+    with pytest.raises(hip.LiteNNHipError, match="even"):
+        hip.rope_interleaved(T(hip, np.zeros((2, 3))), 1, 3)
+
+
+def test_kv_append_f16_uses_litenn_rounding(hip, oracle, golden):
+    rng = np.random.default_rng(3)
+    cur = np.concatenate([rng.standard_normal(4096) * 30,
+                          [1.0 + 2.0**-11, -(2.0 + 2.0**-10), 65520.0, 3.1e-8, 1e-6, -0.0]]).astype(np.float32)
+    width = cur.size // 2
+    cache = hip.Tensor((8, width), DT_F16)
+    hip.DeviceTraits.ZeroFill(hip.HIP(0), cache.ptr, DT_F16, cache.size)
+    hip.kv_append(cache, 3, T(hip, cur), width)
+    raw = cache.numpy()  # float16 view
+    assert np.array_equal(raw[3:5].reshape(-1).view(np.uint16), oracle.f32_to_f16_bits(cur))
+    assert np.all(raw[:3] == 0) and np.all(raw[5:] == 0)
+    g = golden["kv_append"]
+    c32 = hip.Tensor((3, 2), DT_F32)
+    hip.kv_append(c32, 0, T(hip, g["past_k"]), 2)
+    hip.kv_append(c32, 2, T(hip, g["new_k"]), 2)
+    assert np.array_equal(c32.numpy(), np.array(g["expected_k"], np.float32))
+
+
+@pytest.mark.parametrize("cache_dtype", [DT_F32, DT_F16])
+def test_attention_decode(hip, oracle, cache_dtype):
+    rng = np.random.default_rng(4)
+    for m, past, H, KH, hd in [(1, 0, 4, 4, 128), (1, 383, 32, 32, 128), (1, 1023, 32, 8, 128), (6, 10, 8, 2, 64),
+                               (2, 1, 2, 1, 2), (3, 0, 4, 2, 80)]:
+        L = past + m
+        q = rng.standard_normal((m, H * hd)).astype(np.float32)
+        k = rng.standard_normal((L, KH * hd)).astype(np.float32)
+        v = rng.standard_normal((L, KH * hd)).astype(np.float32)
+        if cache_dtype == DT_F16:
+            k = oracle.f16_to_f32(oracle.f32_to_f16_bits(k))
+            v = oracle.f16_to_f32(oracle.f32_to_f16_bits(v))
+            kc, vc = T(hip, k, np.float16), T(hip, v, np.float16)
+        else:
+            kc, vc = T(hip, k), T(hip, v)
+        got = hip.attn_decode(T(hip, q), kc, vc, m, past, H, KH, hd).numpy()
+        want = np.empty_like(got)
+        for h in range(H):
+            kvh = h // (H // KH)
+            want[:, h * hd:(h + 1) * hd] = oracle.attention_head(
+                q[:, h * hd:(h + 1) * hd].copy(), k[:, kvh * hd:(kvh + 1) * hd].copy(),
+                v[:, kvh * hd:(kvh + 1) * hd].copy(), 1.0 / math.sqrt(hd), True, 0, past)
+        assert rel_l2(got, want) < 1e-5, (m, past, H, KH, hd)
+
+
+def test_attention_reference_vectors(hip, golden):
+    c0, c1 = golden["attention"]
+    # causal 3x3, head_dim 2 (scale 1/sqrt(2) is the kernel's own 1/sqrt(head_dim))
+    # values are [L, 1] in the reference case; widen to head_dim 2 with a zero column
+    v2 = np.concatenate([np.array(c0["v"], np.float32), np.zeros((3, 1), np.float32)], axis=1)
+    got = hip.attn_decode(T(hip, c0["q"]), T(hip, c0["k"]), T(hip, v2), 3, 0, 1, 1, 2).numpy()
+    q, k, v = (np.array(c0[n], np.float64) for n in ("q", "k", "v"))
+    for row in range(3):
+        s = (k[:row + 1] @ q[row]) / math.sqrt(2.0)
+        p = np.exp(s - s.max())
+        p /= p.sum()
+        assert abs(got[row, 0] - float(p @ v[:row + 1, 0])) < c0["tol"]
+        assert got[row, 1] == 0.0
+
+
+def test_silu_mul_and_argmax(hip, oracle):
+    rng = np.random.default_rng(5)
+    g = (rng.standard_normal(11008 * 3) * 4).astype(np.float32)
+    u = rng.standard_normal(11008 * 3).astype(np.float32)
+    got = hip.silu_mul(T(hip, g), T(hip, u)).numpy()
+    assert rel_l2(got, oracle.silu_mul(g, u)) < 1e-6
+    x = rng.standard_normal((3, 128256)).astype(np.float32)
+    x[1, 500] = x[1, 90000] = 99.0  # tie: lowest index wins
+    x[2, :] = -np.inf
+    idx = hip.argmax(T(hip, x)).numpy()
+    assert idx.tolist() == [int(np.argmax(x[0])), 500, 0]
