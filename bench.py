@@ -143,6 +143,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--buffers", type=int, default=16)
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--decode-prompt", type=int, default=128, help="prompt length of the decode run")
+    ap.add_argument("--decode-new", type=int, default=256, help="tokens generated by the decode run")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -203,7 +205,7 @@ def main() -> int:
         }
         log(f"[bench] CPU baseline: {s_per_call * 1e3:.1f} ms/call over {calls} calls")
     if not args.no_decode:
-        line["decode"] = bench_decode(ln)
+        line["decode"] = bench_decode(ln, args.decode_prompt, args.decode_new)
         log(f"[bench] decode: {line['decode']['tokens_per_s']} tok/s")
     print(json.dumps(line), flush=True)
     return 0

@@ -184,7 +184,11 @@ def mul_mat_q(fmt: int, wq: Tensor, n: int, k: int, x: Tensor, y: Tensor | None 
               flags: int = 0, stream=None, synchronize: bool = True) -> Tensor:
     """y[m, n] = x[m, k] . deq(wq)[n, k]^T (+ residual); wq holds the raw GGUF payload."""
     m = x.size // k if k else 0
-    if wq.size * DTYPE_SIZE[wq.dtype] != n * row_bytes(fmt, k):
+    try:
+        expected = n * row_bytes(fmt, k)
+    except ValueError:
+        expected = None  # unknown format or ragged row: the C ABI reports it
+    if expected is not None and wq.size * DTYPE_SIZE[wq.dtype] != expected:
         raise LiteNNHipError("HIP quantized matmul failed: payload size does not match [n, k] for this format")
     if y is None:
         y = Tensor((m, n), DT_F32, x.device)

@@ -118,7 +118,7 @@ def test_errors_and_empty_inputs(hip):
         hip.mul_mat_q(Q4_K, wq, 2, 256, x)
     with pytest.raises(hip.LiteNNHipError, match="unsupported block format"):
         hip.mul_mat_q(2, wq, 1, 256, x)
-    with pytest.raises(ValueError):
+    with pytest.raises(hip.LiteNNHipError, match="block size"):
         hip.mul_mat_q(Q4_K, wq, 1, 128, x)
     empty = hip.mul_mat_q(Q4_K, hip.Tensor.from_numpy(np.zeros(0, np.uint8)), 0, 256, x)
     assert empty.shape == (1, 0)
