@@ -127,6 +127,19 @@ int litenn_hip_permute(int dev, void* dst, int dtype, const size_t* src_shape, s
 #define LITENN_HIP_MATMUL_PRECISE 1u
 int litenn_hip_mul_mat_q(int dev, int fmt, const void* wq, size_t n, size_t k, const void* x, int x_dtype, size_t m,
                          void* y, const void* residual, unsigned flags, const litenn_hip_exec* opts);
+/* One activation row through an operator group of the decoder block, fused into a single
+ * launch when the shape allows and composed from separate launches otherwise:
+ *   [RMSNorm(x, norm_w, eps)] -> count (1..3) linears of one format sharing that input
+ *   -> [residual added to y[0]] or [SwiGLU: y[0] = silu(x.W0) * (x.W1)]
+ * i.e. AddRMSNorm + AddLinear x3 (tools/gguf/LLaMABuilder.cpp:588-591), the front half of
+ * AddSwiGLUMLP (src/LiteNN/Layer/SwiGLU.h:59-66), or AddLinear + Add (:652-653,661-663).
+ * wq[i] is [n[i], k] raw payload, y[i] f32 [n[i]]; norm_w (f32 [k]) and residual (f32 [n[0]],
+ * count == 1 only, may alias y[0]) may be NULL; with LITENN_HIP_GROUP_SILU_MUL count must be 2
+ * with n[0] == n[1] and only y[0] is written. */
+#define LITENN_HIP_GROUP_SILU_MUL 1u
+int litenn_hip_linear_group(int dev, int fmt, size_t count, const void* const* wq, const size_t* n, size_t k,
+                            const void* x, void* const* y, const void* residual, const void* norm_w, double eps,
+                            unsigned flags, const litenn_hip_exec* opts);
 /* f32 [rows, k] = dequantised rows of wq (ggml to_float as called at
  * tools/gguf/LLaMABuilder.cpp:144-150). */
 int litenn_hip_dequantize(int dev, int fmt, const void* wq, size_t rows, size_t k, void* dst,

@@ -7,10 +7,10 @@ GPU; the first call that needs the library loads it and raises if it has not bee
 from . import formats, synth
 from ._lib import LiteNNHipError, LIB_PATH
 from .device import (HIP, DeviceTraits, HIPDeviceCount, IsHIPDeviceAvailable, Tensor, argmax, attn_decode,
-                     dequantize, get_rows_q, kv_append, mul_mat_q, rmsnorm, rope_interleaved, silu_mul,
+                     dequantize, get_rows_q, kv_append, linear_group, mul_mat_q, rmsnorm, rope_interleaved, silu_mul,
                      MATMUL_PRECISE)
 from .llama import LLaMA
 
 __all__ = ["formats", "synth", "LiteNNHipError", "LIB_PATH", "HIP", "DeviceTraits", "HIPDeviceCount",
            "IsHIPDeviceAvailable", "Tensor", "argmax", "attn_decode", "dequantize", "get_rows_q", "kv_append",
-           "mul_mat_q", "rmsnorm", "rope_interleaved", "silu_mul", "MATMUL_PRECISE", "LLaMA"]
+           "mul_mat_q", "linear_group", "rmsnorm", "rope_interleaved", "silu_mul", "MATMUL_PRECISE", "LLaMA"]

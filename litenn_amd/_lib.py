@@ -50,6 +50,7 @@ SIGNATURES = {
     "litenn_hip_get_rows": [_i, _vp, _i, _szp, _sz, _vp, _i, _szp, _sz, _vp, _ex],
     "litenn_hip_permute": [_i, _vp, _i, _szp, _sz, _vp, _szp, _ex],
     "litenn_hip_mul_mat_q": [_i, _i, _vp, _sz, _sz, _vp, _i, _sz, _vp, _vp, _u, _ex],
+    "litenn_hip_linear_group": [_i, _i, _sz, C.POINTER(_vp), _szp, _sz, _vp, C.POINTER(_vp), _vp, _vp, _d, _u, _ex],
     "litenn_hip_dequantize": [_i, _i, _vp, _sz, _sz, _vp, _ex],
     "litenn_hip_get_rows_q": [_i, _i, _vp, _sz, _sz, _vp, _sz, _vp, _ex],
     "litenn_hip_rmsnorm": [_i, _vp, _vp, _d, _sz, _sz, _vp, _ex],

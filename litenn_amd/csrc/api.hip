@@ -15,6 +15,9 @@ namespace litenn_hip
 	                const float* residual, hipStream_t stream);
 	int launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
 	                const float* residual, hipStream_t stream);
+	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
+	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
+	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream);
 	void launch_dequantize(int fmt, const void* wq, size_t rows, size_t k, float* dst, hipStream_t stream);
 	void launch_get_rows_q(int fmt, const void* table, size_t rows, size_t k, const int32_t* ids, size_t n_ids,
 	                       float* out, int* err_flag, hipStream_t stream);
@@ -522,6 +525,67 @@ extern "C" int litenn_hip_mul_mat_q(int dev, int fmt, const void* wq, size_t n, 
 		launch_gemv(fmt, wq, n, k, xf, m, yf, rf, s);
 	}
 	return finish(action, opts);
+}
+
+extern "C" int litenn_hip_linear_group(int dev, int fmt, size_t count, const void* const* wq, const size_t* n, size_t k,
+                                       const void* x, void* const* y, const void* residual, const void* norm_w,
+                                       double eps, unsigned flags, const litenn_hip_exec* opts)
+{
+	const char* action = "HIP linear group";
+	const bool silu = (flags & LITENN_HIP_GROUP_SILU_MUL) != 0;
+	if (!is_weight_format(fmt))
+	{
+		return fail(action, "unsupported block format");
+	}
+	if (count < 1 || count > 3 || !wq || !n || !y || !x)
+	{
+		return fail(action, "a group holds one to three matrices");
+	}
+	if (row_bytes(fmt, k) == 0 || k == 0)
+	{
+		return fail(action, "row width is incompatible with the block size of the format");
+	}
+	if (silu && (count != 2 || n[0] != n[1]))
+	{
+		return fail(action, "SwiGLU needs exactly two matrices of equal height");
+	}
+	if (residual && count != 1)
+	{
+		return fail(action, "a residual goes with a single matrix");
+	}
+	if (norm_w && !(eps > 0.0))
+	{
+		return fail(action, "RMSNorm epsilon must be greater than zero");
+	}
+	float* ys[3] = { nullptr, nullptr, nullptr };
+	for (size_t i = 0; i < count; ++i)
+	{
+		if (n[i] == 0 || n[i] > 0x3fffffffu || k > 0x7fffffffu || !wq[i] || (!y[i] && !(silu && i == 1)))
+		{
+			return fail(action, "bad matrix in the group");
+		}
+		ys[i] = static_cast<float*>(y[i]);
+	}
+	GUARD(action, dev);
+	hipStream_t s = stream_of(opts);
+	// scratch for the composed form; private to the call, so it always completes before returning
+	float* scratch = nullptr;
+	const size_t scratch_floats = k + 2 * n[0];
+	LITENN_HIP_TRY(action, hipMalloc(reinterpret_cast<void**>(&scratch), sizeof(float) * scratch_floats));
+	launch_linear_group(fmt, static_cast<int>(count), wq, ys, n, k, static_cast<const float*>(x),
+	                    static_cast<const float*>(residual), static_cast<const float*>(norm_w), eps, silu, scratch,
+	                    scratch + k, scratch + k + n[0], s);
+	hipError_t e = hipGetLastError();
+	if (e == hipSuccess)
+	{
+		e = hipStreamSynchronize(s);
+	}
+	(void)hipFree(scratch);
+	if (e != hipSuccess)
+	{
+		return fail_hip(action, e);
+	}
+	return 0;
 }
 
 extern "C" int litenn_hip_dequantize(int dev, int fmt, const void* wq, size_t rows, size_t k, void* dst,

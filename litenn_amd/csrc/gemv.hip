@@ -2,23 +2,24 @@
 //
 //   y[n] = sum_k x[k] * deq(W)[n, k]        (+ residual[n])
 //
-// W is the raw .gguf payload: row n is K/block consecutive blocks.  The kernel is
-// HBM-bound by construction: each weight byte is read exactly once with wide
-// coalesced loads, and everything else stays on chip.
+// W is the raw .gguf payload: row n is K/block consecutive blocks.  The kernels are HBM-bound by
+// construction: each weight byte is read exactly once with wide coalesced loads, and everything
+// else stays on chip.
 //
-// Work decomposition
-//   * a "unit" is 64 weights of one row handled by one lane: a Q4_0/Q8_0 block pair,
-//     one 64-wide group of a Q4_K super-block, or a quarter of a Q6_K super-block.
-//   * a wavefront owns one 4096-wide slice of K (64 lanes x 64 weights).  The lane keeps
-//     its 64 activations in registers for the whole kernel, so the inner loop touches
-//     neither LDS nor L2 for x: it is weight loads, nibble unpack and FMAs only.
-//   * the wavefront walks down a run of consecutive rows (contiguous in memory), RU rows
-//     per trip so RU independent wide loads are in flight per lane.
-//   * per row the 64 lane partials are summed with DPP (no LDS); when K > 4096 the
-//     slices of one row live in sibling wavefronts of the workgroup and meet in LDS.
+// Work decomposition (both kernels)
+//   * a "unit" is 64 weights of one row handled by one lane: a Q4_0/Q8_0 block pair, one 64-wide
+//     group of a Q4_K super-block, or a quarter of a Q6_K super-block.
+//   * a wavefront owns one 4096-wide slice of K (64 lanes x 64 weights).  The lane keeps its 64
+//     activations in registers for the whole kernel (staged once per workgroup through LDS), so
+//     the row loop is weight traffic, nibble unpack and FMAs only.
+//   * the wavefront walks down a run of consecutive rows (contiguous in memory).
+//   * per row the 64 lane partials are summed with DPP (no LDS); when K > 4096 the slices of one
+//     row live in sibling wavefronts of the workgroup and meet in LDS.
 //   * per-block constants are factored out of the inner loop:
 //       sum_k (q_k - z) * s * x_k = s * (sum_k q_k x_k  -  z * sum_k x_k)
 //     and sum_k x_k over each block is a per-lane constant computed once.
+//   * quants enter the FMA as binary16 subnormals (value * 2^-24), so no int->float conversion
+//     is issued: a mask produces the operand of v_fma_mix_f32.
 #include "common.hpp"
 
 #include <cstdlib>
@@ -102,6 +103,16 @@ namespace litenn_hip
 		{
 			asm volatile("ds_write_b128 %0, %1" : : "v"(addr), "v"(v) : "memory");
 		}
+		__device__ __forceinline__ void lds_wr64(uint32_t addr, double v)
+		{
+			asm volatile("ds_write_b64 %0, %1" : : "v"(addr), "v"(v) : "memory");
+		}
+		__device__ __forceinline__ double lds_rd_f64(uint32_t addr)
+		{
+			double v;
+			asm volatile("ds_read_b64 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
+			return v;
+		}
 		__device__ __forceinline__ void lds_wr32(uint32_t addr, float v)
 		{
 			asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(v) : "memory");
@@ -183,15 +194,25 @@ namespace litenn_hip
 		constexpr float kLoNibbleScale = 16777216.0f; // 2^24
 		constexpr float kHiNibbleScale = 1048576.0f;  // 2^20
 
+		// sum of n (16 or 32) consecutive registers as a balanced tree (short dependency chains)
 		__device__ __forceinline__ float sum_run(const float* x, int n)
 		{
-			float s = 0.0f;
+			float t[32];
 #pragma unroll
-			for (int i = 0; i < n; ++i)
+			for (int i = 0; i < 32; ++i)
 			{
-				s += x[i];
+				t[i] = i < n ? x[i] : 0.0f;
 			}
-			return s;
+#pragma unroll
+			for (int w = 16; w >= 1; w >>= 1)
+			{
+#pragma unroll
+				for (int i = 0; i < w; ++i)
+				{
+					t[i] += t[i + w];
+				}
+			}
+			return t[0];
 		}
 
 		// ------------------------------------------------------------------
@@ -512,212 +533,6 @@ namespace litenn_hip
 			}
 		}
 
-		constexpr int kMaxSlices = 8;       // K <= 32768
-		constexpr int kMaxRowsPerWave = 64; // bound of the LDS exchange buffer
-		constexpr int kLdsUnitStride = 68;  // floats between the staged activations of consecutive units
-		constexpr size_t kMaxLdsBytes = 96 * 1024;
-		constexpr int kXPerThread = 8;      // float4 loads of x per thread while staging
-
-		template <typename U, int RU>
-		__device__ __forceinline__ void load_batch(typename U::Raw (&raw)[RU], const uint8_t* __restrict__ w,
-		                                           size_t row_bytes, int r, int row_end, int unit)
-		{
-#pragma unroll
-			for (int u = 0; u < RU; ++u)
-			{
-				const int rr = min(r + u, row_end - 1); // the tail repeats the last row; results are dropped
-				raw[u] = U::load(w + static_cast<size_t>(rr) * row_bytes, unit);
-			}
-		}
-
-		// grid.x workgroups; workgroup = slices x groups wavefronts.  Wavefront (s, g) of
-		// workgroup b handles slice s of rows [ (b*groups + g) * rows_per_wave, +rows_per_wave ).
-		// Dynamic LDS: [k/64 units of staged x when x_in_lds][slices * groups * rows_per_wave partials
-		// when slices > 1].
-		template <typename U, int RU>
-		__global__ __launch_bounds__(512) void gemv_kernel(const uint8_t* __restrict__ w,
-		                                                    const float* __restrict__ x, float* __restrict__ y,
-		                                                    const float* __restrict__ residual, int n, int k,
-		                                                    size_t row_bytes, int slices, int groups,
-		                                                    int rows_per_wave, int x_in_lds)
-		{
-			extern __shared__ __attribute__((aligned(16))) float smem[];
-			float* part = smem + (x_in_lds ? (k >> 6) * kLdsUnitStride : 0);
-			const int lane = threadIdx.x & 63;
-			// the wavefront index is uniform: keeping it in a scalar register makes every row
-			// address, bound and branch below scalar work
-			const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-			const int s = wave % slices;
-			const int g = wave / slices;
-			const int unit = s * 64 + lane; // unit index within the row
-			const int units_per_row = k >> 6;
-			const bool active = unit < units_per_row;
-			const int row0 = (blockIdx.x * groups + g) * rows_per_wave;
-			const int row_end = min(row0 + rows_per_wave, n);
-			const bool has_rows = row0 < row_end;
-
-			// 1. activations: the oldest loads in flight, so waiting for them never waits for weights
-			float4 xv[kXPerThread];
-			if (x_in_lds)
-			{
-#pragma unroll
-				for (int j = 0; j < kXPerThread; ++j)
-				{
-					const int i = (threadIdx.x + j * blockDim.x) * 4;
-					if (i < k)
-					{
-						xv[j] = *reinterpret_cast<const float4*>(x + i);
-					}
-				}
-			}
-
-			// 2. the first two weight batches go out before anything is waited for
-			typename U::Raw a[RU], b[RU];
-			if (active && has_rows)
-			{
-				load_batch<U, RU>(a, w, row_bytes, row0, row_end, unit);
-				if (row0 + RU < row_end)
-				{
-					load_batch<U, RU>(b, w, row_bytes, row0 + RU, row_end, unit);
-				}
-			}
-
-			// 3. activations are staged once per workgroup in LDS; each float4 lands in the slot of
-			// the unit that will consume it.  Units are kLdsUnitStride floats apart so that the
-			// per-lane 128-bit reads below (one unit per lane) fall on distinct banks.  Each lane
-			// then keeps its 64 values in registers for the whole row loop.
-			float xr[64];
-			if (x_in_lds)
-			{
-#pragma unroll
-				for (int j = 0; j < kXPerThread; ++j)
-				{
-					const int i = (threadIdx.x + j * blockDim.x) * 4;
-					if (i < k)
-					{
-						*reinterpret_cast<float4*>(smem + U::unit_of(i) * kLdsUnitStride + U::index_of(i)) = xv[j];
-					}
-				}
-				__syncthreads();
-			}
-			if (active)
-			{
-				// x_offset maps runs of >= 16 consecutive i to consecutive k: 128-bit accesses
-				if (x_in_lds)
-				{
-#pragma unroll
-					for (int i = 0; i < 64; i += 4)
-					{
-						const float4 v = *reinterpret_cast<const float4*>(smem + unit * kLdsUnitStride + i);
-						xr[i] = v.x;
-						xr[i + 1] = v.y;
-						xr[i + 2] = v.z;
-						xr[i + 3] = v.w;
-					}
-				}
-				else
-				{
-#pragma unroll
-					for (int i = 0; i < 64; i += 4)
-					{
-						const float4 v = *reinterpret_cast<const float4*>(x + U::x_offset(unit, i));
-						xr[i] = v.x;
-						xr[i + 1] = v.y;
-						xr[i + 2] = v.z;
-						xr[i + 3] = v.w;
-					}
-				}
-			}
-			else
-			{
-#pragma unroll
-				for (int i = 0; i < 64; ++i)
-				{
-					xr[i] = 0.0f;
-				}
-			}
-			const typename U::Prep pz = U::prep(xr);
-
-			// lane i keeps the total of row row0 + i; everything is written once after the loop, so no
-			// store or residual load sits between the weight loads in flight
-			float res = 0.0f;
-			auto emit = [&](int rr, float total) { res = (lane == rr - row0) ? total : res; };
-			auto compute = [&](const typename U::Raw (&raw)[RU], int r) {
-#pragma unroll
-				for (int u = 0; u < RU; ++u)
-				{
-					const float p = active ? unit_dot<U>(raw[u], xr, pz, unit) : 0.0f;
-					emit(r + u, wave_sum(p));
-				}
-			};
-
-			// ping-pong over two register batches: while one is unpacked and accumulated, the other
-			// (and the reload of the one just consumed) is in flight
-			for (int r = row0; r < row_end;)
-			{
-				compute(a, r);
-				r += RU;
-				if (r >= row_end)
-				{
-					break;
-				}
-				if (active && r + RU < row_end)
-				{
-					load_batch<U, RU>(a, w, row_bytes, r + RU, row_end, unit);
-				}
-				compute(b, r);
-				r += RU;
-				if (active && r + RU < row_end)
-				{
-					load_batch<U, RU>(b, w, row_bytes, r + RU, row_end, unit);
-				}
-			}
-
-			const int count = row_end - row0;
-			if (slices == 1)
-			{
-				if (lane < count)
-				{
-					y[row0 + lane] = residual ? residual[row0 + lane] + res : res;
-				}
-				return;
-			}
-			if (lane < count)
-			{
-				part[s * (groups * rows_per_wave) + g * rows_per_wave + lane] = res;
-			}
-			__syncthreads();
-			const int per_block = groups * rows_per_wave;
-			for (int t = threadIdx.x; t < per_block; t += blockDim.x)
-			{
-				const int gg = t / rows_per_wave;
-				const int rr = (blockIdx.x * groups + gg) * rows_per_wave + (t % rows_per_wave);
-				if (rr < n)
-				{
-					float total = part[t];
-					for (int ss = 1; ss < slices; ++ss)
-					{
-						total += part[ss * per_block + t];
-					}
-					y[rr] = residual ? residual[rr] + total : total;
-				}
-			}
-		}
-
-
-		// ------------------------------------------------------------------
-		// Streaming kernel: rows go HBM -> LDS with direct, fully coalesced 128-bit loads.
-		//
-		// Each wavefront owns RB consecutive rows of one 4096-wide slice and keeps PD of them in
-		// flight: consecutive lanes fetch consecutive 16-byte chunks, every cache line is consumed by
-		// one instruction and nothing passes through registers.  It walks the rows in order: wait
-		// until row r has landed (vmcnt), let every lane pull its unit out of LDS, unpack,
-		// multiply-accumulate against the activations held in registers, reduce across the
-		// wavefront, then request row r + PD.  All wavefronts advance at the same pace, so rows
-		// arrive in the order they are consumed and only the last row's arithmetic is exposed after
-		// the last byte has arrived.
-		// LDS (dynamic): [staged activations][nwaves x RB row slots of kSliceBytes][slice partials].
-		// ------------------------------------------------------------------
 		template <typename U>
 		__device__ __forceinline__ typename U::Raw unit_lds_load(uint32_t p, int u)
 		{
@@ -731,9 +546,89 @@ namespace litenn_hip
 			}
 		}
 
-		// Row R has landed once only the loads of the rows issued after it are outstanding.  Rows are
-		// issued PD ahead of the row being consumed, so that is min(PD - 1, RB - 1 - R) rows of
-		// `loads_per_row` instructions each (uniform over the wavefront).
+		constexpr int kMaxSlices = 8;       // K <= 32768
+		constexpr int kMaxRowsPerWave = 64; // rows a wavefront of the register kernel may own
+		constexpr int kLdsUnitStride = 68;  // floats between the staged activations of consecutive units
+		constexpr int kXPerThread = 8;      // most 128-bit activation loads a thread issues while staging
+		constexpr int kMaxStreamRows = 8;   // most rows a wavefront of the streaming kernel owns
+		constexpr int kPrefetchRows = 3;    // rows in flight ahead of the row being consumed
+		constexpr size_t kStreamLdsLimit = 160 * 1024;
+
+#ifdef LITENN_GEMV_TRACE
+		__device__ unsigned long long g_trace[4096 * 16];
+#define GEMV_TRACE(slot)                                                                                               \
+	if (lane == 0)                                                                                                     \
+	{                                                                                                                  \
+		g_trace[(blockIdx.x * 8 + wave) % 4096 * 16 + (slot)] = __builtin_readcyclecounter();                          \
+	}
+#else
+#define GEMV_TRACE(slot)
+#endif
+
+		// ------------------------------------------------------------------
+		// Streaming kernel: rows go HBM -> LDS with direct, fully coalesced 128-bit loads.
+		//
+		// Each wavefront owns RB consecutive rows of one 4096-wide slice and keeps kPrefetchRows of
+		// them in flight: consecutive lanes fetch consecutive 16-byte chunks, every cache line is
+		// consumed by one instruction and nothing passes through registers.  It walks the rows in
+		// order: wait until row r has landed (vmcnt), let every lane pull its unit out of LDS,
+		// unpack, multiply-accumulate against the activations held in registers, reduce across the
+		// wavefront, then request row r + kPrefetchRows.  All wavefronts advance at the same pace, so
+		// rows arrive in the order they are consumed and only the last row's arithmetic is exposed
+		// after the last byte has arrived.
+		//
+		// One launch can serve the operator groups of the decoder block that share an input:
+		//   * up to three matrices of one format over the same x (q/k/v projections): their rows
+		//     are simply concatenated;
+		//   * RMSNorm folded into the activation staging (x is normalised in f64 and scaled by the
+		//     norm weight while it moves to LDS; every workgroup recomputes the 4096-element sum,
+		//     which costs no HBM traffic and removes a kernel launch);
+		//   * SwiGLU: gate and up rows interleaved, the epilogue writes silu(gate) * up;
+		//   * a residual added to the output.
+		//
+		// LDS (dynamic): [staged activations][nwaves x RB row slots of kSliceBytes][slice partials]
+		// [norm partial sums].
+		// ------------------------------------------------------------------
+		struct GemvArgs
+		{
+			const uint8_t* w[3];
+			float* y[3];
+			int n[3];              // rows of each matrix, 0 when unused
+			const float* x;
+			const float* residual; // added to y[0]; single-matrix launches only
+			const float* norm_w;   // non-null: x is RMS-normalised and scaled by norm_w while staged
+			double eps;
+			int n_total;           // rows walked: n0 + n1 + n2, or 2 * n0 when interleaved
+			int k;
+			uint32_t row_bytes;
+			int slices, groups;
+			int silu_mul;          // 1: w[0] = gate, w[1] = up, row 2i + m; y[0][i] = silu(gate_i) * up_i
+		};
+
+		__device__ __forceinline__ void locate_row(const GemvArgs& a, int vr, int& m, int& local)
+		{
+			if (a.silu_mul)
+			{
+				m = vr & 1;
+				local = vr >> 1;
+				return;
+			}
+			m = 0;
+			local = vr;
+			if (local >= a.n[0])
+			{
+				local -= a.n[0];
+				m = 1;
+				if (local >= a.n[1])
+				{
+					local -= a.n[1];
+					m = 2;
+				}
+			}
+		}
+
+		// Row R has landed once only the loads of the rows issued after it are outstanding: that
+		// is min(PD - 1, RB - 1 - R) rows of `loads_per_row` instructions (uniform over the wavefront).
 		template <int RB, int PD, int R>
 		__device__ __forceinline__ void wait_row_landed(int loads_per_row)
 		{
@@ -770,35 +665,53 @@ namespace litenn_hip
 			static __device__ __forceinline__ void run(int, I&&, F&&) {}
 		};
 
-#ifdef LITENN_GEMV_TRACE
-		__device__ unsigned long long g_trace[4096 * 16];
-#define GEMV_TRACE(slot)                                                                                               \
-	if (lane == 0)                                                                                                     \
-	{                                                                                                                  \
-		g_trace[(blockIdx.x * 8 + wave) % 4096 * 16 + (slot)] = __builtin_readcyclecounter();                          \
-	}
-#else
-#define GEMV_TRACE(slot)
-#endif
-
-		constexpr int kMaxStreamRows = 8;
-		constexpr size_t kStreamLdsLimit = 160 * 1024;
-
-		template <typename U, int RB, int PD, int XP>
-		__global__ __launch_bounds__(512) void gemv_stream_kernel(const uint8_t* __restrict__ w,
-		                                                           const float* __restrict__ x,
-		                                                           float* __restrict__ y,
-		                                                           const float* __restrict__ residual, int n, int k,
-		                                                           uint32_t row_bytes, int slices, int groups)
+		template <int Ctrl, int RowMask>
+		__device__ __forceinline__ double dpp_f64(double x)
 		{
+			const unsigned long long b = __builtin_bit_cast(unsigned long long, x);
+			const unsigned lo = static_cast<unsigned>(
+			    __builtin_amdgcn_update_dpp(0, static_cast<int>(b), Ctrl, RowMask, 0xF, false));
+			const unsigned hi = static_cast<unsigned>(
+			    __builtin_amdgcn_update_dpp(0, static_cast<int>(b >> 32), Ctrl, RowMask, 0xF, false));
+			return __builtin_bit_cast(double, (static_cast<unsigned long long>(hi) << 32) | lo);
+		}
+
+		// f64 sum over the wavefront with DPP on the two halves; the total is returned in every lane
+		__device__ __forceinline__ double wave_sum_f64(double v)
+		{
+			v += dpp_f64<0xB1, 0xF>(v);
+			v += dpp_f64<0x4E, 0xF>(v);
+			v += dpp_f64<0x141, 0xF>(v);
+			v += dpp_f64<0x140, 0xF>(v);
+			v += dpp_f64<0x142, 0xA>(v);
+			v += dpp_f64<0x143, 0xC>(v);
+			const unsigned long long b = __builtin_bit_cast(unsigned long long, v);
+			const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(b), 63));
+			const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(b >> 32), 63));
+			return __builtin_bit_cast(double, (static_cast<unsigned long long>(hi) << 32) | lo);
+		}
+
+		// silu(g) * u with the separately rounded steps of the reference chain
+		// (Activation.h:22-35,56-63; SwiGLU.h:63-66)
+		__device__ __forceinline__ float silu_mul_value(float g, float u)
+		{
+			const float sig = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf(-g)));
+			return __fmul_rn(__fmul_rn(g, sig), u);
+		}
+
+		template <typename U, int RB, int XP>
+		__global__ __launch_bounds__(512) void gemv_stream_kernel(const GemvArgs a)
+		{
+			constexpr int PD = kPrefetchRows;
 			constexpr int kLoadsPerRowMax = (U::kSliceBytes + 1023) / 1024;
-			static_assert(kLoadsPerRowMax <= 5 && (PD - 1) * kLoadsPerRowMax <= 63 &&
-			                  PD * kLoadsPerRowMax <= 63,
-			              "vmcnt range");
+			static_assert(kLoadsPerRowMax <= 5 && PD * kLoadsPerRowMax <= 63, "vmcnt range");
 			extern __shared__ __attribute__((aligned(16))) uint8_t smem_b[];
 			const uint32_t lds0 = lds_address(smem_b);
 			const int lane = threadIdx.x & 63;
+			// the wavefront index is uniform: keeping it in a scalar register makes every row
+			// address, bound and branch below scalar work
 			const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+			const int slices = a.slices, groups = a.groups, k = a.k;
 			const int s = wave % slices;
 			const int g = wave / slices;
 			const int unit = s * 64 + lane;
@@ -808,29 +721,44 @@ namespace litenn_hip
 			const uint32_t x_bytes = static_cast<uint32_t>(units_per_row) * kLdsUnitStride * 4u;
 			const uint32_t rows_base = x_bytes + static_cast<uint32_t>(wave) * (RB * U::kSliceBytes);
 			const uint32_t part_base = x_bytes + static_cast<uint32_t>(nwaves) * (RB * U::kSliceBytes);
+			const uint32_t norm_base = part_base + static_cast<uint32_t>(nwaves) * RB * 4u;
 			const int row0 = (blockIdx.x * groups + g) * RB;
-			const int count = max(0, min(RB, n - row0));
+			const int count = max(0, min(RB, a.n_total - row0));
 			const uint32_t slice_off = static_cast<uint32_t>(s) * U::kSliceBytes;
-			const uint32_t slice_len = min(static_cast<uint32_t>(U::kSliceBytes), row_bytes - slice_off);
+			const uint32_t slice_len = min(static_cast<uint32_t>(U::kSliceBytes), a.row_bytes - slice_off);
 			const int loads_per_row = static_cast<int>((slice_len + 1023u) >> 10);
+			const bool fuse_norm = a.norm_w != nullptr;
 
 			GEMV_TRACE(0);
-			// 1. activations first: the oldest loads in flight.  XP 128-bit loads per thread, clamped
-			// so that every lane issues every one of them.
-			f32x4 xv[XP];
+			// 1. activations (and norm weights) first: the oldest loads in flight.  XP 128-bit loads
+			// per thread, clamped so that every lane issues every one of them.  They are issued
+			// outside the compiler's view: it may only order them against the direct-to-LDS loads
+			// below by waiting for everything.
+			f32x4 xv[XP], nw[XP];
 #pragma unroll
 			for (int j = 0; j < XP; ++j)
 			{
 				const int i = min(static_cast<int>(threadIdx.x + j * blockDim.x) * 4, k - 4);
-				xv[j] = asm_global_load128(x, static_cast<uint32_t>(i) * 4u);
+				xv[j] = asm_global_load128(a.x, static_cast<uint32_t>(i) * 4u);
+			}
+			if (fuse_norm)
+			{
+#pragma unroll
+				for (int j = 0; j < XP; ++j)
+				{
+					const int i = min(static_cast<int>(threadIdx.x + j * blockDim.x) * 4, k - 4);
+					nw[j] = asm_global_load128(a.norm_w, static_cast<uint32_t>(i) * 4u);
+				}
 			}
 
-			// 2. the first PD rows of the wavefront, straight into their LDS slots.  Rows past the end
-			// of the matrix re-read the last row so that the number of loads in flight is the same
-			// for every wavefront (the waits count them).
+			// 2. the first rows of the wavefront, straight into their LDS slots.  Rows past the end
+			// re-read the last row so that the number of loads in flight is the same for every
+			// wavefront (the waits count them).
 			auto issue_row = [&](int r) {
-				const int rr = min(row0 + r, n - 1);
-				const uint8_t* grow = w + static_cast<size_t>(rr) * row_bytes + slice_off;
+				int m, local;
+				locate_row(a, min(row0 + r, a.n_total - 1), m, local);
+				const uint8_t* wm = m == 0 ? a.w[0] : (m == 1 ? a.w[1] : a.w[2]);
+				const uint8_t* grow = wm + static_cast<size_t>(local) * a.row_bytes + slice_off;
 				uint8_t* slot = smem_b + rows_base + r * U::kSliceBytes;
 #pragma unroll
 				for (int i = 0; i < kLoadsPerRowMax; ++i)
@@ -846,18 +774,15 @@ namespace litenn_hip
 					}
 				}
 			};
-			constexpr int kFirstRows = RB < PD ? RB : PD; // rows in flight before the loop starts
+			constexpr int kFirstRows = RB < PD ? RB : PD;
 #pragma unroll
 			for (int r = 0; r < kFirstRows; ++r)
 			{
 				issue_row(r);
 			}
 
-			// 3. activations into LDS as soon as THEY have arrived (the row loads issued after them
-			// stay in flight): each float4 lands in the slot of the unit that consumes it, units
-			// kLdsUnitStride floats apart to keep the 128-bit reads below conflict-free
-			// (the kFirstRows rows issued after the activations may stay in flight; the activation
-			// registers are only ever read by the LDS writes below, after this wait)
+			// 3. activations into LDS as soon as THEY have arrived (the rows issued after them stay
+			// in flight; the activation registers are only read after this wait)
 			switch (loads_per_row)
 			{
 			case 1: vm_wait<kFirstRows * 1>(); break;
@@ -866,6 +791,46 @@ namespace litenn_hip
 			case 4: vm_wait<kFirstRows * 4>(); break;
 			default: vm_wait<kFirstRows * 5>(); break;
 			}
+			if (fuse_norm)
+			{
+				// RMSNorm with f64 accumulation (ComputePrimitives.h:792-817): every workgroup sums
+				// the whole vector, so no other kernel or pass over x is needed
+				double ss = 0.0;
+#pragma unroll
+				for (int j = 0; j < XP; ++j)
+				{
+					if (static_cast<int>(threadIdx.x + j * blockDim.x) * 4 < k)
+					{
+						const double x0 = xv[j].x, x1 = xv[j].y, x2 = xv[j].z, x3 = xv[j].w;
+						ss += x0 * x0;
+						ss += x1 * x1;
+						ss += x2 * x2;
+						ss += x3 * x3;
+					}
+				}
+				ss = wave_sum_f64(ss);
+				if (lane == 0)
+				{
+					lds_wr64(lds0 + norm_base + static_cast<uint32_t>(wave) * 8u, ss);
+				}
+				lds_barrier();
+				double total = 0.0;
+				for (int wv = 0; wv < nwaves; ++wv)
+				{
+					total += lds_rd_f64(lds0 + norm_base + static_cast<uint32_t>(wv) * 8u);
+				}
+				const double inv = 1.0 / sqrt(total / static_cast<double>(k) + a.eps);
+#pragma unroll
+				for (int j = 0; j < XP; ++j)
+				{
+					xv[j].x = static_cast<float>(static_cast<double>(xv[j].x) * inv * static_cast<double>(nw[j].x));
+					xv[j].y = static_cast<float>(static_cast<double>(xv[j].y) * inv * static_cast<double>(nw[j].y));
+					xv[j].z = static_cast<float>(static_cast<double>(xv[j].z) * inv * static_cast<double>(nw[j].z));
+					xv[j].w = static_cast<float>(static_cast<double>(xv[j].w) * inv * static_cast<double>(nw[j].w));
+				}
+			}
+			// each float4 lands in the slot of the unit that consumes it, units kLdsUnitStride floats
+			// apart so that the per-lane 128-bit reads below fall on distinct banks
 #pragma unroll
 			for (int j = 0; j < XP; ++j)
 			{
@@ -939,6 +904,123 @@ namespace litenn_hip
 			});
 			GEMV_TRACE(15);
 
+			// 6. slices of one row meet in LDS; afterwards thread t of the workgroup holds row
+			// block_row0 + t in `res`
+			int vr = row0 + lane;
+			bool have = lane < count;
+			if (slices > 1)
+			{
+				if (lane < RB)
+				{
+					lds_wr32(lds0 + part_base + static_cast<uint32_t>((s * groups + g) * RB + lane) * 4u, res);
+				}
+				lds_barrier();
+				const int t = threadIdx.x;
+				vr = blockIdx.x * groups * RB + t;
+				have = t < groups * RB && vr < a.n_total;
+				res = 0.0f;
+				if (have)
+				{
+					const int gg = t / RB, rl = t % RB;
+					for (int ss = 0; ss < slices; ++ss)
+					{
+						float v = __uint_as_float(
+						    lds_rd32<0>(lds0 + part_base + static_cast<uint32_t>((ss * groups + gg) * RB + rl) * 4u));
+						lds_wait(v);
+						res += v;
+					}
+				}
+			}
+			if (a.silu_mul)
+			{
+				// even lanes hold gate_i, their odd neighbours up_i (row 2i + m); RB and every block
+				// origin are even, so pairs never straddle wavefronts
+				const float other = dpp_f32<0xB1>(res); // quad_perm [1,0,3,2]
+				if (have && (vr & 1) == 0)
+				{
+					a.y[0][vr >> 1] = silu_mul_value(res, other);
+				}
+				return;
+			}
+			if (have)
+			{
+				int m, local;
+				locate_row(a, vr, m, local);
+				float* ym = m == 0 ? a.y[0] : (m == 1 ? a.y[1] : a.y[2]);
+				if (m == 0 && a.residual)
+				{
+					res += a.residual[local];
+				}
+				ym[local] = res;
+			}
+		}
+
+		// ------------------------------------------------------------------
+		// Register kernel: the same decomposition with the rows loaded straight into registers.
+		// Used for shapes the streaming kernel does not take (rows that are not a multiple of 16
+		// bytes, K beyond what fits in LDS).  One row is prefetched while the previous one is
+		// consumed.
+		// ------------------------------------------------------------------
+		template <typename U>
+		__global__ __launch_bounds__(512) void gemv_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+		                                                    float* __restrict__ y,
+		                                                    const float* __restrict__ residual, int n, int k,
+		                                                    size_t row_bytes, int slices, int groups,
+		                                                    int rows_per_wave)
+		{
+			extern __shared__ __attribute__((aligned(16))) float part[]; // [slices][groups * rows_per_wave]
+			const int lane = threadIdx.x & 63;
+			const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+			const int s = wave % slices;
+			const int g = wave / slices;
+			const int unit = s * 64 + lane;
+			const int units_per_row = k >> 6;
+			const bool active = unit < units_per_row;
+			const int row0 = (blockIdx.x * groups + g) * rows_per_wave;
+			const int row_end = min(row0 + rows_per_wave, n);
+
+			typename U::Raw cur, nxt;
+			if (active && row0 < row_end)
+			{
+				cur = U::load(w + static_cast<size_t>(row0) * row_bytes, unit);
+			}
+			float xr[64];
+			if (active)
+			{
+#pragma unroll
+				for (int i = 0; i < 64; i += 4)
+				{
+					const float4 v = *reinterpret_cast<const float4*>(x + U::x_offset(unit, i));
+					xr[i] = v.x;
+					xr[i + 1] = v.y;
+					xr[i + 2] = v.z;
+					xr[i + 3] = v.w;
+				}
+			}
+			else
+			{
+#pragma unroll
+				for (int i = 0; i < 64; ++i)
+				{
+					xr[i] = 0.0f;
+				}
+			}
+			const typename U::Prep pz = U::prep(xr);
+
+			float res = 0.0f; // lane i keeps the total of row row0 + i
+			for (int r = row0; r < row_end; ++r)
+			{
+				if (active && r + 1 < row_end)
+				{
+					nxt = U::load(w + static_cast<size_t>(r + 1) * row_bytes, unit);
+				}
+				const float p = active ? unit_dot<U>(cur, xr, pz, unit) : 0.0f;
+				const float total = wave_sum(p);
+				res = (lane == r - row0) ? total : res;
+				cur = nxt;
+			}
+
+			const int count = row_end - row0;
 			if (slices == 1)
 			{
 				if (lane < count)
@@ -947,26 +1029,22 @@ namespace litenn_hip
 				}
 				return;
 			}
-			// slices of one row meet in LDS
-			if (lane < RB)
+			if (lane < count)
 			{
-				lds_wr32(lds0 + part_base + static_cast<uint32_t>((s * groups + g) * RB + lane) * 4u, res);
+				part[s * (groups * rows_per_wave) + g * rows_per_wave + lane] = res;
 			}
-			lds_barrier();
-			const int t = threadIdx.x;
-			if (t < groups * RB)
+			__syncthreads();
+			const int per_block = groups * rows_per_wave;
+			for (int t = threadIdx.x; t < per_block; t += blockDim.x)
 			{
-				const int gg = t / RB, rl = t % RB;
-				const int rr = (blockIdx.x * groups + gg) * RB + rl;
+				const int gg = t / rows_per_wave;
+				const int rr = (blockIdx.x * groups + gg) * rows_per_wave + (t % rows_per_wave);
 				if (rr < n)
 				{
-					float total = 0.0f;
-					for (int ss = 0; ss < slices; ++ss)
+					float total = part[t];
+					for (int ss = 1; ss < slices; ++ss)
 					{
-						float v = __uint_as_float(
-						    lds_rd32<0>(lds0 + part_base + static_cast<uint32_t>((ss * groups + gg) * RB + rl) * 4u));
-						lds_wait(v);
-						total += v;
+						total += part[ss * per_block + t];
 					}
 					y[rr] = residual ? residual[rr] + total : total;
 				}
@@ -1112,195 +1190,252 @@ namespace litenn_hip
 			return (v && *v) ? atoi(v) : fallback;
 		}
 
-		template <typename U, int RU>
-		void launch_fast_ru(const uint8_t* w, const float* x, float* y, const float* residual, int n, int k, size_t rb,
-		                    hipStream_t stream)
+		int compute_units()
 		{
-			const int slices = (k + 4095) / 4096;
-			// LITENN_HIP_GEMV_WAVES: wavefronts the launch is spread over (default: 8 per CU on 256 CUs)
-			static const int target_waves = env_int("LITENN_HIP_GEMV_WAVES", 2048);
-			int groups = 8 / slices;
-			if (groups < 1)
-			{
-				groups = 1;
-			}
-			int rows_per_wave = (n * slices + target_waves - 1) / target_waves;
-			rows_per_wave = rows_per_wave < 1 ? 1 : (rows_per_wave > kMaxRowsPerWave ? kMaxRowsPerWave : rows_per_wave);
-			const int rows_per_block = groups * rows_per_wave;
-			const int blocks = (n + rows_per_block - 1) / rows_per_block;
-			const size_t part_bytes = slices > 1 ? sizeof(float) * slices * rows_per_block : 0;
-			static const int lds_x = env_int("LITENN_HIP_GEMV_LDS_X", 1);
-			const size_t x_bytes = sizeof(float) * (static_cast<size_t>(k) / 64) * kLdsUnitStride;
-			const int x_in_lds = (lds_x && x_bytes + part_bytes <= kMaxLdsBytes &&
-			                      k <= 64 * slices * groups * 4 * kXPerThread)
-			                         ? 1
-			                         : 0;
-			const size_t lds = part_bytes + (x_in_lds ? x_bytes : 0);
-			static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<U, RU>),
-			                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
-			                                                   static_cast<int>(kMaxLdsBytes));
-			(void)attr;
-			gemv_kernel<U, RU><<<dim3(blocks), dim3(64 * slices * groups), lds, stream>>>(
-			    w, x, y, residual, n, k, rb, slices, groups, rows_per_wave, x_in_lds);
+			static const int cus = [] {
+				int dev = 0;
+				hipDeviceProp_t prop;
+				if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+				{
+					return 256;
+				}
+				return prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+			}();
+			return cus;
 		}
 
-		template <typename U, int RB, int PD, int XP>
-		void launch_stream_rb_pd_xp(const uint8_t* w, const float* x, float* y, const float* residual, int n, int k,
-		                            size_t rb, int slices, int groups, size_t lds, hipStream_t stream)
+		template <typename U, int RB, int XP>
+		void launch_stream_variant(const GemvArgs& a, size_t lds, hipStream_t stream)
 		{
 			static const hipError_t attr =
-			    hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_stream_kernel<U, RB, PD, XP>),
+			    hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_stream_kernel<U, RB, XP>),
 			                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kStreamLdsLimit));
 			(void)attr;
-			const int rows_per_block = groups * RB;
-			const int blocks = (n + rows_per_block - 1) / rows_per_block;
-			gemv_stream_kernel<U, RB, PD, XP><<<dim3(blocks), dim3(64 * slices * groups), lds, stream>>>(
-			    w, x, y, residual, n, k, static_cast<uint32_t>(rb), slices, groups);
-		}
-
-		template <typename U, int RB, int PD>
-		void launch_stream_rb_pd(const uint8_t* w, const float* x, float* y, const float* residual, int n, int k,
-		                         size_t rb, int slices, int groups, size_t lds, hipStream_t stream)
-		{
-			// 128-bit activation loads per thread while staging x
-			const int per_thread = (k / 4 + 64 * slices * groups - 1) / (64 * slices * groups);
-			if (per_thread <= 2)
-			{
-				launch_stream_rb_pd_xp<U, RB, PD, 2>(w, x, y, residual, n, k, rb, slices, groups, lds, stream);
-			}
-			else if (per_thread <= 4)
-			{
-				launch_stream_rb_pd_xp<U, RB, PD, 4>(w, x, y, residual, n, k, rb, slices, groups, lds, stream);
-			}
-			else
-			{
-				launch_stream_rb_pd_xp<U, RB, PD, kXPerThread>(w, x, y, residual, n, k, rb, slices, groups, lds,
-				                                               stream);
-			}
+			const int rows_per_block = a.groups * RB;
+			const int blocks = (a.n_total + rows_per_block - 1) / rows_per_block;
+			gemv_stream_kernel<U, RB, XP><<<dim3(blocks), dim3(64 * a.slices * a.groups), lds, stream>>>(a);
 		}
 
 		template <typename U, int RB>
-		void launch_stream_rb(const uint8_t* w, const float* x, float* y, const float* residual, int n, int k,
-		                      size_t rb, int slices, int groups, size_t lds, hipStream_t stream)
+		void launch_stream_rows(const GemvArgs& a, size_t lds, hipStream_t stream)
 		{
-			// LITENN_HIP_GEMV_PREFETCH: rows kept in flight ahead of the row being consumed
-			static const int pd = env_int("LITENN_HIP_GEMV_PREFETCH", 3);
-			if (pd <= 2)
+			const int threads = 64 * a.slices * a.groups;
+			const int per_thread = (a.k / 4 + threads - 1) / threads; // 128-bit activation loads per thread
+			if (per_thread <= 2)
 			{
-				launch_stream_rb_pd<U, RB, 2>(w, x, y, residual, n, k, rb, slices, groups, lds, stream);
+				launch_stream_variant<U, RB, 2>(a, lds, stream);
+			}
+			else if (per_thread <= 4)
+			{
+				launch_stream_variant<U, RB, 4>(a, lds, stream);
 			}
 			else
 			{
-				launch_stream_rb_pd<U, RB, 3>(w, x, y, residual, n, k, rb, slices, groups, lds, stream);
+				launch_stream_variant<U, RB, kXPerThread>(a, lds, stream);
 			}
 		}
 
-		// Returns false when the shape does not fit the streaming kernel (the register kernel runs then).
+		// Returns false when the shape does not fit the streaming kernel.
 		template <typename U>
-		bool launch_stream(const uint8_t* w, const float* x, float* y, const float* residual, int n, int k, size_t rb,
-		                   hipStream_t stream)
+		bool launch_stream(GemvArgs a, hipStream_t stream)
 		{
-			const int slices = (k + 4095) / 4096;
-			if (slices > 8 || rb % 16 != 0 || reinterpret_cast<uintptr_t>(w) % 16 != 0 || rb > 0xffffffffull)
+			const int k = a.k;
+			a.slices = (k + 4095) / 4096;
+			if (a.slices > kMaxSlices || a.row_bytes % 16 != 0)
 			{
 				return false;
 			}
-			const int groups = 8 / slices;
-			if (k > 64 * slices * groups * 4 * kXPerThread)
+			for (int m = 0; m < 3; ++m)
+			{
+				if (a.n[m] > 0 && reinterpret_cast<uintptr_t>(a.w[m]) % 16 != 0)
+				{
+					return false;
+				}
+			}
+			if (reinterpret_cast<uintptr_t>(a.x) % 16 != 0 || (a.norm_w && reinterpret_cast<uintptr_t>(a.norm_w) % 16 != 0))
 			{
 				return false;
 			}
-			// rows per wavefront: spread the matrix over about `target_waves` wavefronts, within LDS
-			static const int target_waves = env_int("LITENN_HIP_GEMV_WAVES", 2048);
-			static const int forced_rb = env_int("LITENN_HIP_GEMV_ROWS", 0);
-			int want = forced_rb > 0 ? forced_rb : (n * slices + target_waves - 1) / target_waves;
-			want = want < 1 ? 1 : (want > kMaxStreamRows ? kMaxStreamRows : want);
+			a.groups = 8 / a.slices;
+			const int nwaves = a.slices * a.groups;
+			if (k > 64 * nwaves * 4 * kXPerThread)
+			{
+				return false;
+			}
+			// Rows per wavefront: the workgroups of one launch should fill the CUs once (a second,
+			// partial round costs a whole start-up), then as few rows as possible.
 			const size_t x_bytes = sizeof(float) * (static_cast<size_t>(k) / 64) * kLdsUnitStride;
 			auto lds_for = [&](int r) {
-				return x_bytes + static_cast<size_t>(slices * groups) * r * U::kSliceBytes +
-				       sizeof(float) * slices * groups * r;
+				return x_bytes + static_cast<size_t>(nwaves) * r * U::kSliceBytes + sizeof(float) * nwaves * r +
+				       sizeof(double) * nwaves;
 			};
-			while (want > 1 && lds_for(want) > kStreamLdsLimit)
+			static const int forced_rows = env_int("LITENN_HIP_GEMV_ROWS", 0);
+			const int cus = compute_units();
+			int best = 0;
+			double best_cost = 0.0;
+			for (int r = 1; r <= kMaxStreamRows; ++r)
 			{
-				--want;
+				if ((a.silu_mul && (r & 1)) || lds_for(r) > kStreamLdsLimit)
+				{
+					continue;
+				}
+				const int blocks = (a.n_total + a.groups * r - 1) / (a.groups * r);
+				const double rounds = static_cast<double>((blocks + cus - 1) / cus);
+				const double cost = rounds * (3.0 + 0.75 * r);
+				if (forced_rows == r || best == 0 || (forced_rows == 0 && cost < best_cost))
+				{
+					best = r;
+					best_cost = cost;
+					if (forced_rows == r)
+					{
+						break;
+					}
+				}
 			}
-			if (lds_for(want) > kStreamLdsLimit)
+			if (best == 0)
 			{
 				return false;
 			}
-			const size_t lds = lds_for(want);
-			switch (want)
+			const size_t lds = lds_for(best);
+			switch (best)
 			{
-			case 1: launch_stream_rb<U, 1>(w, x, y, residual, n, k, rb, slices, groups, lds, stream); break;
-			case 2: launch_stream_rb<U, 2>(w, x, y, residual, n, k, rb, slices, groups, lds, stream); break;
-			case 3: launch_stream_rb<U, 3>(w, x, y, residual, n, k, rb, slices, groups, lds, stream); break;
-			case 4: launch_stream_rb<U, 4>(w, x, y, residual, n, k, rb, slices, groups, lds, stream); break;
-			case 5: launch_stream_rb<U, 5>(w, x, y, residual, n, k, rb, slices, groups, lds, stream); break;
-			case 6: launch_stream_rb<U, 6>(w, x, y, residual, n, k, rb, slices, groups, lds, stream); break;
-			case 7: launch_stream_rb<U, 7>(w, x, y, residual, n, k, rb, slices, groups, lds, stream); break;
-			default: launch_stream_rb<U, 8>(w, x, y, residual, n, k, rb, slices, groups, lds, stream); break;
+			case 1: launch_stream_rows<U, 1>(a, lds, stream); break;
+			case 2: launch_stream_rows<U, 2>(a, lds, stream); break;
+			case 3: launch_stream_rows<U, 3>(a, lds, stream); break;
+			case 4: launch_stream_rows<U, 4>(a, lds, stream); break;
+			case 5: launch_stream_rows<U, 5>(a, lds, stream); break;
+			case 6: launch_stream_rows<U, 6>(a, lds, stream); break;
+			case 7: launch_stream_rows<U, 7>(a, lds, stream); break;
+			default: launch_stream_rows<U, 8>(a, lds, stream); break;
 			}
 			return true;
 		}
 
 		template <typename U>
-		void launch_fast(const uint8_t* w, const float* x, float* y, const float* residual, int n, int k, size_t rb,
-		                 hipStream_t stream)
+		void launch_register(const uint8_t* w, const float* x, float* y, const float* residual, int n, int k, size_t rb,
+		                     hipStream_t stream)
+		{
+			const int slices = (k + 4095) / 4096;
+			int groups = 8 / slices;
+			if (groups < 1)
+			{
+				groups = 1;
+			}
+			const int target_waves = 8 * compute_units();
+			int rows_per_wave = (n * slices + target_waves - 1) / target_waves;
+			rows_per_wave = rows_per_wave < 1 ? 1 : (rows_per_wave > kMaxRowsPerWave ? kMaxRowsPerWave : rows_per_wave);
+			const int rows_per_block = groups * rows_per_wave;
+			const int blocks = (n + rows_per_block - 1) / rows_per_block;
+			const size_t lds = slices > 1 ? sizeof(float) * slices * rows_per_block : 0;
+			gemv_kernel<U><<<dim3(blocks), dim3(64 * slices * groups), lds, stream>>>(w, x, y, residual, n, k, rb, slices,
+			                                                                         groups, rows_per_wave);
+		}
+
+		bool is_block_format(int fmt)
+		{
+			return fmt == LITENN_FMT_Q4_0 || fmt == LITENN_FMT_Q8_0 || fmt == LITENN_FMT_Q4_K || fmt == LITENN_FMT_Q6_K;
+		}
+
+		bool stream_dispatch(int fmt, const GemvArgs& a, hipStream_t stream)
 		{
 			// LITENN_HIP_GEMV_STREAM=0 keeps the rows in registers instead of LDS
 			static const int use_stream = env_int("LITENN_HIP_GEMV_STREAM", 1);
-			if (use_stream && launch_stream<U>(w, x, y, residual, n, k, rb, stream))
+			if (!use_stream || !is_block_format(fmt) || a.k % 256 != 0)
 			{
-				return;
+				return false;
 			}
-			static const int ru = env_int("LITENN_HIP_GEMV_RU", 1);
-			if (ru >= 4)
+			switch (fmt)
 			{
-				launch_fast_ru<U, 4>(w, x, y, residual, n, k, rb, stream);
-			}
-			else if (ru == 1)
-			{
-				launch_fast_ru<U, 1>(w, x, y, residual, n, k, rb, stream);
-			}
-			else
-			{
-				launch_fast_ru<U, 2>(w, x, y, residual, n, k, rb, stream);
+			case LITENN_FMT_Q4_0: return launch_stream<Q4_0Unit>(a, stream);
+			case LITENN_FMT_Q8_0: return launch_stream<Q8_0Unit>(a, stream);
+			case LITENN_FMT_Q4_K: return launch_stream<Q4_KUnit>(a, stream);
+			default: return launch_stream<Q6_KUnit>(a, stream);
 			}
 		}
 	} // namespace
 
-	// Launches y[m, n] = x[m, k] . W^T one activation row at a time through the GEMV.
+	// One fused launch over up to three same-format matrices that share x (see GemvArgs).  Returns
+	// false, launching nothing, when the streaming kernel does not take the shape; the caller then
+	// composes the operators from separate launches.
+	bool launch_gemv_fused(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
+	                       const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
+	                       hipStream_t stream)
+	{
+		if (count < 1 || count > 3 || k > 0x7fffffffu || (silu_mul && (count != 2 || n[0] != n[1])) ||
+		    (residual && count != 1))
+		{
+			return false;
+		}
+		GemvArgs a{};
+		size_t total = 0;
+		for (int m = 0; m < count; ++m)
+		{
+			if (n[m] == 0 || n[m] > 0x3fffffffu)
+			{
+				return false;
+			}
+			a.w[m] = static_cast<const uint8_t*>(w[m]);
+			a.y[m] = y[m];
+			a.n[m] = static_cast<int>(n[m]);
+			total += n[m];
+		}
+		if (total > 0x7fffffffu)
+		{
+			return false;
+		}
+		const size_t rb = row_bytes(fmt, k);
+		if (rb == 0 || rb > 0xffffffffull)
+		{
+			return false;
+		}
+		a.x = x;
+		a.residual = residual;
+		a.norm_w = norm_w;
+		a.eps = eps;
+		a.n_total = static_cast<int>(total);
+		a.k = static_cast<int>(k);
+		a.row_bytes = static_cast<uint32_t>(rb);
+		a.silu_mul = silu_mul ? 1 : 0;
+		return stream_dispatch(fmt, a, stream);
+	}
+
+	// y[m, n] = x[m, k] . W^T (+ residual), one activation row at a time.
 	int launch_gemv(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
 	                const float* residual, hipStream_t stream)
 	{
 		const size_t rb = row_bytes(fmt, k);
 		const uint8_t* w = static_cast<const uint8_t*>(wq);
-		const bool quant = fmt == LITENN_FMT_Q4_0 || fmt == LITENN_FMT_Q8_0 || fmt == LITENN_FMT_Q4_K ||
-		                   fmt == LITENN_FMT_Q6_K;
-		// fast path: whole 64-weight units, 16-byte aligned activations, K within the slice budget
-		const bool fast = quant && (k % 256 == 0) && k <= static_cast<size_t>(kMaxSlices) * 4096 &&
-		                  (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(w) % 4 == 0) &&
-		                  env_int("LITENN_HIP_GEMV_GENERIC", 0) == 0;
+		// register kernel: whole 64-weight units, 16-byte aligned activations, K within the slice budget
+		const bool regs_ok = is_block_format(fmt) && (k % 256 == 0) && k <= static_cast<size_t>(kMaxSlices) * 4096 &&
+		                     (reinterpret_cast<uintptr_t>(w) % 4 == 0) && env_int("LITENN_HIP_GEMV_GENERIC", 0) == 0;
 		for (size_t i = 0; i < m; ++i)
 		{
 			const float* xi = x + i * k;
 			float* yi = y + i * n;
 			const float* ri = residual ? residual + i * n : nullptr;
-			if (fast && (reinterpret_cast<uintptr_t>(xi) % 16 == 0))
+			const void* ws[1] = { wq };
+			float* ys[1] = { yi };
+			const size_t ns[1] = { n };
+			if (env_int("LITENN_HIP_GEMV_GENERIC", 0) == 0 &&
+			    launch_gemv_fused(fmt, 1, ws, ys, ns, k, xi, ri, nullptr, 0.0, false, stream))
+			{
+				continue;
+			}
+			if (regs_ok && (reinterpret_cast<uintptr_t>(xi) % 16 == 0))
 			{
 				switch (fmt)
 				{
 				case LITENN_FMT_Q4_0:
-					launch_fast<Q4_0Unit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
+					launch_register<Q4_0Unit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
 					break;
 				case LITENN_FMT_Q8_0:
-					launch_fast<Q8_0Unit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
+					launch_register<Q8_0Unit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
 					break;
 				case LITENN_FMT_Q4_K:
-					launch_fast<Q4_KUnit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
+					launch_register<Q4_KUnit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
 					break;
 				default:
-					launch_fast<Q6_KUnit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
+					launch_register<Q6_KUnit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
 					break;
 				}
 			}
@@ -1312,6 +1447,41 @@ namespace litenn_hip
 			}
 		}
 		return 0;
+	}
+
+	void launch_rmsnorm(const float* x, const float* w, double eps, size_t m, size_t d, float* y, hipStream_t s);
+	void launch_silu_mul(const float* gate, const float* up, float* y, size_t n, hipStream_t s);
+
+	// RMSNorm (optional) -> up to three same-format linears over one activation row -> SwiGLU or
+	// residual (optional): one fused launch when the streaming kernel takes the shape, otherwise the
+	// same operators from separate launches.  scratch_x holds k floats (used when norm_w is given and
+	// the fused kernel is not applicable); scratch_gate / scratch_up hold n[0] floats (same, SwiGLU).
+	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
+	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
+	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream)
+	{
+		static const int fuse = env_int("LITENN_HIP_FUSE", 1);
+		if (fuse && launch_gemv_fused(fmt, count, w, y, n, k, x, residual, norm_w, eps, silu_mul, stream))
+		{
+			return;
+		}
+		const float* xin = x;
+		if (norm_w)
+		{
+			launch_rmsnorm(x, norm_w, eps, 1, k, scratch_x, stream);
+			xin = scratch_x;
+		}
+		if (silu_mul)
+		{
+			launch_gemv(fmt, w[0], n[0], k, xin, 1, scratch_gate, nullptr, stream);
+			launch_gemv(fmt, w[1], n[1], k, xin, 1, scratch_up, nullptr, stream);
+			launch_silu_mul(scratch_gate, scratch_up, y[0], n[0], stream);
+			return;
+		}
+		for (int m = 0; m < count; ++m)
+		{
+			launch_gemv(fmt, w[m], n[m], k, xin, 1, y[m], m == 0 ? residual : nullptr, stream);
+		}
 	}
 
 	void launch_dequantize(int fmt, const void* wq, size_t rows, size_t k, float* dst, hipStream_t stream)

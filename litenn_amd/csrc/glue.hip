@@ -10,11 +10,11 @@ namespace litenn_hip
 	namespace
 	{
 		// ---------------- RMSNorm (f64 accumulate, ComputePrimitives.h:792-817) -------------
-		__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x,
-		                                                       const float* __restrict__ w, double eps, int d,
-		                                                       float* __restrict__ y)
+		__global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__ x,
+		                                                        const float* __restrict__ w, double eps, int d,
+		                                                        float* __restrict__ y)
 		{
-			__shared__ double red[4];
+			__shared__ double red[16];
 			const float* xr = x + static_cast<size_t>(blockIdx.x) * d;
 			float* yr = y + static_cast<size_t>(blockIdx.x) * d;
 			double acc = 0.0;
@@ -37,10 +37,12 @@ namespace litenn_hip
 			{
 				total += red[i];
 			}
-			const double denom = sqrt(total / static_cast<double>(d) + eps);
+			// x / denom as a multiplication by the f64 reciprocal: one f64 ulp from the quotient,
+			// invisible after the final rounding to f32
+			const double inv = 1.0 / sqrt(total / static_cast<double>(d) + eps);
 			for (int i = threadIdx.x; i < d; i += blockDim.x)
 			{
-				double v = static_cast<double>(xr[i]) / denom;
+				double v = static_cast<double>(xr[i]) * inv;
 				if (w)
 				{
 					v *= static_cast<double>(w[i]);
@@ -374,7 +376,7 @@ namespace litenn_hip
 	// ---- launchers used by the C ABI and by the decoder runtime ---------------------------
 	void launch_rmsnorm(const float* x, const float* w, double eps, size_t m, size_t d, float* y, hipStream_t s)
 	{
-		rmsnorm_kernel<<<dim3(m), dim3(256), 0, s>>>(x, w, eps, static_cast<int>(d), y);
+		rmsnorm_kernel<<<dim3(m), dim3(d >= 4096 ? 1024 : 256), 0, s>>>(x, w, eps, static_cast<int>(d), y);
 	}
 
 	void launch_rope_table(float* cos_t, float* sin_t, size_t positions, size_t half, double base, double freq_scale,

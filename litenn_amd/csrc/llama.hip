@@ -20,6 +20,9 @@ namespace litenn_hip
 	                const float* residual, hipStream_t stream);
 	int launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
 	                const float* residual, hipStream_t stream);
+	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
+	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
+	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream);
 	void launch_get_rows_q(int fmt, const void* table, size_t rows, size_t k, const int32_t* ids, size_t n_ids,
 	                       float* out, int* err_flag, hipStream_t stream);
 	void launch_rmsnorm(const float* x, const float* w, double eps, size_t m, size_t d, float* y, hipStream_t s);
@@ -86,7 +89,7 @@ struct litenn_hip_llama
 	// activations for `cap_rows` rows
 	size_t cap_rows = 0, cap_logit_rows = 0;
 	float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *gate = nullptr,
-	      *up = nullptr, *logits = nullptr;
+	      *gate2 = nullptr, *up = nullptr, *logits = nullptr;
 	int32_t* d_tokens = nullptr;
 	int32_t* d_next = nullptr; // token produced by the last arg-max
 	int32_t* d_out = nullptr;  // generated tokens
@@ -104,7 +107,7 @@ namespace
 
 	void free_scratch(litenn_hip_llama* m)
 	{
-		float** bufs[] = { &m->x, &m->xn, &m->q, &m->k, &m->v, &m->attn, &m->gate, &m->up };
+		float** bufs[] = { &m->x, &m->xn, &m->q, &m->k, &m->v, &m->attn, &m->gate, &m->gate2, &m->up };
 		for (float** b : bufs)
 		{
 			if (*b)
@@ -146,7 +149,8 @@ namespace
 			drop_graph(m); // the captured step references the old buffers
 			free_scratch(m);
 			struct { float** p; size_t n; } bufs[] = { { &m->x, d }, { &m->xn, d }, { &m->q, qw }, { &m->k, kvw },
-				                                        { &m->v, kvw }, { &m->attn, qw }, { &m->gate, ff }, { &m->up, ff } };
+				                                        { &m->v, kvw }, { &m->attn, qw }, { &m->gate, ff }, { &m->gate2, ff },
+				                                        { &m->up, ff } };
 			for (auto& b : bufs)
 			{
 				LITENN_HIP_TRY(kAction, hipMalloc(reinterpret_cast<void**>(b.p), sizeof(float) * rows * b.n));
@@ -200,10 +204,89 @@ namespace
 		}
 	}
 
+	// One operator group of the single-token step (see launch_linear_group).
+	void group(litenn_hip_llama* m, int count, const Weight* const* ws, float* const* ys, const float* x,
+	           const float* residual, const float* norm_w, bool silu_mul, hipStream_t s)
+	{
+		const void* w[3] = { nullptr, nullptr, nullptr };
+		size_t n[3] = { 0, 0, 0 };
+		for (int i = 0; i < count; ++i)
+		{
+			w[i] = ws[i]->data;
+			n[i] = ws[i]->n;
+		}
+		// scratch used only when the fused kernel does not take the shape: xn for the normalised
+		// activations, gate2 / up for the separate gate and up projections
+		launch_linear_group(ws[0]->fmt, count, w, ys, n, ws[0]->k, x, residual, norm_w, m->p.rms_norm_epsilon, silu_mul,
+		                    m->xn, m->gate2, m->up, s);
+	}
+
+	// The single-token step: six fused launches per decoder block
+	//   [RMSNorm + q/k/v] [RoPE + cache append] [attention] [o + residual] [RMSNorm + gate/up + SwiGLU]
+	//   [down + residual]
+	// (matrices of different formats cannot share a launch and go out one by one).
+	void forward_token(litenn_hip_llama* m, const int32_t* ids)
+	{
+		hipStream_t s = m->stream;
+		const size_t d = m->p.embedding_length;
+		const size_t H = m->p.head_count, KH = m->p.head_count_kv, hd = m->head_dim;
+		const int* past_dev = m->d_counters;
+		launch_get_rows_q(m->tok_embd.fmt, m->tok_embd.data, m->tok_embd.n, d, ids, 1, m->x, m->d_err, s);
+		for (Layer& L : m->layers)
+		{
+			const Weight* qkv[3] = { &L.wq, &L.wk, &L.wv };
+			float* qkv_out[3] = { m->q, m->k, m->v };
+			for (int i = 0; i < 3;)
+			{
+				int j = i + 1;
+				while (j < 3 && qkv[j]->fmt == qkv[i]->fmt)
+				{
+					++j;
+				}
+				group(m, j - i, qkv + i, qkv_out + i, m->x, nullptr, L.attn_norm, false, s);
+				i = j;
+			}
+			launch_rope_qkv_append(m->q, m->k, m->v, L.kcache, L.vcache, m->p.kv_dtype, past_dev, 1, H, KH, hd,
+			                       m->p.rope_dimension_count, m->cos_t, m->sin_t, s);
+			launch_attn_decode(m->q, L.kcache, L.vcache, m->p.kv_dtype, 1, past_dev, 0, m->p.context_length, H, KH, hd,
+			                   m->attn, s);
+			const Weight* wo[1] = { &L.wo };
+			float* xo[1] = { m->x };
+			group(m, 1, wo, xo, m->attn, m->x, nullptr, false, s); // x = x + attn . Wo
+			if (L.gate.fmt == L.up.fmt)
+			{
+				const Weight* gu[2] = { &L.gate, &L.up };
+				float* h[1] = { m->gate };
+				group(m, 2, gu, h, m->x, nullptr, L.ffn_norm, true, s); // gate = silu(x'.Wg) * (x'.Wu)
+			}
+			else
+			{
+				const Weight* wg[1] = { &L.gate };
+				const Weight* wu[1] = { &L.up };
+				float* og[1] = { m->gate };
+				float* ou[1] = { m->up };
+				group(m, 1, wg, og, m->x, nullptr, L.ffn_norm, false, s);
+				group(m, 1, wu, ou, m->x, nullptr, L.ffn_norm, false, s);
+				launch_silu_mul(m->gate, m->up, m->gate, m->p.feed_forward_length, s);
+			}
+			const Weight* wd[1] = { &L.down };
+			group(m, 1, wd, xo, m->gate, m->x, nullptr, false, s); // x = x + mlp
+		}
+		const Weight* head[1] = { m->output.data ? &m->output : &m->tok_embd };
+		float* lg[1] = { m->logits };
+		group(m, 1, head, lg, m->x, nullptr, m->output_norm, false, s);
+	}
+
 	// Enqueues the decoder over `rows` tokens whose ids are at `ids` (device); positions start at
 	// counters[0].  Logits are produced for the last `logit_rows` rows into m->logits.
 	void forward(litenn_hip_llama* m, const int32_t* ids, size_t rows, size_t logit_rows, unsigned flags)
 	{
+		static const bool fuse_token = !(getenv("LITENN_HIP_FUSE") && getenv("LITENN_HIP_FUSE")[0] == '0');
+		if (rows == 1 && logit_rows == 1 && fuse_token)
+		{
+			forward_token(m, ids);
+			return;
+		}
 		hipStream_t s = m->stream;
 		const size_t d = m->p.embedding_length;
 		const size_t H = m->p.head_count, KH = m->p.head_count_kv, hd = m->head_dim;

@@ -198,6 +198,26 @@ def mul_mat_q(fmt: int, wq: Tensor, n: int, k: int, x: Tensor, y: Tensor | None 
     return y
 
 
+GROUP_SILU_MUL = 1
+
+
+def linear_group(fmt: int, weights, ns, k: int, x: Tensor, residual: Tensor | None = None,
+                 norm_w: Tensor | None = None, eps: float = 1e-5, silu_mul: bool = False):
+    """[RMSNorm] -> 1..3 linears of one format over one activation row -> [residual | SwiGLU].
+
+    Returns the list of outputs (one per matrix; a single tensor list for SwiGLU)."""
+    count = len(weights)
+    outs = [Tensor((1, ns[0]), DT_F32, x.device)] if silu_mul else [Tensor((1, n), DT_F32, x.device) for n in ns]
+    wptrs = (C.c_void_p * count)(*[w.ptr for w in weights])
+    yptrs = (C.c_void_p * count)(*[(outs[i].ptr if i < len(outs) else None) for i in range(count)])
+    narr = (C.c_size_t * count)(*ns)
+    check(_lib.load().litenn_hip_linear_group(x.device.deviceIndex, fmt, count, wptrs, narr, k, x.ptr, yptrs,
+                                              residual.ptr if residual is not None else None,
+                                              norm_w.ptr if norm_w is not None else None, eps,
+                                              GROUP_SILU_MUL if silu_mul else 0, None))
+    return outs
+
+
 def dequantize(fmt: int, wq: Tensor, rows: int, k: int) -> Tensor:
     out = Tensor((rows, k), DT_F32, wq.device)
     check(_lib.load().litenn_hip_dequantize(wq.device.deviceIndex, fmt, wq.ptr, rows, k, out.ptr, None))
@@ -256,6 +276,7 @@ def argmax(x: Tensor) -> Tensor:
     return out
 
 
-__all__ = ["HIP", "HIPDeviceCount", "IsHIPDeviceAvailable", "DeviceTraits", "Tensor", "mul_mat_q", "dequantize",
+__all__ = ["HIP", "HIPDeviceCount", "IsHIPDeviceAvailable", "DeviceTraits", "Tensor", "mul_mat_q", "linear_group",
+           "dequantize",
            "get_rows_q", "rmsnorm", "rope_interleaved", "kv_append", "attn_decode", "silu_mul", "argmax",
            "MATMUL_PRECISE", "LiteNNHipError", "F32"]

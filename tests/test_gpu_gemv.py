@@ -122,3 +122,52 @@ def test_errors_and_empty_inputs(hip):
         hip.mul_mat_q(Q4_K, wq, 1, 128, x)
     empty = hip.mul_mat_q(Q4_K, hip.Tensor.from_numpy(np.zeros(0, np.uint8)), 0, 256, x)
     assert empty.shape == (1, 0)
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("k,ns", [(4096, (4096, 1024, 1024)), (4096, (256, 256, 256)), (11008, (96,)), (512, (40, 24))])
+def test_linear_group_norm_and_concat(hip, oracle, fmt, k, ns):
+    """RMSNorm folded into up to three projections that share the input (the q/k/v group)."""
+    ws = [synth.quant_weights(fmt, n, k, 31, i) for i, n in enumerate(ns)]
+    x = synth.activations(1, k, 32) * 3.0
+    nw = (1.0 + 0.1 * synth.activations(1, k, 33)).reshape(-1)
+    eps = float(np.float32(1e-5))
+    outs = hip.linear_group(fmt, [hip.Tensor.from_numpy(w) for w in ws], list(ns), k, hip.Tensor.from_numpy(x),
+                            norm_w=hip.Tensor.from_numpy(nw), eps=eps)
+    xn = oracle.rmsnorm(x, nw, eps)
+    for w, n, out in zip(ws, ns, outs):
+        assert rel_l2(out.numpy(), oracle.mul_mat_q(fmt, w, n, k, xn)) <= TOL
+    # without the norm
+    outs = hip.linear_group(fmt, [hip.Tensor.from_numpy(w) for w in ws], list(ns), k, hip.Tensor.from_numpy(x))
+    for w, n, out in zip(ws, ns, outs):
+        assert rel_l2(out.numpy(), oracle.mul_mat_q(fmt, w, n, k, x)) <= TOL
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("n,k", [(11008, 4096), (14336, 4096), (300, 8192), (50, 512)])
+def test_linear_group_swiglu(hip, oracle, fmt, n, k):
+    """RMSNorm -> gate/up -> silu(gate) * up in one launch (front half of the SwiGLU MLP)."""
+    wg, wu = synth.quant_weights(fmt, n, k, 41, 0), synth.quant_weights(fmt, n, k, 41, 1)
+    x = synth.activations(1, k, 42)
+    nw = np.ones(k, np.float32)
+    eps = float(np.float32(1e-5))
+    out, = hip.linear_group(fmt, [hip.Tensor.from_numpy(wg), hip.Tensor.from_numpy(wu)], [n, n], k,
+                            hip.Tensor.from_numpy(x), norm_w=hip.Tensor.from_numpy(nw), eps=eps, silu_mul=True)
+    xn = oracle.rmsnorm(x, nw, eps)
+    want = oracle.silu_mul(oracle.mul_mat_q(fmt, wg, n, k, xn), oracle.mul_mat_q(fmt, wu, n, k, xn))
+    assert rel_l2(out.numpy(), want) <= TOL
+
+
+def test_linear_group_residual_and_errors(hip, oracle):
+    n, k = 4096, 11008
+    w = synth.quant_weights(Q4_0, n, k, 51)
+    x = synth.activations(1, k, 52)
+    res = synth.activations(1, n, 53)
+    out, = hip.linear_group(Q4_0, [hip.Tensor.from_numpy(w)], [n], k, hip.Tensor.from_numpy(x),
+                            residual=hip.Tensor.from_numpy(res))
+    assert rel_l2(out.numpy(), res + oracle.mul_mat_q(Q4_0, w, n, k, x)) <= TOL
+    wt = hip.Tensor.from_numpy(w)
+    with pytest.raises(hip.LiteNNHipError, match="equal height"):
+        hip.linear_group(Q4_0, [wt, wt, wt], [n, n, n], k, hip.Tensor.from_numpy(x), silu_mul=True)
+    with pytest.raises(hip.LiteNNHipError, match="single matrix"):
+        hip.linear_group(Q4_0, [wt, wt], [n, n], k, hip.Tensor.from_numpy(x), residual=hip.Tensor.from_numpy(res))
