@@ -28,9 +28,11 @@ namespace litenn_hip
 	                 const float* cos_t, const float* sin_t, hipStream_t s);
 	void launch_kv_append(void* cache, int cache_dtype, size_t past_elems, const float* cur, size_t count,
 	                      hipStream_t s);
+	size_t attn_splits(size_t m, size_t max_len, size_t n_head);
+	size_t attn_partial_floats(size_t m, size_t n_head, size_t head_dim, size_t splits);
 	void launch_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
-	                        const int* past_dev, size_t past_host, size_t max_len, size_t n_head, size_t n_kv_head,
-	                        size_t head_dim, float* out, hipStream_t s);
+	                        const int* past_dev, size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim,
+	                        float* out, size_t splits, float* partial, int* counters, hipStream_t s);
 	void launch_silu_mul(const float* gate, const float* up, float* y, size_t n, hipStream_t s);
 	void launch_argmax(const float* x, size_t rows, size_t n, int32_t* out, hipStream_t s);
 
@@ -767,17 +769,45 @@ extern "C" int litenn_hip_attn_decode(int dev, const void* q, const void* kcache
 	{
 		return 0;
 	}
-	if (past + m > 15360)
+	if (past + m > (size_t{ 1 } << 30))
 	{
-		return fail(action, "key length exceeds the 15360 positions the score buffer holds");
+		return fail(action, "key length exceeds 2^30 positions");
 	}
-	if (m > 65535)
+	if (m > 65535 || n_head > 65535)
 	{
-		return fail(action, "too many query rows");
+		return fail(action, "too many query rows or heads");
 	}
 	GUARD(action, dev);
-	launch_attn_decode(static_cast<const float*>(q), kcache, vcache, cache_dtype, m, nullptr, past, past + m, n_head,
-	                   n_kv_head, head_dim, static_cast<float*>(out), stream_of(opts));
+	// a single row against a long cache is cut into chunks that meet in scratch memory, which
+	// this call owns: it is freed after the stream has drained, whatever opts->synchronize says
+	const size_t splits = attn_splits(m, past + m, n_head);
+	float* partial = nullptr;
+	int* counters = nullptr;
+	if (splits > 1)
+	{
+		const size_t bytes = sizeof(float) * attn_partial_floats(m, n_head, head_dim, splits);
+		LITENN_HIP_TRY(action, hipMalloc(reinterpret_cast<void**>(&partial), bytes + sizeof(int) * m * n_head));
+		counters = reinterpret_cast<int*>(reinterpret_cast<char*>(partial) + bytes);
+		const hipError_t e = hipMemsetAsync(counters, 0, sizeof(int) * m * n_head, stream_of(opts));
+		if (e != hipSuccess)
+		{
+			(void)hipFree(partial);
+			return fail_hip(action, e);
+		}
+	}
+	launch_attn_decode(static_cast<const float*>(q), kcache, vcache, cache_dtype, m, nullptr, past, n_head, n_kv_head,
+	                   head_dim, static_cast<float*>(out), splits, partial, counters, stream_of(opts));
+	if (partial)
+	{
+		const hipError_t launched = hipGetLastError();
+		const hipError_t drained = hipStreamSynchronize(stream_of(opts));
+		(void)hipFree(partial);
+		if (launched != hipSuccess || drained != hipSuccess)
+		{
+			return fail_hip(action, launched != hipSuccess ? launched : drained);
+		}
+		return 0;
+	}
 	return finish(action, opts);
 }
 

@@ -5,6 +5,8 @@
 // reference chains and to read every operand once.
 #include "common.hpp"
 
+#include <algorithm>
+
 namespace litenn_hip
 {
 	namespace
@@ -196,24 +198,92 @@ namespace litenn_hip
 		}
 
 		// ---------------- attention of one query row against the cache -----------------------
-		// grid (n_head, m); block 256.  Query row i sits at position past + i and sees keys
-		// 0 .. past + i (the additive -1e9 causal constant of CausalMask.h:16-34 turns every later
-		// key into an exact zero after exp in f32, so those keys are simply not visited).
-		// Scores live in LDS (max_len floats).  head_dim <= 256.
+		// grid (n_head, splits, m); block 256.  Query row i sits at position past + i and sees
+		// keys 0 .. past + i (the additive -1e9 causal constant of CausalMask.h:16-34 turns every
+		// later key into an exact zero after exp in f32, so those keys are simply not visited).
+		//
+		// The keys of a row are cut into `splits` contiguous chunks, one workgroup each.  Inside a
+		// workgroup a key is handled by 16 lanes (each lane owns a contiguous run of the head
+		// dimension), so a wave covers 4 keys and the workgroup 16 keys per step, kUnroll steps in
+		// flight.  Every 16-lane group keeps a running (max, sum, weighted V) triple; the 16 triples
+		// are merged through LDS.  With splits > 1 the workgroup's triple goes to `partial` and the
+		// last workgroup of the row/head to arrive (device-scope counter) merges the splits.
+		// The merged result equals softmax(q.K^T * scale) . V of Attention.h:57-80 up to f32
+		// summation order.  head_dim <= 256.
+		template <typename KV, bool FAST>
+		struct AttnLoad;
+
+		// generic: up to 16 elements per lane, bounds-checked scalar loads
 		template <typename KV>
+		struct AttnLoad<KV, false>
+		{
+			static constexpr int E = 16;
+			__device__ static void load(const KV* p, int first, int per, int head_dim, float (&out)[E])
+			{
+#pragma unroll
+				for (int e = 0; e < E; ++e)
+				{
+					out[e] = (e < per && first + e < head_dim) ? load_kv<KV>(p + first + e) : 0.0f;
+				}
+			}
+		};
+
+		// head_dim 128, 16-byte aligned rows: 8 elements per lane in one or two 16-byte loads
+		template <>
+		struct AttnLoad<uint16_t, true>
+		{
+			static constexpr int E = 8;
+			__device__ static void load(const uint16_t* p, int first, int, int, float (&out)[E])
+			{
+				const uint4 raw = *reinterpret_cast<const uint4*>(p + first);
+				const uint32_t w[4] = { raw.x, raw.y, raw.z, raw.w };
+#pragma unroll
+				for (int i = 0; i < 4; ++i)
+				{
+					out[2 * i] = f16_bits_to_f32(static_cast<uint16_t>(w[i] & 0xffffu));
+					out[2 * i + 1] = f16_bits_to_f32(static_cast<uint16_t>(w[i] >> 16));
+				}
+			}
+		};
+
+		template <>
+		struct AttnLoad<float, true>
+		{
+			static constexpr int E = 8;
+			__device__ static void load(const float* p, int first, int, int, float (&out)[E])
+			{
+				const float4 a = *reinterpret_cast<const float4*>(p + first);
+				const float4 b = *reinterpret_cast<const float4*>(p + first + 4);
+				out[0] = a.x, out[1] = a.y, out[2] = a.z, out[3] = a.w;
+				out[4] = b.x, out[5] = b.y, out[6] = b.z, out[7] = b.w;
+			}
+		};
+
+		__device__ __forceinline__ float softmax_weight(float m, float m_all)
+		{
+			return m == -INFINITY ? 0.0f : expf(m - m_all);
+		}
+
+		template <typename KV, bool FAST>
 		__global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q,
 		                                                           const KV* __restrict__ kcache,
 		                                                           const KV* __restrict__ vcache,
 		                                                           float* __restrict__ out,
 		                                                           const int* __restrict__ past_dev, int past_host,
 		                                                           int n_head, int n_kv_head, int head_dim,
-		                                                           float scale)
+		                                                           float scale, float* __restrict__ partial,
+		                                                           int* __restrict__ counters)
 		{
-			extern __shared__ float smem[];
-			__shared__ float red[8];
-			__shared__ float part_o[256];
+			using Load = AttnLoad<KV, FAST>;
+			constexpr int E = Load::E;
+			constexpr int kUnroll = 4;
+			__shared__ float s_m[16], s_l[16];
+			__shared__ float s_o[16][256 + 4];
+			__shared__ int s_last;
 			const int h = blockIdx.x;
-			const int row = blockIdx.y;
+			const int split = blockIdx.y, splits = gridDim.y;
+			const int row = blockIdx.z;
+			const int tid = threadIdx.x;
 			const int past = past_dev ? *past_dev : past_host;
 			const int len = past + row + 1;
 			const int kvh = h / (n_head / n_kv_head);
@@ -221,90 +291,159 @@ namespace litenn_hip
 			const float* qr = q + (static_cast<size_t>(row) * n_head + h) * head_dim;
 			const KV* kbase = kcache + static_cast<size_t>(kvh) * head_dim;
 			const KV* vbase = vcache + static_cast<size_t>(kvh) * head_dim;
-			float* scores = smem;
 
-			// scores: 16 lanes per key, head_dim/16 elements per lane
-			const int sub = threadIdx.x & 15;
-			const int grp = threadIdx.x >> 4; // 16 key groups per block
-			const int per = (head_dim + 15) >> 4;
-			float qv[16];
+			const int sub = tid & 15; // lane within the key's group
+			const int grp = tid >> 4; // key slot of the workgroup
+			const int per = FAST ? 8 : (head_dim + 15) >> 4;
+			const int first = sub * per;
+			float qv[E];
+			AttnLoad<float, FAST>::load(qr, first, per, head_dim, qv);
+
+			const int chunk = (len + splits - 1) / splits;
+			const int t_begin = split * chunk;
+			const int t_end = min(len, t_begin + chunk);
+
+			float run_m = -INFINITY, run_l = 0.0f;
+			float o[E];
 #pragma unroll
-			for (int e = 0; e < 16; ++e)
+			for (int e = 0; e < E; ++e)
 			{
-				qv[e] = (e < per && sub * per + e < head_dim) ? qr[sub * per + e] : 0.0f;
+				o[e] = 0.0f;
 			}
-			for (int t0 = 0; t0 < len; t0 += 16)
+			for (int t0 = t_begin + grp; t0 < t_end; t0 += 16 * kUnroll)
 			{
-				const int t = t0 + grp;
-				float acc = 0.0f;
-				if (t < len)
-				{
-					const KV* kr = kbase + static_cast<size_t>(t) * kvw + sub * per;
+				float kf[kUnroll][E], vf[kUnroll][E];
+				float s[kUnroll];
 #pragma unroll
-					for (int e = 0; e < 16; ++e)
+				for (int u = 0; u < kUnroll; ++u)
+				{
+					// keys past the chunk re-read a valid one and get weight zero below
+					const int t = min(t0 + 16 * u, t_end - 1);
+					Load::load(kbase + static_cast<size_t>(t) * kvw, first, per, head_dim, kf[u]);
+					Load::load(vbase + static_cast<size_t>(t) * kvw, first, per, head_dim, vf[u]);
+				}
+				float step_m = run_m;
+#pragma unroll
+				for (int u = 0; u < kUnroll; ++u)
+				{
+					float acc = 0.0f;
+#pragma unroll
+					for (int e = 0; e < E; ++e)
 					{
-						if (e < per && sub * per + e < head_dim)
-						{
-							acc = fmaf(qv[e], load_kv<KV>(kr + e), acc);
-						}
+						acc = fmaf(qv[e], kf[u][e], acc);
+					}
+					acc = row16_sum(acc) * scale;
+					s[u] = (t0 + 16 * u < t_end) ? acc : -INFINITY;
+					step_m = fmaxf(step_m, s[u]);
+				}
+				// step_m is finite: the first key of the step is always inside the chunk
+				const float corr = expf(run_m - step_m);
+				run_l *= corr;
+#pragma unroll
+				for (int e = 0; e < E; ++e)
+				{
+					o[e] *= corr;
+				}
+#pragma unroll
+				for (int u = 0; u < kUnroll; ++u)
+				{
+					const float p = expf(s[u] - step_m);
+					run_l += p;
+#pragma unroll
+					for (int e = 0; e < E; ++e)
+					{
+						o[e] = fmaf(p, vf[u][e], o[e]);
 					}
 				}
-				acc = row16_sum(acc);
-				if (t < len && sub == 0)
-				{
-					scores[t] = acc * scale;
-				}
+				run_m = step_m;
 			}
-			__syncthreads();
-			float mx = -INFINITY;
-			for (int t = threadIdx.x; t < len; t += blockDim.x)
-			{
-				mx = fmaxf(mx, scores[t]);
-			}
-			mx = wave_max(mx);
-			if ((threadIdx.x & 63) == 0)
-			{
-				red[threadIdx.x >> 6] = mx;
-			}
-			__syncthreads();
-			mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-			float sum = 0.0f;
-			for (int t = threadIdx.x; t < len; t += blockDim.x)
-			{
-				const float e = expf(scores[t] - mx);
-				scores[t] = e;
-				sum += e;
-			}
-			sum = wave_sum(sum);
-			if ((threadIdx.x & 63) == 0)
-			{
-				red[4 + (threadIdx.x >> 6)] = sum;
-			}
-			__syncthreads();
-			const float denom = (red[4] + red[5]) + (red[6] + red[7]);
 
-			// output: thread (part, c) accumulates keys t = part, part + parts, ...
-			const int parts = 256 / head_dim > 0 ? 256 / head_dim : 1;
-			const int c = threadIdx.x % head_dim;
-			const int part = threadIdx.x / head_dim;
-			float o = 0.0f;
-			if (part < parts)
+			if (sub == 0)
 			{
-				for (int t = part; t < len; t += parts)
+				s_m[grp] = run_m;
+				s_l[grp] = run_l;
+			}
+#pragma unroll
+			for (int e = 0; e < E; ++e)
+			{
+				if (e < per && first + e < head_dim)
 				{
-					o = fmaf(scores[t], load_kv<KV>(vbase + static_cast<size_t>(t) * kvw + c), o);
+					s_o[grp][first + e] = o[e];
 				}
 			}
-			part_o[threadIdx.x] = o;
 			__syncthreads();
-			if (threadIdx.x < head_dim)
+			float m_all = -INFINITY, l_all = 0.0f, o_all = 0.0f;
+			if (tid < head_dim)
 			{
-				float total = 0.0f;
-				for (int pp = 0; pp < parts; ++pp)
+#pragma unroll
+				for (int g = 0; g < 16; ++g)
 				{
-					total += part_o[pp * head_dim + threadIdx.x];
+					m_all = fmaxf(m_all, s_m[g]);
 				}
-				out[(static_cast<size_t>(row) * n_head + h) * head_dim + threadIdx.x] = total / denom;
+#pragma unroll
+				for (int g = 0; g < 16; ++g)
+				{
+					const float w = softmax_weight(s_m[g], m_all);
+					l_all = fmaf(s_l[g], w, l_all);
+					o_all = fmaf(s_o[g][tid], w, o_all);
+				}
+			}
+			float* dst = out + (static_cast<size_t>(row) * n_head + h) * head_dim;
+			if (splits == 1)
+			{
+				if (tid < head_dim)
+				{
+					dst[tid] = o_all / l_all;
+				}
+				return;
+			}
+
+			// several splits: publish this chunk's triple, the last arrival merges them
+			const size_t slot = static_cast<size_t>(row) * n_head + h;
+			const int stride = head_dim + 2;
+			float* mine = partial + (slot * splits + split) * stride;
+			if (tid < head_dim)
+			{
+				mine[2 + tid] = o_all;
+				if (tid == 0)
+				{
+					mine[0] = m_all;
+					mine[1] = l_all;
+				}
+			}
+			__threadfence();
+			__syncthreads();
+			if (tid == 0)
+			{
+				const int arrived = atomicAdd(&counters[slot], 1);
+				s_last = arrived == splits - 1;
+				if (s_last)
+				{
+					counters[slot] = 0; // ready for the next launch on this stream
+				}
+			}
+			__syncthreads();
+			if (!s_last)
+			{
+				return;
+			}
+			__threadfence();
+			if (tid < head_dim)
+			{
+				const float* all = partial + slot * splits * stride;
+				float mm = -INFINITY;
+				for (int sidx = 0; sidx < splits; ++sidx)
+				{
+					mm = fmaxf(mm, __builtin_nontemporal_load(all + sidx * stride));
+				}
+				float ll = 0.0f, oo = 0.0f;
+				for (int sidx = 0; sidx < splits; ++sidx)
+				{
+					const float w = softmax_weight(__builtin_nontemporal_load(all + sidx * stride), mm);
+					ll = fmaf(__builtin_nontemporal_load(all + sidx * stride + 1), w, ll);
+					oo = fmaf(__builtin_nontemporal_load(all + sidx * stride + 2 + tid), w, oo);
+				}
+				dst[tid] = oo / ll;
 			}
 		}
 
@@ -433,27 +572,58 @@ namespace litenn_hip
 		}
 	}
 
-	// max_len: upper bound of past + m (sizes the LDS score buffer)
-	void launch_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
-	                        const int* past_dev, size_t past_host, size_t max_len, size_t n_head, size_t n_kv_head,
-	                        size_t head_dim, float* out, hipStream_t s)
+	// Number of key chunks one query row is cut into.  Only a single row is ever split (several
+	// rows already give the machine enough workgroups); the count depends on the upper bound of
+	// the key length alone, so a captured launch stays valid while the cache fills.
+	size_t attn_splits(size_t m, size_t max_len, size_t n_head)
 	{
-		const dim3 grid(n_head, m), block(256);
-		const size_t lds = sizeof(float) * max_len;
+		if (m != 1)
+		{
+			return 1;
+		}
+		const size_t by_len = (max_len + 63) / 64;
+		const size_t by_heads = (1024 + n_head - 1) / n_head;
+		return std::max<size_t>(1, std::min<size_t>({ 16, by_len, by_heads }));
+	}
+
+	// floats of `partial` a launch with that many splits needs (and m * n_head zeroed ints of counters)
+	size_t attn_partial_floats(size_t m, size_t n_head, size_t head_dim, size_t splits)
+	{
+		return splits > 1 ? m * n_head * splits * (head_dim + 2) : 0;
+	}
+
+	template <typename KV>
+	static void launch_attn_typed(const float* q, const KV* kcache, const KV* vcache, size_t m, const int* past_dev,
+	                              size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim, float* out,
+	                              size_t splits, float* partial, int* counters, hipStream_t s)
+	{
+		const dim3 grid(n_head, splits, m), block(256);
 		const float scale = static_cast<float>(1.0 / sqrt(static_cast<double>(head_dim)));
+		const auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+		const bool fast = head_dim == 128 && aligned(q) && aligned(kcache) && aligned(vcache);
+		auto kernel = fast ? attn_decode_kernel<KV, true> : attn_decode_kernel<KV, false>;
+		kernel<<<grid, block, 0, s>>>(q, kcache, vcache, out, past_dev, static_cast<int>(past_host),
+		                              static_cast<int>(n_head), static_cast<int>(n_kv_head),
+		                              static_cast<int>(head_dim), scale, partial, counters);
+	}
+
+	// splits > 1 needs `partial` (attn_partial_floats) and `counters` (m * n_head ints, zero before
+	// the first launch; every launch leaves them zero again)
+	void launch_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
+	                        const int* past_dev, size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim,
+	                        float* out, size_t splits, float* partial, int* counters, hipStream_t s)
+	{
 		if (cache_dtype == LITENN_F16)
 		{
-			attn_decode_kernel<uint16_t><<<grid, block, lds, s>>>(
-			    q, static_cast<const uint16_t*>(kcache), static_cast<const uint16_t*>(vcache), out, past_dev,
-			    static_cast<int>(past_host), static_cast<int>(n_head), static_cast<int>(n_kv_head),
-			    static_cast<int>(head_dim), scale);
+			launch_attn_typed<uint16_t>(q, static_cast<const uint16_t*>(kcache), static_cast<const uint16_t*>(vcache),
+			                            m, past_dev, past_host, n_head, n_kv_head, head_dim, out, splits, partial,
+			                            counters, s);
 		}
 		else
 		{
-			attn_decode_kernel<float><<<grid, block, lds, s>>>(
-			    q, static_cast<const float*>(kcache), static_cast<const float*>(vcache), out, past_dev,
-			    static_cast<int>(past_host), static_cast<int>(n_head), static_cast<int>(n_kv_head),
-			    static_cast<int>(head_dim), scale);
+			launch_attn_typed<float>(q, static_cast<const float*>(kcache), static_cast<const float*>(vcache), m,
+			                         past_dev, past_host, n_head, n_kv_head, head_dim, out, splits, partial, counters,
+			                         s);
 		}
 	}
 

@@ -29,9 +29,11 @@ namespace litenn_hip
 	void launch_rope_qkv_append(float* q, const float* k, const float* v, void* kcache, void* vcache, int cache_dtype,
 	                            const int* past_dev, size_t m, size_t n_head, size_t n_kv_head, size_t head_dim,
 	                            size_t rope_dims, const float* cos_t, const float* sin_t, hipStream_t s);
+	size_t attn_splits(size_t m, size_t max_len, size_t n_head);
+	size_t attn_partial_floats(size_t m, size_t n_head, size_t head_dim, size_t splits);
 	void launch_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
-	                        const int* past_dev, size_t past_host, size_t max_len, size_t n_head, size_t n_kv_head,
-	                        size_t head_dim, float* out, hipStream_t s);
+	                        const int* past_dev, size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim,
+	                        float* out, size_t splits, float* partial, int* counters, hipStream_t s);
 	void launch_silu_mul(const float* gate, const float* up, float* y, size_t n, hipStream_t s);
 	void launch_argmax(const float* x, size_t rows, size_t n, int32_t* out, hipStream_t s);
 	bool launch_convert(int src_dtype, const void* src, size_t n, int dst_dtype, void* dst, hipStream_t s);
@@ -96,6 +98,10 @@ struct litenn_hip_llama
 	size_t cap_out = 0;
 	int* d_counters = nullptr; // {past, emitted}
 	int* d_err = nullptr;
+	// single-row attention: key chunks per head, their meeting place and arrival counters
+	size_t attn_splits = 1;
+	float* attn_partial = nullptr;
+	int* attn_counters = nullptr;
 	int past = 0;
 	hipGraphExec_t step_exec = nullptr;
 	hipGraph_t step_graph = nullptr;
@@ -248,8 +254,8 @@ namespace
 			}
 			launch_rope_qkv_append(m->q, m->k, m->v, L.kcache, L.vcache, m->p.kv_dtype, past_dev, 1, H, KH, hd,
 			                       m->p.rope_dimension_count, m->cos_t, m->sin_t, s);
-			launch_attn_decode(m->q, L.kcache, L.vcache, m->p.kv_dtype, 1, past_dev, 0, m->p.context_length, H, KH, hd,
-			                   m->attn, s);
+			launch_attn_decode(m->q, L.kcache, L.vcache, m->p.kv_dtype, 1, past_dev, 0, H, KH, hd, m->attn,
+			                   m->attn_splits, m->attn_partial, m->attn_counters, s);
 			const Weight* wo[1] = { &L.wo };
 			float* xo[1] = { m->x };
 			group(m, 1, wo, xo, m->attn, m->x, nullptr, false, s); // x = x + attn . Wo
@@ -301,8 +307,8 @@ namespace
 			matmul(L.wv, m->xn, rows, m->v, nullptr, flags, s);
 			launch_rope_qkv_append(m->q, m->k, m->v, L.kcache, L.vcache, m->p.kv_dtype, past_dev, rows, H, KH, hd,
 			                       m->p.rope_dimension_count, m->cos_t, m->sin_t, s);
-			launch_attn_decode(m->q, L.kcache, L.vcache, m->p.kv_dtype, rows, past_dev, 0, m->p.context_length, H, KH,
-			                   hd, m->attn, s);
+			launch_attn_decode(m->q, L.kcache, L.vcache, m->p.kv_dtype, rows, past_dev, 0, H, KH, hd, m->attn,
+			                   rows == 1 ? m->attn_splits : 1, m->attn_partial, m->attn_counters, s);
 			matmul(L.wo, m->attn, rows, m->x, m->x, flags, s); // x = x + attn . Wo
 			launch_rmsnorm(m->x, L.ffn_norm, m->p.rms_norm_epsilon, rows, d, m->xn, s);
 			matmul(L.gate, m->xn, rows, m->gate, nullptr, flags, s);
@@ -437,6 +443,18 @@ extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* p
 	{
 		return bail(e);
 	}
+	m->attn_splits = attn_splits(1, static_cast<size_t>(p.context_length), static_cast<size_t>(p.head_count));
+	if (m->attn_splits > 1)
+	{
+		const size_t heads = static_cast<size_t>(p.head_count);
+		const size_t floats = attn_partial_floats(1, heads, static_cast<size_t>(head_dim), m->attn_splits);
+		if ((e = hipMalloc(reinterpret_cast<void**>(&m->attn_partial), sizeof(float) * floats)) != hipSuccess ||
+		    (e = hipMalloc(reinterpret_cast<void**>(&m->attn_counters), sizeof(int) * heads)) != hipSuccess ||
+		    (e = hipMemset(m->attn_counters, 0, sizeof(int) * heads)) != hipSuccess)
+		{
+			return bail(e);
+		}
+	}
 	*out = m;
 	return 0;
 }
@@ -465,7 +483,8 @@ extern "C" int litenn_hip_llama_free(litenn_hip_llama* m)
 			(void)hipFree(L.vcache);
 		}
 	}
-	void* singles[] = { m->cos_t, m->sin_t, m->logits, m->d_next, m->d_out, m->d_counters, m->d_err };
+	void* singles[] = { m->cos_t, m->sin_t,      m->logits,       m->d_next,       m->d_out,
+	                    m->d_counters, m->d_err, m->attn_partial, m->attn_counters };
 	for (void* ptr : singles)
 	{
 		if (ptr)

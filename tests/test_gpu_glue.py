@@ -74,7 +74,8 @@ def test_kv_append_f16_uses_litenn_rounding(hip, oracle, golden):
 def test_attention_decode(hip, oracle, cache_dtype):
     rng = np.random.default_rng(4)
     for m, past, H, KH, hd in [(1, 0, 4, 4, 128), (1, 383, 32, 32, 128), (1, 1023, 32, 8, 128), (6, 10, 8, 2, 64),
-                               (2, 1, 2, 1, 2), (3, 0, 4, 2, 80)]:
+                               (2, 1, 2, 1, 2), (3, 0, 4, 2, 80), (1, 100, 32, 32, 128), (1, 4000, 8, 8, 128),
+                               (1, 70, 5, 5, 128), (1, 200, 4, 2, 96), (40, 0, 8, 8, 128)]:
         L = past + m
         q = rng.standard_normal((m, H * hd)).astype(np.float32)
         k = rng.standard_normal((L, KH * hd)).astype(np.float32)
