@@ -259,6 +259,17 @@ namespace litenn_hip
 			}
 		};
 
+		constexpr int kMaxAttnSplits = 16;
+
+		__device__ __forceinline__ void device_store(float* p, float v)
+		{
+			__hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		}
+		__device__ __forceinline__ float device_load(const float* p)
+		{
+			return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		}
+
 		__device__ __forceinline__ float softmax_weight(float m, float m_all)
 		{
 			return m == -INFINITY ? 0.0f : expf(m - m_all);
@@ -402,24 +413,30 @@ namespace litenn_hip
 			const size_t slot = static_cast<size_t>(row) * n_head + h;
 			const int stride = head_dim + 2;
 			float* mine = partial + (slot * splits + split) * stride;
+			// The triples cross between workgroups (and between the chip's L2 slices) through
+			// device-scope relaxed atomics, which write through and read around the non-coherent
+			// cache levels; a full device fence would instead flush the whole L2 in every workgroup.
+			// Order: triple stores complete (vmcnt 0) -> barrier -> counter increment; the merging
+			// workgroup reads the triples only after it has seen the last increment.
 			if (tid < head_dim)
 			{
-				mine[2 + tid] = o_all;
+				device_store(mine + 2 + tid, o_all);
 				if (tid == 0)
 				{
-					mine[0] = m_all;
-					mine[1] = l_all;
+					device_store(mine, m_all);
+					device_store(mine + 1, l_all);
 				}
 			}
-			__threadfence();
+			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 			__syncthreads();
 			if (tid == 0)
 			{
-				const int arrived = atomicAdd(&counters[slot], 1);
+				const int arrived = __hip_atomic_fetch_add(&counters[slot], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 				s_last = arrived == splits - 1;
 				if (s_last)
 				{
-					counters[slot] = 0; // ready for the next launch on this stream
+					// ready for the next launch on this stream
+					__hip_atomic_store(&counters[slot], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 				}
 			}
 			__syncthreads();
@@ -427,21 +444,32 @@ namespace litenn_hip
 			{
 				return;
 			}
-			__threadfence();
 			if (tid < head_dim)
 			{
+				// every split's triple is fetched before the first is used: one memory latency
 				const float* all = partial + slot * splits * stride;
-				float mm = -INFINITY;
-				for (int sidx = 0; sidx < splits; ++sidx)
+				float pm[kMaxAttnSplits], pl[kMaxAttnSplits], po[kMaxAttnSplits];
+#pragma unroll
+				for (int sidx = 0; sidx < kMaxAttnSplits; ++sidx)
 				{
-					mm = fmaxf(mm, __builtin_nontemporal_load(all + sidx * stride));
+					const float* src = all + min(sidx, splits - 1) * stride;
+					pm[sidx] = device_load(src);
+					pl[sidx] = device_load(src + 1);
+					po[sidx] = device_load(src + 2 + tid);
+				}
+				float mm = -INFINITY;
+#pragma unroll
+				for (int sidx = 0; sidx < kMaxAttnSplits; ++sidx)
+				{
+					mm = fmaxf(mm, pm[sidx]);
 				}
 				float ll = 0.0f, oo = 0.0f;
-				for (int sidx = 0; sidx < splits; ++sidx)
+#pragma unroll
+				for (int sidx = 0; sidx < kMaxAttnSplits; ++sidx)
 				{
-					const float w = softmax_weight(__builtin_nontemporal_load(all + sidx * stride), mm);
-					ll = fmaf(__builtin_nontemporal_load(all + sidx * stride + 1), w, ll);
-					oo = fmaf(__builtin_nontemporal_load(all + sidx * stride + 2 + tid), w, oo);
+					const float w = sidx < splits ? softmax_weight(pm[sidx], mm) : 0.0f;
+					ll = fmaf(pl[sidx], w, ll);
+					oo = fmaf(po[sidx], w, oo);
 				}
 				dst[tid] = oo / ll;
 			}
@@ -583,7 +611,7 @@ namespace litenn_hip
 		}
 		const size_t by_len = (max_len + 63) / 64;
 		const size_t by_heads = (1024 + n_head - 1) / n_head;
-		return std::max<size_t>(1, std::min<size_t>({ 16, by_len, by_heads }));
+		return std::max<size_t>(1, std::min<size_t>({ kMaxAttnSplits, by_len, by_heads }));
 	}
 
 	// floats of `partial` a launch with that many splits needs (and m * n_head zeroed ints of counters)
