@@ -74,38 +74,25 @@ namespace litenn_hip
 	// same way.  Not IEEE round-to-nearest-even, so the hardware converter is not used.
 	__device__ __forceinline__ uint16_t f32_to_f16_bits_litenn(float value)
 	{
+		// branch-free: every range is computed and the result selected, so a wave converting a
+		// handful of values does not serialise through divergent paths
 		const uint32_t bits = __float_as_uint(value);
 		const uint32_t sign = (bits >> 16) & 0x8000u;
-		const int exponent = static_cast<int>((bits >> 23) & 0xffu) - 127;
-		uint32_t mantissa = bits & 0x7fffffu;
-		if ((bits & 0x7fffffffu) == 0)
-		{
-			return static_cast<uint16_t>(sign);
-		}
-		if (((bits >> 23) & 0xffu) == 0xffu)
-		{
-			return static_cast<uint16_t>(sign | 0x7c00u | (mantissa ? 0x0200u : 0u));
-		}
-		if (exponent > 15)
-		{
-			return static_cast<uint16_t>(sign | 0x7c00u);
-		}
-		if (exponent < -14)
-		{
-			if (exponent < -24)
-			{
-				return static_cast<uint16_t>(sign);
-			}
-			mantissa |= 0x800000u;
-			const uint32_t shift = static_cast<uint32_t>(-exponent - 1);
-			uint32_t half_mantissa = mantissa >> shift;
-			half_mantissa += (mantissa >> (shift - 1)) & 1u;
-			return static_cast<uint16_t>(sign | half_mantissa);
-		}
-		// adding the rounding bit carries into the exponent exactly as the reference's
-		// explicit mantissa-overflow branch does, and saturates at infinity (0x7c00)
-		uint32_t half = (static_cast<uint32_t>(exponent + 15) << 10) | (mantissa >> 13);
-		half += (mantissa >> 12) & 1u;
+		const uint32_t mag = bits & 0x7fffffffu;
+		const uint32_t exp_field = mag >> 23; // biased by 127
+		// normal halves (exponent -14 .. 15): adding the first dropped bit carries into the
+		// exponent exactly as the reference's explicit mantissa-overflow branch does, and
+		// saturates at infinity (0x7c00)
+		const uint32_t normal = ((mag + 0x1000u) >> 13) - 0x1c000u;
+		// subnormal halves (exponent -24 .. -15): shift = -exponent - 1 in [14, 23]
+		const uint32_t mantissa = (mag & 0x7fffffu) | 0x800000u;
+		const uint32_t shift = 126u - exp_field;
+		const uint32_t subnormal = ((mantissa >> ((shift - 1u) & 31u)) + 1u) >> 1;
+		uint32_t half = normal;
+		half = exp_field < 113u ? subnormal : half;
+		half = exp_field < 103u ? 0u : half;         // below 2^-24 (and f32 zero/subnormals): zero
+		half = mag >= 0x47800000u ? 0x7c00u : half; // exponent above 15, infinity
+		half = mag > 0x7f800000u ? 0x7e00u : half;  // NaN
 		return static_cast<uint16_t>(sign | half);
 	}
 

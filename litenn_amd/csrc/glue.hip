@@ -210,6 +210,8 @@ namespace litenn_hip
 		// last workgroup of the row/head to arrive (device-scope counter) merges the splits.
 		// The merged result equals softmax(q.K^T * scale) . V of Attention.h:57-80 up to f32
 		// summation order.  head_dim <= 256.
+		// AttnLoad: the run of the head dimension a lane owns, fetched as raw words (so several
+		// rows can be in flight before any is converted) and unpacked to f32 afterwards.
 		template <typename KV, bool FAST>
 		struct AttnLoad;
 
@@ -218,12 +220,26 @@ namespace litenn_hip
 		struct AttnLoad<KV, false>
 		{
 			static constexpr int E = 16;
-			__device__ static void load(const KV* p, int first, int per, int head_dim, float (&out)[E])
+			struct Raw
+			{
+				KV v[E];
+			};
+			__device__ static Raw load(const KV* p, int first, int per, int head_dim)
+			{
+				Raw r;
+#pragma unroll
+				for (int e = 0; e < E; ++e)
+				{
+					r.v[e] = (e < per && first + e < head_dim) ? p[first + e] : KV{};
+				}
+				return r;
+			}
+			__device__ static void unpack(const Raw& r, float (&out)[E])
 			{
 #pragma unroll
 				for (int e = 0; e < E; ++e)
 				{
-					out[e] = (e < per && first + e < head_dim) ? load_kv<KV>(p + first + e) : 0.0f;
+					out[e] = load_kv<KV>(&r.v[e]);
 				}
 			}
 		};
@@ -233,9 +249,13 @@ namespace litenn_hip
 		struct AttnLoad<uint16_t, true>
 		{
 			static constexpr int E = 8;
-			__device__ static void load(const uint16_t* p, int first, int, int, float (&out)[E])
+			using Raw = uint4;
+			__device__ static Raw load(const uint16_t* p, int first, int, int)
 			{
-				const uint4 raw = *reinterpret_cast<const uint4*>(p + first);
+				return *reinterpret_cast<const uint4*>(p + first);
+			}
+			__device__ static void unpack(const Raw& raw, float (&out)[E])
+			{
 				const uint32_t w[4] = { raw.x, raw.y, raw.z, raw.w };
 #pragma unroll
 				for (int i = 0; i < 4; ++i)
@@ -250,12 +270,18 @@ namespace litenn_hip
 		struct AttnLoad<float, true>
 		{
 			static constexpr int E = 8;
-			__device__ static void load(const float* p, int first, int, int, float (&out)[E])
+			struct Raw
 			{
-				const float4 a = *reinterpret_cast<const float4*>(p + first);
-				const float4 b = *reinterpret_cast<const float4*>(p + first + 4);
-				out[0] = a.x, out[1] = a.y, out[2] = a.z, out[3] = a.w;
-				out[4] = b.x, out[5] = b.y, out[6] = b.z, out[7] = b.w;
+				float4 a, b;
+			};
+			__device__ static Raw load(const float* p, int first, int, int)
+			{
+				return Raw{ *reinterpret_cast<const float4*>(p + first), *reinterpret_cast<const float4*>(p + first + 4) };
+			}
+			__device__ static void unpack(const Raw& r, float (&out)[E])
+			{
+				out[0] = r.a.x, out[1] = r.a.y, out[2] = r.a.z, out[3] = r.a.w;
+				out[4] = r.b.x, out[5] = r.b.y, out[6] = r.b.z, out[7] = r.b.w;
 			}
 		};
 
@@ -275,17 +301,79 @@ namespace litenn_hip
 			return m == -INFINITY ? 0.0f : expf(m - m_all);
 		}
 
-		template <typename KV, bool FAST>
-		__global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q,
-		                                                           const KV* __restrict__ kcache,
-		                                                           const KV* __restrict__ vcache,
-		                                                           float* __restrict__ out,
+		// What the single-token step adds when the rotation and the cache append ride inside the
+		// attention launch (tools/gguf/LLaMABuilder.cpp:596-622,640-645): q, k_new and v_new are the
+		// un-rotated projections of the one new row; the tables are [ctx, rope_dims / 2].
+		struct AttnStep
+		{
+			const float* k_new;
+			const float* v_new;
+			const float* cos_t;
+			const float* sin_t;
+			int rope_dims;
+		};
+
+		template <typename KV>
+		__device__ __forceinline__ float through_cache(float v);
+		template <>
+		__device__ __forceinline__ float through_cache<float>(float v) { return v; }
+		template <>
+		__device__ __forceinline__ float through_cache<uint16_t>(float v)
+		{
+			return f16_bits_to_f32(f32_to_f16_bits_litenn(v));
+		}
+
+		__device__ __forceinline__ void store8(float* dst, const float (&v)[8])
+		{
+			reinterpret_cast<float4*>(dst)[0] = make_float4(v[0], v[1], v[2], v[3]);
+			reinterpret_cast<float4*>(dst)[1] = make_float4(v[4], v[5], v[6], v[7]);
+		}
+		__device__ __forceinline__ void store8(uint16_t* dst, const float (&v)[8])
+		{
+			uint32_t w[4];
+#pragma unroll
+			for (int i = 0; i < 4; ++i)
+			{
+				w[i] = static_cast<uint32_t>(f32_to_f16_bits_litenn(v[2 * i])) |
+				       (static_cast<uint32_t>(f32_to_f16_bits_litenn(v[2 * i + 1])) << 16);
+			}
+			*reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+		}
+
+		// the four interleaved pairs a lane owns, rotated by the angles of its position
+		__device__ __forceinline__ void rotate8(float (&v)[8], const float4& c, const float4& sn)
+		{
+			const float cs[4] = { c.x, c.y, c.z, c.w }, ss[4] = { sn.x, sn.y, sn.z, sn.w };
+#pragma unroll
+			for (int i = 0; i < 4; ++i)
+			{
+				float o0, o1;
+				rotate(v[2 * i], v[2 * i + 1], cs[i], ss[i], o0, o1);
+				v[2 * i] = o0;
+				v[2 * i + 1] = o1;
+			}
+		}
+
+		// FUSED (single new row, head_dim 128): q arrives un-rotated and is rotated in registers;
+		// the cache holds positions 0 .. past - 1 and the new position's key/value come from
+		// step.k_new / step.v_new, rounded through the cache's type exactly as an append followed
+		// by a read would round them.  The first query head of every KV head also writes them to
+		// the cache, which no workgroup of this launch reads at that position.
+		//
+		// Every global load that does not depend on another is issued before the first wait (the
+		// row's operands, the first batch of cached keys), so a launch costs about two memory
+		// latencies however it is configured.
+		template <typename KV, bool FAST, bool FUSED>
+		__global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, KV* __restrict__ kcache,
+		                                                           KV* __restrict__ vcache, float* __restrict__ out,
 		                                                           const int* __restrict__ past_dev, int past_host,
 		                                                           int n_head, int n_kv_head, int head_dim,
 		                                                           float scale, float* __restrict__ partial,
-		                                                           int* __restrict__ counters)
+		                                                           int* __restrict__ counters, AttnStep step)
 		{
+			static_assert(!FUSED || FAST, "the fused step exists for 128-wide heads only");
 			using Load = AttnLoad<KV, FAST>;
+			using LoadF = AttnLoad<float, FAST>;
 			constexpr int E = Load::E;
 			constexpr int kUnroll = 4;
 			__shared__ float s_m[16], s_l[16];
@@ -296,7 +384,8 @@ namespace litenn_hip
 			const int row = blockIdx.z;
 			const int tid = threadIdx.x;
 			const int past = past_dev ? *past_dev : past_host;
-			const int len = past + row + 1;
+			const int pos = past + row;
+			const int len = FUSED ? pos : pos + 1; // keys read from the cache
 			const int kvh = h / (n_head / n_kv_head);
 			const size_t kvw = static_cast<size_t>(n_kv_head) * head_dim;
 			const float* qr = q + (static_cast<size_t>(row) * n_head + h) * head_dim;
@@ -307,12 +396,61 @@ namespace litenn_hip
 			const int grp = tid >> 4; // key slot of the workgroup
 			const int per = FAST ? 8 : (head_dim + 15) >> 4;
 			const int first = sub * per;
-			float qv[E];
-			AttnLoad<float, FAST>::load(qr, first, per, head_dim, qv);
 
 			const int chunk = (len + splits - 1) / splits;
 			const int t_begin = split * chunk;
 			const int t_end = min(len, t_begin + chunk);
+
+			// ---- issue: the row's operands, then the first batch of keys and values
+			const typename LoadF::Raw q_raw = LoadF::load(qr, first, per, head_dim);
+			const bool new_key_here = FUSED && split == splits - 1 && grp == 0;
+			float4 cos4 = {}, sin4 = {};
+			typename LoadF::Raw kn_raw = {}, vn_raw = {};
+			const bool rotates = FUSED && first < step.rope_dims;
+			if constexpr (FUSED)
+			{
+				// lanes outside the rotary width fetch (and ignore) the first angles of the row
+				const size_t at = static_cast<size_t>(pos) * (step.rope_dims >> 1) + (rotates ? first >> 1 : 0);
+				cos4 = *reinterpret_cast<const float4*>(step.cos_t + at);
+				sin4 = *reinterpret_cast<const float4*>(step.sin_t + at);
+				kn_raw = LoadF::load(step.k_new + static_cast<size_t>(kvh) * head_dim, first, per, head_dim);
+				vn_raw = LoadF::load(step.v_new + static_cast<size_t>(kvh) * head_dim, first, per, head_dim);
+			}
+			typename Load::Raw k_raw[kUnroll], v_raw[kUnroll];
+			int t0 = t_begin + grp;
+			const auto issue = [&](int from) {
+#pragma unroll
+				for (int u = 0; u < kUnroll; ++u)
+				{
+					// keys past the chunk re-read a valid one and get weight zero below
+					const int t = min(from + 16 * u, t_end - 1);
+					k_raw[u] = Load::load(kbase + static_cast<size_t>(t) * kvw, first, per, head_dim);
+					v_raw[u] = Load::load(vbase + static_cast<size_t>(t) * kvw, first, per, head_dim);
+				}
+			};
+			if (t0 < t_end)
+			{
+				issue(t0);
+			}
+
+			float qv[E];
+			LoadF::unpack(q_raw, qv);
+			float kn[E], vn[E];
+			if constexpr (FUSED)
+			{
+				LoadF::unpack(kn_raw, kn);
+				LoadF::unpack(vn_raw, vn);
+				if (rotates)
+				{
+					rotate8(qv, cos4, sin4);
+					rotate8(kn, cos4, sin4);
+				}
+				if (new_key_here && h % (n_head / n_kv_head) == 0)
+				{
+					store8(kcache + static_cast<size_t>(pos) * kvw + kvh * head_dim + first, kn);
+					store8(vcache + static_cast<size_t>(pos) * kvw + kvh * head_dim + first, vn);
+				}
+			}
 
 			float run_m = -INFINITY, run_l = 0.0f;
 			float o[E];
@@ -321,17 +459,20 @@ namespace litenn_hip
 			{
 				o[e] = 0.0f;
 			}
-			for (int t0 = t_begin + grp; t0 < t_end; t0 += 16 * kUnroll)
+			while (t0 < t_end)
 			{
 				float kf[kUnroll][E], vf[kUnroll][E];
 				float s[kUnroll];
 #pragma unroll
 				for (int u = 0; u < kUnroll; ++u)
 				{
-					// keys past the chunk re-read a valid one and get weight zero below
-					const int t = min(t0 + 16 * u, t_end - 1);
-					Load::load(kbase + static_cast<size_t>(t) * kvw, first, per, head_dim, kf[u]);
-					Load::load(vbase + static_cast<size_t>(t) * kvw, first, per, head_dim, vf[u]);
+					Load::unpack(k_raw[u], kf[u]);
+					Load::unpack(v_raw[u], vf[u]);
+				}
+				const int t_next = t0 + 16 * kUnroll;
+				if (t_next < t_end)
+				{
+					issue(t_next);
 				}
 				float step_m = run_m;
 #pragma unroll
@@ -367,6 +508,31 @@ namespace litenn_hip
 					}
 				}
 				run_m = step_m;
+				t0 = t_next;
+			}
+
+			if constexpr (FUSED)
+			{
+				if (new_key_here)
+				{
+					float acc = 0.0f;
+#pragma unroll
+					for (int e = 0; e < E; ++e)
+					{
+						acc = fmaf(qv[e], through_cache<KV>(kn[e]), acc);
+					}
+					const float sc = row16_sum(acc) * scale;
+					const float step_m = fmaxf(run_m, sc);
+					const float corr = expf(run_m - step_m);
+					const float pw = expf(sc - step_m);
+					run_l = fmaf(run_l, corr, pw);
+#pragma unroll
+					for (int e = 0; e < E; ++e)
+					{
+						o[e] = fmaf(pw, through_cache<KV>(vn[e]), o[e] * corr);
+					}
+					run_m = step_m;
+				}
 			}
 
 			if (sub == 0)
@@ -621,18 +787,37 @@ namespace litenn_hip
 	}
 
 	template <typename KV>
-	static void launch_attn_typed(const float* q, const KV* kcache, const KV* vcache, size_t m, const int* past_dev,
+	static void launch_attn_typed(const float* q, KV* kcache, KV* vcache, size_t m, const int* past_dev,
 	                              size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim, float* out,
-	                              size_t splits, float* partial, int* counters, hipStream_t s)
+	                              size_t splits, float* partial, int* counters, const AttnStep* step, hipStream_t s)
 	{
 		const dim3 grid(n_head, splits, m), block(256);
 		const float scale = static_cast<float>(1.0 / sqrt(static_cast<double>(head_dim)));
 		const auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
 		const bool fast = head_dim == 128 && aligned(q) && aligned(kcache) && aligned(vcache);
-		auto kernel = fast ? attn_decode_kernel<KV, true> : attn_decode_kernel<KV, false>;
+		auto kernel = step ? attn_decode_kernel<KV, true, true>
+		                   : fast ? attn_decode_kernel<KV, true, false> : attn_decode_kernel<KV, false, false>;
 		kernel<<<grid, block, 0, s>>>(q, kcache, vcache, out, past_dev, static_cast<int>(past_host),
 		                              static_cast<int>(n_head), static_cast<int>(n_kv_head),
-		                              static_cast<int>(head_dim), scale, partial, counters);
+		                              static_cast<int>(head_dim), scale, partial, counters,
+		                              step ? *step : AttnStep{});
+	}
+
+	static void launch_attn_any(const float* q, void* kcache, void* vcache, int cache_dtype, size_t m,
+	                            const int* past_dev, size_t past_host, size_t n_head, size_t n_kv_head,
+	                            size_t head_dim, float* out, size_t splits, float* partial, int* counters,
+	                            const AttnStep* step, hipStream_t s)
+	{
+		if (cache_dtype == LITENN_F16)
+		{
+			launch_attn_typed<uint16_t>(q, static_cast<uint16_t*>(kcache), static_cast<uint16_t*>(vcache), m, past_dev,
+			                            past_host, n_head, n_kv_head, head_dim, out, splits, partial, counters, step, s);
+		}
+		else
+		{
+			launch_attn_typed<float>(q, static_cast<float*>(kcache), static_cast<float*>(vcache), m, past_dev, past_host,
+			                         n_head, n_kv_head, head_dim, out, splits, partial, counters, step, s);
+		}
 	}
 
 	// splits > 1 needs `partial` (attn_partial_floats) and `counters` (m * n_head ints, zero before
@@ -641,18 +826,28 @@ namespace litenn_hip
 	                        const int* past_dev, size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim,
 	                        float* out, size_t splits, float* partial, int* counters, hipStream_t s)
 	{
-		if (cache_dtype == LITENN_F16)
-		{
-			launch_attn_typed<uint16_t>(q, static_cast<const uint16_t*>(kcache), static_cast<const uint16_t*>(vcache),
-			                            m, past_dev, past_host, n_head, n_kv_head, head_dim, out, splits, partial,
-			                            counters, s);
-		}
-		else
-		{
-			launch_attn_typed<float>(q, static_cast<const float*>(kcache), static_cast<const float*>(vcache), m,
-			                         past_dev, past_host, n_head, n_kv_head, head_dim, out, splits, partial, counters,
-			                         s);
-		}
+		launch_attn_any(q, const_cast<void*>(kcache), const_cast<void*>(vcache), cache_dtype, m, past_dev, past_host,
+		                n_head, n_kv_head, head_dim, out, splits, partial, counters, nullptr, s);
+	}
+
+	// Whether one new row's rotation, cache append and attention can run as a single launch.
+	bool attn_step_fusable(const float* q, const float* k, const float* v, const void* kcache, const void* vcache,
+	                       size_t head_dim, size_t rope_dims, const float* cos_t, const float* sin_t)
+	{
+		const auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+		return head_dim == 128 && rope_dims % 8 == 0 && rope_dims <= head_dim && aligned(q) && aligned(k) &&
+		       aligned(v) && aligned(kcache) && aligned(vcache) && aligned(cos_t) && aligned(sin_t);
+	}
+
+	// rope(q), rope(k) -> cache, v -> cache, attention of the new row: one launch.  Position = *past_dev.
+	void launch_attn_step(const float* q, const float* k, const float* v, void* kcache, void* vcache, int cache_dtype,
+	                      const int* past_dev, size_t n_head, size_t n_kv_head, size_t head_dim, size_t rope_dims,
+	                      const float* cos_t, const float* sin_t, float* out, size_t splits, float* partial,
+	                      int* counters, hipStream_t s)
+	{
+		const AttnStep step{ k, v, cos_t, sin_t, static_cast<int>(rope_dims) };
+		launch_attn_any(q, kcache, vcache, cache_dtype, 1, past_dev, 0, n_head, n_kv_head, head_dim, out, splits,
+		                partial, counters, &step, s);
 	}
 
 	void launch_silu_mul(const float* gate, const float* up, float* y, size_t n, hipStream_t s)

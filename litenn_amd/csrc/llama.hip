@@ -29,6 +29,12 @@ namespace litenn_hip
 	void launch_rope_qkv_append(float* q, const float* k, const float* v, void* kcache, void* vcache, int cache_dtype,
 	                            const int* past_dev, size_t m, size_t n_head, size_t n_kv_head, size_t head_dim,
 	                            size_t rope_dims, const float* cos_t, const float* sin_t, hipStream_t s);
+	bool attn_step_fusable(const float* q, const float* k, const float* v, const void* kcache, const void* vcache,
+	                       size_t head_dim, size_t rope_dims, const float* cos_t, const float* sin_t);
+	void launch_attn_step(const float* q, const float* k, const float* v, void* kcache, void* vcache, int cache_dtype,
+	                      const int* past_dev, size_t n_head, size_t n_kv_head, size_t head_dim, size_t rope_dims,
+	                      const float* cos_t, const float* sin_t, float* out, size_t splits, float* partial,
+	                      int* counters, hipStream_t s);
 	size_t attn_splits(size_t m, size_t max_len, size_t n_head);
 	size_t attn_partial_floats(size_t m, size_t n_head, size_t head_dim, size_t splits);
 	void launch_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
@@ -252,10 +258,19 @@ namespace
 				group(m, j - i, qkv + i, qkv_out + i, m->x, nullptr, L.attn_norm, false, s);
 				i = j;
 			}
-			launch_rope_qkv_append(m->q, m->k, m->v, L.kcache, L.vcache, m->p.kv_dtype, past_dev, 1, H, KH, hd,
-			                       m->p.rope_dimension_count, m->cos_t, m->sin_t, s);
-			launch_attn_decode(m->q, L.kcache, L.vcache, m->p.kv_dtype, 1, past_dev, 0, H, KH, hd, m->attn,
-			                   m->attn_splits, m->attn_partial, m->attn_counters, s);
+			const size_t rope_dims = m->p.rope_dimension_count;
+			if (attn_step_fusable(m->q, m->k, m->v, L.kcache, L.vcache, hd, rope_dims, m->cos_t, m->sin_t))
+			{
+				launch_attn_step(m->q, m->k, m->v, L.kcache, L.vcache, m->p.kv_dtype, past_dev, H, KH, hd, rope_dims,
+				                 m->cos_t, m->sin_t, m->attn, m->attn_splits, m->attn_partial, m->attn_counters, s);
+			}
+			else
+			{
+				launch_rope_qkv_append(m->q, m->k, m->v, L.kcache, L.vcache, m->p.kv_dtype, past_dev, 1, H, KH, hd,
+				                       rope_dims, m->cos_t, m->sin_t, s);
+				launch_attn_decode(m->q, L.kcache, L.vcache, m->p.kv_dtype, 1, past_dev, 0, H, KH, hd, m->attn,
+				                   m->attn_splits, m->attn_partial, m->attn_counters, s);
+			}
 			const Weight* wo[1] = { &L.wo };
 			float* xo[1] = { m->x };
 			group(m, 1, wo, xo, m->attn, m->x, nullptr, false, s); // x = x + attn . Wo
