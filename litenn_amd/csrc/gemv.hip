@@ -22,6 +22,7 @@
 //     is issued: a mask produces the operand of v_fma_mix_f32.
 #include "common.hpp"
 
+#include <algorithm>
 #include <cstdlib>
 
 namespace litenn_hip
@@ -550,8 +551,8 @@ namespace litenn_hip
 		constexpr int kMaxRowsPerWave = 64; // rows a wavefront of the register kernel may own
 		constexpr int kLdsUnitStride = 68;  // floats between the staged activations of consecutive units
 		constexpr int kXPerThread = 8;      // most 128-bit activation loads a thread issues while staging
-		constexpr int kMaxStreamRows = 8;   // most rows a wavefront of the streaming kernel owns
-		constexpr int kPrefetchRows = 3;    // rows in flight ahead of the row being consumed
+		constexpr int kMaxStreamRows = 64;  // most rows a wavefront of the streaming kernel owns (one per lane)
+		constexpr int kPrefetchRows = 3;    // rows a wavefront keeps in flight (= its LDS row slots)
 		constexpr size_t kStreamLdsLimit = 160 * 1024;
 
 #ifdef LITENN_GEMV_TRACE
@@ -568,14 +569,15 @@ namespace litenn_hip
 		// ------------------------------------------------------------------
 		// Streaming kernel: rows go HBM -> LDS with direct, fully coalesced 128-bit loads.
 		//
-		// Each wavefront owns RB consecutive rows of one 4096-wide slice and keeps kPrefetchRows of
-		// them in flight: consecutive lanes fetch consecutive 16-byte chunks, every cache line is
-		// consumed by one instruction and nothing passes through registers.  It walks the rows in
-		// order: wait until row r has landed (vmcnt), let every lane pull its unit out of LDS,
-		// unpack, multiply-accumulate against the activations held in registers, reduce across the
-		// wavefront, then request row r + kPrefetchRows.  All wavefronts advance at the same pace, so
-		// rows arrive in the order they are consumed and only the last row's arithmetic is exposed
-		// after the last byte has arrived.
+		// Each wavefront owns a run of consecutive rows of one 4096-wide slice and keeps
+		// kPrefetchRows of them in flight, each in its own LDS slot: consecutive lanes fetch
+		// consecutive 16-byte chunks, every cache line is consumed by one instruction and nothing
+		// passes through registers.  It walks the rows in order: wait until row r has landed
+		// (vmcnt), let every lane pull its unit out of LDS, unpack, multiply-accumulate against the
+		// activations held in registers, reduce across the wavefront, then request row
+		// r + kPrefetchRows into the slot just emptied.  The run length is a launch parameter, so a
+		// launch is always one round of workgroups (at most one per CU) however many rows there
+		// are: the start-up (activations to LDS to registers) is paid once per CU.
 		//
 		// One launch can serve the operator groups of the decoder block that share an input:
 		//   * up to three matrices of one format over the same x (q/k/v projections): their rows
@@ -586,7 +588,7 @@ namespace litenn_hip
 		//   * SwiGLU: gate and up rows interleaved, the epilogue writes silu(gate) * up;
 		//   * a residual added to the output.
 		//
-		// LDS (dynamic): [staged activations][nwaves x RB row slots of kSliceBytes][slice partials]
+		// LDS (dynamic): [staged activations][nwaves x kPrefetchRows row slots of kSliceBytes][slice partials]
 		// [norm partial sums].
 		// ------------------------------------------------------------------
 		struct GemvArgs
@@ -602,6 +604,7 @@ namespace litenn_hip
 			int k;
 			uint32_t row_bytes;
 			int slices, groups;
+			int rows_per_group;    // consecutive rows one wavefront group walks (<= 64)
 			int silu_mul;          // 1: w[0] = gate, w[1] = up, row 2i + m; y[0][i] = silu(gate_i) * up_i
 		};
 
@@ -627,43 +630,47 @@ namespace litenn_hip
 			}
 		}
 
-		// Row R has landed once only the loads of the rows issued after it are outstanding: that
-		// is min(PD - 1, RB - 1 - R) rows of `loads_per_row` instructions (uniform over the wavefront).
-		template <int RB, int PD, int R>
-		__device__ __forceinline__ void wait_row_landed(int loads_per_row)
+		// vmcnt wait until at most ROWS rows of `loads_per_row` (1 .. 5, wavefront-uniform) load
+		// instructions are outstanding
+		template <int ROWS>
+		__device__ __forceinline__ void wait_rows_outstanding(int loads_per_row)
 		{
-			constexpr int kYounger = (PD - 1) < (RB - 1 - R) ? (PD - 1) : (RB - 1 - R);
-			switch (loads_per_row)
+			if constexpr (ROWS == 0)
 			{
-			case 1: vm_wait<kYounger * 1>(); break;
-			case 2: vm_wait<kYounger * 2>(); break;
-			case 3: vm_wait<kYounger * 3>(); break;
-			case 4: vm_wait<kYounger * 4>(); break;
-			default: vm_wait<kYounger * 5>(); break;
+				vm_wait<0>();
+			}
+			else
+			{
+				switch (loads_per_row)
+				{
+				case 1: vm_wait<ROWS * 1>(); break;
+				case 2: vm_wait<ROWS * 2>(); break;
+				case 3: vm_wait<ROWS * 3>(); break;
+				case 4: vm_wait<ROWS * 4>(); break;
+				default: vm_wait<ROWS * 5>(); break;
+				}
 			}
 		}
 
-		template <int RB, int PD, int R>
-		struct RowLoop
+		template <int MAX>
+		__device__ __forceinline__ void wait_rows_outstanding_dyn(int rows, int loads_per_row)
 		{
-			template <typename I, typename F>
-			static __device__ __forceinline__ void run(int loads_per_row, I&& issue, F&& body)
+			if constexpr (MAX == 0)
 			{
-				wait_row_landed<RB, PD, R>(loads_per_row);
-				body(R);
-				if constexpr (R + PD < RB)
-				{
-					issue(R + PD);
-				}
-				RowLoop<RB, PD, R + 1>::run(loads_per_row, issue, body);
+				vm_wait<0>();
 			}
-		};
-		template <int RB, int PD>
-		struct RowLoop<RB, PD, RB>
-		{
-			template <typename I, typename F>
-			static __device__ __forceinline__ void run(int, I&&, F&&) {}
-		};
+			else
+			{
+				if (rows >= MAX)
+				{
+					wait_rows_outstanding<MAX>(loads_per_row);
+				}
+				else
+				{
+					wait_rows_outstanding_dyn<MAX - 1>(rows, loads_per_row);
+				}
+			}
+		}
 
 		template <int Ctrl, int RowMask>
 		__device__ __forceinline__ double dpp_f64(double x)
@@ -699,7 +706,7 @@ namespace litenn_hip
 			return __fmul_rn(__fmul_rn(g, sig), u);
 		}
 
-		template <typename U, int RB, int XP>
+		template <typename U, int XP>
 		__global__ __launch_bounds__(512) void gemv_stream_kernel(const GemvArgs a)
 		{
 			constexpr int PD = kPrefetchRows;
@@ -719,11 +726,12 @@ namespace litenn_hip
 			const bool active = unit < units_per_row;
 			const int nwaves = slices * groups;
 			const uint32_t x_bytes = static_cast<uint32_t>(units_per_row) * kLdsUnitStride * 4u;
-			const uint32_t rows_base = x_bytes + static_cast<uint32_t>(wave) * (RB * U::kSliceBytes);
-			const uint32_t part_base = x_bytes + static_cast<uint32_t>(nwaves) * (RB * U::kSliceBytes);
-			const uint32_t norm_base = part_base + static_cast<uint32_t>(nwaves) * RB * 4u;
-			const int row0 = (blockIdx.x * groups + g) * RB;
-			const int count = max(0, min(RB, a.n_total - row0));
+			const int rpg = a.rows_per_group;
+			const uint32_t rows_base = x_bytes + static_cast<uint32_t>(wave) * (PD * U::kSliceBytes);
+			const uint32_t part_base = x_bytes + static_cast<uint32_t>(nwaves) * (PD * U::kSliceBytes);
+			const uint32_t norm_base = part_base + ((static_cast<uint32_t>(nwaves * rpg) * 4u + 7u) & ~7u);
+			const int row0 = (blockIdx.x * groups + g) * rpg;
+			const int count = max(0, min(rpg, a.n_total - row0));
 			const uint32_t slice_off = static_cast<uint32_t>(s) * U::kSliceBytes;
 			const uint32_t slice_len = min(static_cast<uint32_t>(U::kSliceBytes), a.row_bytes - slice_off);
 			const int loads_per_row = static_cast<int>((slice_len + 1023u) >> 10);
@@ -751,15 +759,32 @@ namespace litenn_hip
 				}
 			}
 
-			// 2. the first rows of the wavefront, straight into their LDS slots.  Rows past the end
-			// re-read the last row so that the number of loads in flight is the same for every
-			// wavefront (the waits count them).
-			auto issue_row = [&](int r) {
-				int m, local;
-				locate_row(a, min(row0 + r, a.n_total - 1), m, local);
-				const uint8_t* wm = m == 0 ? a.w[0] : (m == 1 ? a.w[1] : a.w[2]);
-				const uint8_t* grow = wm + static_cast<size_t>(local) * a.row_bytes + slice_off;
-				uint8_t* slot = smem_b + rows_base + r * U::kSliceBytes;
+			// 2. the first rows of the wavefront, straight into their LDS slots
+			// The rows are requested strictly in order, so a cursor walks them: `next_a` is the row
+			// about to be requested; with gate/up pairing `next_b` is the one after it and the two
+			// swap roles after every request; otherwise the cursor hops to the next matrix when the
+			// current one runs out.
+			const uint8_t* next_a;
+			const uint8_t* next_b = nullptr;
+			int cursor_m = 0, cursor_left = 0;
+			{
+				int local = 0;
+				locate_row(a, min(row0, a.n_total - 1), cursor_m, local);
+				if (a.silu_mul)
+				{
+					next_a = a.w[0] + static_cast<size_t>(local) * a.row_bytes + slice_off; // row0 is even
+					next_b = a.w[1] + static_cast<size_t>(local) * a.row_bytes + slice_off;
+				}
+				else
+				{
+					const uint8_t* wm = cursor_m == 0 ? a.w[0] : (cursor_m == 1 ? a.w[1] : a.w[2]);
+					next_a = wm + static_cast<size_t>(local) * a.row_bytes + slice_off;
+					cursor_left = a.n[cursor_m] - local;
+				}
+			}
+			auto issue_row = [&](uint32_t slot_off) {
+				const uint8_t* grow = next_a;
+				uint8_t* slot = smem_b + rows_base + slot_off;
 #pragma unroll
 				for (int i = 0; i < kLoadsPerRowMax; ++i)
 				{
@@ -773,24 +798,33 @@ namespace litenn_hip
 						}
 					}
 				}
+				next_a += a.row_bytes;
+				if (a.silu_mul)
+				{
+					const uint8_t* t = next_a;
+					next_a = next_b;
+					next_b = t;
+				}
+				else if (--cursor_left == 0 && cursor_m < 2)
+				{
+					++cursor_m;
+					next_a = (cursor_m == 1 ? a.w[1] : a.w[2]) + slice_off;
+					cursor_left = a.n[cursor_m];
+				}
 			};
-			constexpr int kFirstRows = RB < PD ? RB : PD;
+			const int first_rows = min(count, PD);
 #pragma unroll
-			for (int r = 0; r < kFirstRows; ++r)
+			for (int r = 0; r < PD; ++r)
 			{
-				issue_row(r);
+				if (r < first_rows) // uniform
+				{
+					issue_row(static_cast<uint32_t>(r) * U::kSliceBytes);
+				}
 			}
 
 			// 3. activations into LDS as soon as THEY have arrived (the rows issued after them stay
 			// in flight; the activation registers are only read after this wait)
-			switch (loads_per_row)
-			{
-			case 1: vm_wait<kFirstRows * 1>(); break;
-			case 2: vm_wait<kFirstRows * 2>(); break;
-			case 3: vm_wait<kFirstRows * 3>(); break;
-			case 4: vm_wait<kFirstRows * 4>(); break;
-			default: vm_wait<kFirstRows * 5>(); break;
-			}
+			wait_rows_outstanding_dyn<PD>(first_rows, loads_per_row);
 			if (fuse_norm)
 			{
 				// RMSNorm with f64 accumulation (ComputePrimitives.h:792-817): every workgroup sums
@@ -892,16 +926,44 @@ namespace litenn_hip
 			const typename U::Prep pz = U::prep(xr);
 			GEMV_TRACE(3);
 
-			// 5. rows in arrival order; lane r keeps the total of row row0 + r
+			// 5. rows in arrival order; lane r keeps the total of row row0 + r.  Row r has landed
+			// once only the rows issued after it are outstanding: min(PD - 1, count - 1 - r) rows of
+			// `loads_per_row` instructions.  The slot is refilled only after the lanes' LDS reads of
+			// it have returned (unit_dot consumes them before the refill is issued).
 			const uint32_t lane_p = lds0 + rows_base + U::lds_lane_offset(lane);
 			float res = 0.0f;
-			RowLoop<RB, PD, 0>::run(loads_per_row, issue_row, [&](int r) {
-				GEMV_TRACE(4 + r);
-				const typename U::Raw raw = unit_lds_load<U>(lane_p + static_cast<uint32_t>(r) * U::kSliceBytes, lane);
+			uint32_t slot_off = 0;
+			auto consume = [&](int r) {
+#ifdef LITENN_GEMV_TRACE
+				if (r < 11)
+				{
+					GEMV_TRACE(4 + r);
+				}
+#endif
+				const typename U::Raw raw = unit_lds_load<U>(lane_p + slot_off, lane);
 				const float p = active ? unit_dot<U>(raw, xr, pz, unit) : 0.0f;
 				const float total = wave_sum(p);
 				res = (lane == r) ? total : res;
-			});
+			};
+			// A loop rather than straight-line code per row: in a decoder every launch meets a cold
+			// instruction cache, and the unrolled form (16 KB and more) measured slower there.
+			int r = 0;
+			for (; r + PD <= count; ++r) // steady state: PD - 1 younger rows stay in flight
+			{
+				wait_rows_outstanding<PD - 1>(loads_per_row);
+				consume(r);
+				if (r + PD < count)
+				{
+					issue_row(slot_off);
+				}
+				slot_off = slot_off + U::kSliceBytes == PD * U::kSliceBytes ? 0u : slot_off + U::kSliceBytes;
+			}
+			for (; r < count; ++r) // the last rows: nothing left to request
+			{
+				wait_rows_outstanding_dyn<PD - 2>(count - 1 - r, loads_per_row);
+				consume(r);
+				slot_off = slot_off + U::kSliceBytes == PD * U::kSliceBytes ? 0u : slot_off + U::kSliceBytes;
+			}
 			GEMV_TRACE(15);
 
 			// 6. slices of one row meet in LDS; afterwards thread t of the workgroup holds row
@@ -910,22 +972,22 @@ namespace litenn_hip
 			bool have = lane < count;
 			if (slices > 1)
 			{
-				if (lane < RB)
+				if (lane < rpg)
 				{
-					lds_wr32(lds0 + part_base + static_cast<uint32_t>((s * groups + g) * RB + lane) * 4u, res);
+					lds_wr32(lds0 + part_base + static_cast<uint32_t>((s * groups + g) * rpg + lane) * 4u, res);
 				}
 				lds_barrier();
 				const int t = threadIdx.x;
-				vr = blockIdx.x * groups * RB + t;
-				have = t < groups * RB && vr < a.n_total;
+				vr = blockIdx.x * groups * rpg + t;
+				have = t < groups * rpg && vr < a.n_total;
 				res = 0.0f;
 				if (have)
 				{
-					const int gg = t / RB, rl = t % RB;
+					const int gg = t / rpg, rl = t % rpg;
 					for (int ss = 0; ss < slices; ++ss)
 					{
 						float v = __uint_as_float(
-						    lds_rd32<0>(lds0 + part_base + static_cast<uint32_t>((ss * groups + gg) * RB + rl) * 4u));
+						    lds_rd32<0>(lds0 + part_base + static_cast<uint32_t>((ss * groups + gg) * rpg + rl) * 4u));
 						lds_wait(v);
 						res += v;
 					}
@@ -933,8 +995,8 @@ namespace litenn_hip
 			}
 			if (a.silu_mul)
 			{
-				// even lanes hold gate_i, their odd neighbours up_i (row 2i + m); RB and every block
-				// origin are even, so pairs never straddle wavefronts
+				// even lanes hold gate_i, their odd neighbours up_i (row 2i + m); the run length and
+				// every block origin are even, so pairs never straddle wavefronts
 				const float other = dpp_f32<0xB1>(res); // quad_perm [1,0,3,2]
 				if (have && (vr & 1) == 0)
 				{
@@ -1204,35 +1266,14 @@ namespace litenn_hip
 			return cus;
 		}
 
-		template <typename U, int RB, int XP>
-		void launch_stream_variant(const GemvArgs& a, size_t lds, hipStream_t stream)
+		template <typename U, int XP>
+		void launch_stream_variant(const GemvArgs& a, int blocks, size_t lds, hipStream_t stream)
 		{
 			static const hipError_t attr =
-			    hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_stream_kernel<U, RB, XP>),
+			    hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_stream_kernel<U, XP>),
 			                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kStreamLdsLimit));
 			(void)attr;
-			const int rows_per_block = a.groups * RB;
-			const int blocks = (a.n_total + rows_per_block - 1) / rows_per_block;
-			gemv_stream_kernel<U, RB, XP><<<dim3(blocks), dim3(64 * a.slices * a.groups), lds, stream>>>(a);
-		}
-
-		template <typename U, int RB>
-		void launch_stream_rows(const GemvArgs& a, size_t lds, hipStream_t stream)
-		{
-			const int threads = 64 * a.slices * a.groups;
-			const int per_thread = (a.k / 4 + threads - 1) / threads; // 128-bit activation loads per thread
-			if (per_thread <= 2)
-			{
-				launch_stream_variant<U, RB, 2>(a, lds, stream);
-			}
-			else if (per_thread <= 4)
-			{
-				launch_stream_variant<U, RB, 4>(a, lds, stream);
-			}
-			else
-			{
-				launch_stream_variant<U, RB, kXPerThread>(a, lds, stream);
-			}
+			gemv_stream_kernel<U, XP><<<dim3(blocks), dim3(64 * a.slices * a.groups), lds, stream>>>(a);
 		}
 
 		// Returns false when the shape does not fit the streaming kernel.
@@ -1262,51 +1303,46 @@ namespace litenn_hip
 			{
 				return false;
 			}
-			// Rows per wavefront: the workgroups of one launch should fill the CUs once (a second,
-			// partial round costs a whole start-up), then as few rows as possible.
+			// Rows per wavefront group: one round of workgroups, at most one per CU, every group
+			// walking the same number of rows (even when gate/up rows are paired).
 			const size_t x_bytes = sizeof(float) * (static_cast<size_t>(k) / 64) * kLdsUnitStride;
-			auto lds_for = [&](int r) {
-				return x_bytes + static_cast<size_t>(nwaves) * r * U::kSliceBytes + sizeof(float) * nwaves * r +
-				       sizeof(double) * nwaves;
-			};
 			static const int forced_rows = env_int("LITENN_HIP_GEMV_ROWS", 0);
 			const int cus = compute_units();
-			int best = 0;
-			double best_cost = 0.0;
-			for (int r = 1; r <= kMaxStreamRows; ++r)
+			int rows = (a.n_total + cus * a.groups - 1) / (cus * a.groups);
+			if (forced_rows > 0)
 			{
-				if ((a.silu_mul && (r & 1)) || lds_for(r) > kStreamLdsLimit)
-				{
-					continue;
-				}
-				const int blocks = (a.n_total + a.groups * r - 1) / (a.groups * r);
-				const double rounds = static_cast<double>((blocks + cus - 1) / cus);
-				const double cost = rounds * (3.0 + 0.75 * r);
-				if (forced_rows == r || best == 0 || (forced_rows == 0 && cost < best_cost))
-				{
-					best = r;
-					best_cost = cost;
-					if (forced_rows == r)
-					{
-						break;
-					}
-				}
+				rows = forced_rows;
 			}
-			if (best == 0)
+			rows = std::min(std::max(rows, 1), kMaxStreamRows);
+			if (a.silu_mul && (rows & 1))
+			{
+				++rows;
+			}
+			a.rows_per_group = rows;
+			const int blocks = (a.n_total + a.groups * rows - 1) / (a.groups * rows);
+			const size_t lds = x_bytes + static_cast<size_t>(nwaves) * kPrefetchRows * U::kSliceBytes +
+			                   ((sizeof(float) * nwaves * rows + 7) & ~size_t{ 7 }) + sizeof(double) * nwaves;
+			if (lds > kStreamLdsLimit)
 			{
 				return false;
 			}
-			const size_t lds = lds_for(best);
-			switch (best)
+			// more than half of the CU's LDS: the dispatcher cannot stack two of these workgroups
+			// on one CU while another CU has none
+			static const int exclusive = env_int("LITENN_HIP_GEMV_EXCLUSIVE", 1);
+			const size_t lds_request = exclusive ? std::max(lds, kStreamLdsLimit / 2 + 1024) : lds;
+			const int threads = 64 * nwaves;
+			const int per_thread = (k / 4 + threads - 1) / threads; // 128-bit activation loads per thread
+			if (per_thread <= 2)
 			{
-			case 1: launch_stream_rows<U, 1>(a, lds, stream); break;
-			case 2: launch_stream_rows<U, 2>(a, lds, stream); break;
-			case 3: launch_stream_rows<U, 3>(a, lds, stream); break;
-			case 4: launch_stream_rows<U, 4>(a, lds, stream); break;
-			case 5: launch_stream_rows<U, 5>(a, lds, stream); break;
-			case 6: launch_stream_rows<U, 6>(a, lds, stream); break;
-			case 7: launch_stream_rows<U, 7>(a, lds, stream); break;
-			default: launch_stream_rows<U, 8>(a, lds, stream); break;
+				launch_stream_variant<U, 2>(a, blocks, lds_request, stream);
+			}
+			else if (per_thread <= 4)
+			{
+				launch_stream_variant<U, 4>(a, blocks, lds_request, stream);
+			}
+			else
+			{
+				launch_stream_variant<U, kXPerThread>(a, blocks, lds_request, stream);
 			}
 			return true;
 		}
