@@ -24,6 +24,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+# HBM bytes one launch of the headline GEMV moves, from the profiler's FETCH_SIZE / WRITE_SIZE
+# counters scaled by a known-size copy (profiles/gemv_q4_k_14336x4096_hbm_traffic.txt); it is a
+# property of the kernel and the shape, not re-measured by this script.
+GEMV_Q4_K_14336x4096_TRAFFIC_BYTES = 33330557
 
 
 def log(*a):
@@ -83,6 +87,22 @@ def bench_gemv(ln, hiprt, fmt, n, k, steps, warmup, n_buffers, seed=1):
         w.free()
     stream.destroy()
     return event_ms / steps, wall_ms / steps
+
+
+def traffic_probe(ln, launches=8, n_elems=16 * 1024 * 1024):
+    """A streaming kernel of known HBM traffic for calibrating the profiler's FETCH_SIZE /
+    WRITE_SIZE counters: element-wise negation of 64 MiB of f32 (reads 64 MiB, writes 64 MiB
+    per launch, far beyond the 4 MiB-per-XCD L2).  Only run under `--traffic-probe`."""
+    from litenn_amd.formats import DT_F32
+    src = ln.Tensor.from_numpy(np.ones(n_elems, np.float32))
+    dst = ln.Tensor((n_elems,))
+    for _ in range(launches):
+        ln.DeviceTraits.DoUnaryOp(ln.HIP(0), 0, dst.ptr, DT_F32, (n_elems,), src.ptr)  # 0 = Negate
+    assert float(dst.numpy()[12345]) == -1.0
+    src.free()
+    dst.free()
+    log(f"[bench] traffic probe: {launches} launches of unary_kernel<float>, {4 * n_elems} B read + "
+        f"{4 * n_elems} B written each")
 
 
 def bench_cpu_baseline(fmt, n, k, budget_s=12.0):
@@ -146,6 +166,8 @@ def main() -> int:
     ap.add_argument("--decode-prompt", type=int, default=128, help="prompt length of the decode run")
     ap.add_argument("--decode-new", type=int, default=256, help="tokens generated by the decode run")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also launch a known-size streaming kernel (profiler counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has nothing sharded or exchanged between GPUs; "
@@ -160,6 +182,9 @@ def main() -> int:
         print("bench.py needs a HIP device", file=sys.stderr)
         return 1
     log("[bench]", ln.DeviceTraits.Info(ln.HIP(0)))
+
+    if args.traffic_probe:
+        traffic_probe(ln)
 
     n, k = 14336, 4096
     algo_bytes = n * row_bytes(Q4_K, k) + 4 * k + 4 * n
@@ -190,8 +215,10 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-            "kernel": "gemv_kernel<Q4_KUnit>",
+            "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": GEMV_Q4_K_14336x4096_TRAFFIC_BYTES,
+            "traffic_unit": "bytes/launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
+            "algorithmic_bytes": algo_bytes,
+            "kernel": "gemv_stream_kernel<Q4_KUnit, 2>",
         },
     }
     if not args.no_cpu:
