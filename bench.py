@@ -105,6 +105,66 @@ def traffic_probe(ln, launches=8, n_elems=16 * 1024 * 1024):
         f"{4 * n_elems} B written each")
 
 
+FP16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 matrix rate
+
+
+def bench_gemm(ln, hiprt, fmt, n, k, m, iters=40, n_buffers=8, seed=7):
+    """Prefill matmul Y[m,n] = X[m,k] . deq(W)^T on the matrix cores, rotating weight buffers;
+    returns the HIP-event time per call in ms (the fp16 pre-pass of X included)."""
+    from litenn_amd import synth
+    from litenn_amd._lib import Exec, check, load
+    import ctypes as C
+
+    lib = load()
+    wq_host = synth.quant_weights(fmt, n, k, seed)
+    weights = [ln.Tensor.from_numpy(np.roll(wq_host, b, axis=0).reshape(-1)) for b in range(n_buffers)]
+    x = ln.Tensor.from_numpy(synth.activations(m, k, seed + 1))
+    y = ln.Tensor((m, n))
+    ws_bytes = lib.litenn_hip_mul_mat_q_workspace_bytes(m, k)
+    ws = ln.Tensor((ws_bytes // 4,))
+    stream = hiprt.Stream()
+    opts = Exec(stream.handle, 0)
+
+    def launch(i):
+        check(lib.litenn_hip_mul_mat_q_ws(0, fmt, weights[i % n_buffers].ptr, n, k, x.ptr, 0, m, y.ptr, None, 0,
+                                          ws.ptr, ws_bytes, C.byref(opts)))
+
+    for i in range(n_buffers):
+        launch(i)
+    stream.synchronize()
+    e0, e1 = hiprt.Event(), hiprt.Event()
+    e0.record(stream)
+    for i in range(iters):
+        launch(i)
+    e1.record(stream)
+    stream.synchronize()
+    ms = e0.elapsed_ms(e1) / iters
+    assert np.all(np.isfinite(y.numpy()))
+    for w in weights:
+        w.free()
+    for t in (x, y, ws):
+        t.free()
+    stream.destroy()
+    return ms
+
+
+def bench_prefill_gemm(ln, hiprt):
+    from litenn_amd.formats import Q4_K, Q6_K, row_bytes
+    out = []
+    for name, fmt, n, k in (("Q4_K", Q4_K, 14336, 4096), ("Q6_K", Q6_K, 4096, 4096)):
+        for m in (16, 64, 512):
+            ms = bench_gemm(ln, hiprt, fmt, n, k, m)
+            flops = 2.0 * m * n * k
+            bytes_ = n * row_bytes(fmt, k) + 4 * m * k + 4 * m * n
+            out.append({"format": name, "m": m, "n": n, "k": k, "us": round(ms * 1e3, 2),
+                        "tflops": round(flops / (ms * 1e-3) / 1e12, 1),
+                        "frac_of_fp16_mfma_peak": round(flops / (ms * 1e-3) / 1e12 / FP16_MFMA_PEAK_TFLOPS, 4),
+                        "gbps": round(bytes_ / (ms * 1e-3) / 1e9, 1)})
+            log(f"[bench] GEMM {name} M={m} N={n} K={k}: {ms * 1e3:.1f} us, {out[-1]['tflops']} TFLOP/s, "
+                f"{out[-1]['gbps']} GB/s")
+    return out
+
+
 def bench_cpu_baseline(fmt, n, k, budget_s=12.0):
     """The reference CPU path for the same GEMV, restated by the CPU checker: weights dequantised
     once to f32 [k, n] (the lowering's one-off cost, not timed), then the single-threaded i-k-j
@@ -166,6 +226,7 @@ def main() -> int:
     ap.add_argument("--decode-prompt", type=int, default=128, help="prompt length of the decode run")
     ap.add_argument("--decode-new", type=int, default=256, help="tokens generated by the decode run")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the prefill (batched matmul) measurements")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch a known-size streaming kernel (profiler counter calibration)")
     args = ap.parse_args()
@@ -231,6 +292,8 @@ def main() -> int:
             "ms_per_step": round(s_per_call * 1e3, 3),
         }
         log(f"[bench] CPU baseline: {s_per_call * 1e3:.1f} ms/call over {calls} calls")
+    if not args.no_gemm:
+        line["prefill_gemm"] = bench_prefill_gemm(ln, hiprt)
     if not args.no_decode:
         line["decode"] = bench_decode(ln, args.decode_prompt, args.decode_new)
         log(f"[bench] decode: {line['decode']['tokens_per_s']} tok/s")

@@ -122,11 +122,20 @@ int litenn_hip_permute(int dev, void* dst, int dtype, const size_t* src_shape, s
  * wq is the raw GGUF payload: n rows of k/block blocks.  x_dtype is F32.
  * residual (f32 [m, n]) may be NULL; when given, y = residual + x.W
  * (the Add at tools/gguf/LLaMABuilder.cpp:652-653,661-663).  residual may alias y.
- * m == 1..15 runs the streaming GEMV; m >= 16 runs the MFMA GEMM unless
- * LITENN_HIP_MATMUL_PRECISE is set in `flags`, which keeps f32 activations. */
+ * m == 1..15 runs the streaming GEMV.  m >= 16 (with k a multiple of 256) runs on the matrix
+ * cores: weights and activations are rounded to fp16 once each (activation rows are first scaled
+ * by a power of two into the fp16 range), products accumulate in f32; relative L2 error about
+ * 4e-4.  LITENN_HIP_MATMUL_PRECISE in `flags` keeps f32 operands (GEMV path) for any m.
+ * The matrix-core path needs a device workspace of litenn_hip_mul_mat_q_workspace_bytes(m, k):
+ * litenn_hip_mul_mat_q allocates and frees it itself (and therefore always synchronises for
+ * m >= 16); litenn_hip_mul_mat_q_ws takes the caller's (16-byte aligned; NULL = as above). */
 #define LITENN_HIP_MATMUL_PRECISE 1u
 int litenn_hip_mul_mat_q(int dev, int fmt, const void* wq, size_t n, size_t k, const void* x, int x_dtype, size_t m,
                          void* y, const void* residual, unsigned flags, const litenn_hip_exec* opts);
+size_t litenn_hip_mul_mat_q_workspace_bytes(size_t m, size_t k);
+int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t n, size_t k, const void* x, int x_dtype, size_t m,
+                            void* y, const void* residual, unsigned flags, void* workspace, size_t workspace_bytes,
+                            const litenn_hip_exec* opts);
 /* One activation row through an operator group of the decoder block, fused into a single
  * launch when the shape allows and composed from separate launches otherwise:
  *   [RMSNorm(x, norm_w, eps)] -> count (1..3) linears of one format sharing that input

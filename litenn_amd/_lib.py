@@ -50,6 +50,8 @@ SIGNATURES = {
     "litenn_hip_get_rows": [_i, _vp, _i, _szp, _sz, _vp, _i, _szp, _sz, _vp, _ex],
     "litenn_hip_permute": [_i, _vp, _i, _szp, _sz, _vp, _szp, _ex],
     "litenn_hip_mul_mat_q": [_i, _i, _vp, _sz, _sz, _vp, _i, _sz, _vp, _vp, _u, _ex],
+    "litenn_hip_mul_mat_q_workspace_bytes": [_sz, _sz],
+    "litenn_hip_mul_mat_q_ws": [_i, _i, _vp, _sz, _sz, _vp, _i, _sz, _vp, _vp, _u, _vp, _sz, _ex],
     "litenn_hip_linear_group": [_i, _i, _sz, C.POINTER(_vp), _szp, _sz, _vp, C.POINTER(_vp), _vp, _vp, _d, _u, _ex],
     "litenn_hip_dequantize": [_i, _i, _vp, _sz, _sz, _vp, _ex],
     "litenn_hip_get_rows_q": [_i, _i, _vp, _sz, _sz, _vp, _sz, _vp, _ex],
@@ -68,7 +70,7 @@ SIGNATURES = {
     "litenn_hip_llama_generate": [_vp, _vp, _sz, _sz, _vp, _u, C.POINTER(_d), C.POINTER(_d)],
     "litenn_hip_llama_get_kv": [_vp, _i, _vp, _vp],
 }
-_RESTYPES = {"litenn_hip_last_error": C.c_char_p}
+_RESTYPES = {"litenn_hip_last_error": C.c_char_p, "litenn_hip_mul_mat_q_workspace_bytes": C.c_size_t}
 
 _lib = None
 

@@ -13,8 +13,9 @@ namespace litenn_hip
 	// launchers defined in gemv.hip / gemm.hip / glue.hip
 	int launch_gemv(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
 	                const float* residual, hipStream_t stream);
-	int launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
-	                const float* residual, hipStream_t stream);
+	size_t gemm_scratch_halves(size_t m, size_t k);
+	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
+	                 const float* residual, void* scratch_halves, hipStream_t stream);
 	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
 	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
 	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream);
@@ -476,9 +477,21 @@ static bool is_weight_format(int fmt)
 	return block_elements(fmt) != 0;
 }
 
+extern "C" size_t litenn_hip_mul_mat_q_workspace_bytes(size_t m, size_t k)
+{
+	return m >= 16 ? 2 * gemm_scratch_halves(m, k) : 0;
+}
+
 extern "C" int litenn_hip_mul_mat_q(int dev, int fmt, const void* wq, size_t n, size_t k, const void* x, int x_dtype,
                                     size_t m, void* y, const void* residual, unsigned flags,
                                     const litenn_hip_exec* opts)
+{
+	return litenn_hip_mul_mat_q_ws(dev, fmt, wq, n, k, x, x_dtype, m, y, residual, flags, nullptr, 0, opts);
+}
+
+extern "C" int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t n, size_t k, const void* x,
+                                       int x_dtype, size_t m, void* y, const void* residual, unsigned flags,
+                                       void* workspace, size_t workspace_bytes, const litenn_hip_exec* opts)
 {
 	const char* action = "HIP quantized matmul";
 	if (!is_weight_format(fmt))
@@ -517,15 +530,38 @@ extern "C" int litenn_hip_mul_mat_q(int dev, int fmt, const void* wq, size_t n, 
 	const bool quant = fmt != LITENN_FMT_F16 && fmt != LITENN_FMT_F32;
 	if (m >= 16 && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && k % 256 == 0)
 	{
-		if (launch_gemm(fmt, wq, n, k, xf, m, yf, rf, s) != 0)
+		// the matrix-core path rounds the activations to fp16 into a workspace
+		const size_t need = 2 * gemm_scratch_halves(m, k);
+		if (workspace)
 		{
-			return 1;
+			if (workspace_bytes < need)
+			{
+				return fail(action, "workspace is smaller than litenn_hip_mul_mat_q_workspace_bytes(m, k)");
+			}
+			if (!launch_gemm(fmt, wq, n, k, xf, m, yf, rf, workspace, s))
+			{
+				launch_gemv(fmt, wq, n, k, xf, m, yf, rf, s);
+			}
+			return finish(action, opts);
 		}
+		// none given: this call owns one, and frees it after the stream has drained, whatever
+		// opts->synchronize says
+		void* scratch = nullptr;
+		LITENN_HIP_TRY(action, hipMalloc(&scratch, need));
+		if (!launch_gemm(fmt, wq, n, k, xf, m, yf, rf, scratch, s))
+		{
+			launch_gemv(fmt, wq, n, k, xf, m, yf, rf, s);
+		}
+		const hipError_t launched = hipGetLastError();
+		const hipError_t drained = hipStreamSynchronize(s);
+		(void)hipFree(scratch);
+		if (launched != hipSuccess || drained != hipSuccess)
+		{
+			return fail_hip(action, launched != hipSuccess ? launched : drained);
+		}
+		return 0;
 	}
-	else
-	{
-		launch_gemv(fmt, wq, n, k, xf, m, yf, rf, s);
-	}
+	launch_gemv(fmt, wq, n, k, xf, m, yf, rf, s);
 	return finish(action, opts);
 }
 

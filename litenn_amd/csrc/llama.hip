@@ -9,6 +9,7 @@
 // step captured once into a HIP graph so that a greedy loop never returns to the host.
 #include "common.hpp"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -18,8 +19,9 @@ namespace litenn_hip
 {
 	int launch_gemv(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
 	                const float* residual, hipStream_t stream);
-	int launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
-	                const float* residual, hipStream_t stream);
+	size_t gemm_scratch_halves(size_t m, size_t k);
+	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
+	                 const float* residual, void* scratch_halves, hipStream_t stream);
 	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
 	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
 	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream);
@@ -98,6 +100,7 @@ struct litenn_hip_llama
 	size_t cap_rows = 0, cap_logit_rows = 0;
 	float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *gate = nullptr,
 	      *gate2 = nullptr, *up = nullptr, *logits = nullptr;
+	void* xh = nullptr; // fp16 copy of a matmul's activations (multi-row path), 16-row padded
 	int32_t* d_tokens = nullptr;
 	int32_t* d_next = nullptr; // token produced by the last arg-max
 	int32_t* d_out = nullptr;  // generated tokens
@@ -132,6 +135,11 @@ namespace
 		{
 			(void)hipFree(m->d_tokens);
 			m->d_tokens = nullptr;
+		}
+		if (m->xh)
+		{
+			(void)hipFree(m->xh);
+			m->xh = nullptr;
 		}
 		m->cap_rows = 0;
 	}
@@ -168,6 +176,7 @@ namespace
 				LITENN_HIP_TRY(kAction, hipMalloc(reinterpret_cast<void**>(b.p), sizeof(float) * rows * b.n));
 			}
 			LITENN_HIP_TRY(kAction, hipMalloc(reinterpret_cast<void**>(&m->d_tokens), sizeof(int32_t) * rows));
+			LITENN_HIP_TRY(kAction, hipMalloc(&m->xh, 2 * gemm_scratch_halves(rows, std::max({ d, qw, ff }))));
 			m->cap_rows = rows;
 		}
 		if (logit_rows > m->cap_logit_rows)
@@ -202,18 +211,16 @@ namespace
 		return 0;
 	}
 
-	void matmul(const Weight& w, const float* x, size_t rows, float* y, const float* residual, unsigned flags,
-	            hipStream_t s)
+	void matmul(litenn_hip_llama* m, const Weight& w, const float* x, size_t rows, float* y, const float* residual,
+	            unsigned flags, hipStream_t s)
 	{
 		const bool quant = w.fmt != LITENN_FMT_F16 && w.fmt != LITENN_FMT_F32;
-		if (rows >= 16 && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && w.k % 256 == 0)
+		if (rows >= 16 && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && w.k % 256 == 0 &&
+		    launch_gemm(w.fmt, w.data, w.n, w.k, x, rows, y, residual, m->xh, s))
 		{
-			launch_gemm(w.fmt, w.data, w.n, w.k, x, rows, y, residual, s);
+			return;
 		}
-		else
-		{
-			launch_gemv(w.fmt, w.data, w.n, w.k, x, rows, y, residual, s);
-		}
+		launch_gemv(w.fmt, w.data, w.n, w.k, x, rows, y, residual, s);
 	}
 
 	// One operator group of the single-token step (see launch_linear_group).
@@ -317,24 +324,24 @@ namespace
 		for (Layer& L : m->layers)
 		{
 			launch_rmsnorm(m->x, L.attn_norm, m->p.rms_norm_epsilon, rows, d, m->xn, s);
-			matmul(L.wq, m->xn, rows, m->q, nullptr, flags, s);
-			matmul(L.wk, m->xn, rows, m->k, nullptr, flags, s);
-			matmul(L.wv, m->xn, rows, m->v, nullptr, flags, s);
+			matmul(m, L.wq, m->xn, rows, m->q, nullptr, flags, s);
+			matmul(m, L.wk, m->xn, rows, m->k, nullptr, flags, s);
+			matmul(m, L.wv, m->xn, rows, m->v, nullptr, flags, s);
 			launch_rope_qkv_append(m->q, m->k, m->v, L.kcache, L.vcache, m->p.kv_dtype, past_dev, rows, H, KH, hd,
 			                       m->p.rope_dimension_count, m->cos_t, m->sin_t, s);
 			launch_attn_decode(m->q, L.kcache, L.vcache, m->p.kv_dtype, rows, past_dev, 0, H, KH, hd, m->attn,
 			                   rows == 1 ? m->attn_splits : 1, m->attn_partial, m->attn_counters, s);
-			matmul(L.wo, m->attn, rows, m->x, m->x, flags, s); // x = x + attn . Wo
+			matmul(m, L.wo, m->attn, rows, m->x, m->x, flags, s); // x = x + attn . Wo
 			launch_rmsnorm(m->x, L.ffn_norm, m->p.rms_norm_epsilon, rows, d, m->xn, s);
-			matmul(L.gate, m->xn, rows, m->gate, nullptr, flags, s);
-			matmul(L.up, m->xn, rows, m->up, nullptr, flags, s);
+			matmul(m, L.gate, m->xn, rows, m->gate, nullptr, flags, s);
+			matmul(m, L.up, m->xn, rows, m->up, nullptr, flags, s);
 			launch_silu_mul(m->gate, m->up, m->gate, rows * ff, s);
-			matmul(L.down, m->gate, rows, m->x, m->x, flags, s); // x = x + mlp
+			matmul(m, L.down, m->gate, rows, m->x, m->x, flags, s); // x = x + mlp
 		}
 		const size_t first = rows - logit_rows;
 		launch_rmsnorm(m->x + first * d, m->output_norm, m->p.rms_norm_epsilon, logit_rows, d, m->xn, s);
 		const Weight& head = m->output.data ? m->output : m->tok_embd;
-		matmul(head, m->xn, logit_rows, m->logits, nullptr, flags, s);
+		matmul(m, head, m->xn, logit_rows, m->logits, nullptr, flags, s);
 	}
 
 	int check_error_flag(litenn_hip_llama* m)

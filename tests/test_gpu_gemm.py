@@ -1,0 +1,102 @@
+"""Parity of the batched quantised matmul (prefill, M >= 16, matrix cores) with the CPU checker,
+through the C ABI.
+
+Tolerance: relative L2 error <= 1e-3 on the output (the bar the benchmark definition states).
+The kernel rounds every dequantised weight and every activation to fp16 once and accumulates in
+f32, so the expected error is about 4e-4 (two independent roundings of relative RMS 2^-11/sqrt 3);
+a wrong element order, scale or sign gives errors of order 1."""
+import numpy as np
+import pytest
+
+from conftest import rel_l2
+from litenn_amd import synth
+from litenn_amd.formats import Q4_0, Q4_K, Q6_K, Q8_0, row_bytes
+from litenn_amd.llama import MATMUL_PRECISE
+from llama_util import hip_model, oracle_model
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+FORMATS = [Q4_0, Q8_0, Q4_K, Q6_K]
+
+
+def run_case(hip, oracle, fmt, m, n, k, seed=0, residual=False, rows=None, flags=0):
+    """rows: compare only these weight rows (they are independent), to bound the checker's time."""
+    wq = synth.quant_weights(fmt, n, k, seed, 1)
+    x = synth.activations(m, k, seed, 2)
+    res = synth.activations(m, n, seed, 3) if residual else None
+    y = hip.mul_mat_q(fmt, hip.Tensor.from_numpy(wq), n, k, hip.Tensor.from_numpy(x),
+                      residual=hip.Tensor.from_numpy(res) if residual else None, flags=flags).numpy()
+    assert y.shape == (m, n)
+    if rows is not None:
+        rb = row_bytes(fmt, k)
+        sub = np.ascontiguousarray(wq.reshape(n, rb)[rows]).reshape(-1)
+        ref = oracle.mul_mat_q(fmt, sub, len(rows), k, x)
+        y = y[:, rows]
+        if residual:
+            ref = res[:, rows] + ref
+    else:
+        ref = oracle.mul_mat_q(fmt, wq, n, k, x)
+        if residual:
+            ref = res + ref
+    return rel_l2(y, ref)
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("m,n,k", [(16, 64, 256), (16, 256, 512), (17, 100, 256), (33, 67, 768), (64, 512, 1024),
+                                   (100, 300, 2048), (133, 260, 512), (256, 1024, 256), (300, 96, 4096)])
+def test_gemm_matches_checker(hip, oracle, fmt, m, n, k):
+    err = run_case(hip, oracle, fmt, m, n, k, seed=m + n + k)
+    assert err <= TOL, err
+    assert err > 1e-6  # the fp16 path ran, not the f32 GEMV
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+def test_gemm_residual_and_precise_flag(hip, oracle, fmt):
+    assert run_case(hip, oracle, fmt, 48, 200, 512, seed=9, residual=True) <= TOL
+    # the flag keeps f32 activations (GEMV path): error drops to summation-order level
+    assert run_case(hip, oracle, fmt, 48, 200, 512, seed=9, flags=MATMUL_PRECISE) <= 1e-5
+
+
+@pytest.mark.parametrize("m", [16, 64, 512])
+def test_config3_q4_k_14336x4096(hip, oracle, m):
+    """BASELINE config 3: K=4096, N=14336 Q4_K at full size (a 768-row sample of N is checked)."""
+    rows = np.sort(np.random.default_rng(m).choice(14336, 768, replace=False))
+    rows[0], rows[-1] = 0, 14335
+    assert run_case(hip, oracle, Q4_K, m, 14336, 4096, seed=30 + m, rows=rows) <= TOL
+
+
+@pytest.mark.parametrize("m", [16, 64, 512])
+def test_config3_q6_k_4096x4096(hip, oracle, m):
+    """BASELINE config 3: K=4096, N=4096 Q6_K at full size (a 768-row sample of N is checked)."""
+    rows = np.sort(np.random.default_rng(m).choice(4096, 768, replace=False))
+    rows[0], rows[-1] = 0, 4095
+    assert run_case(hip, oracle, Q6_K, m, 4096, 4096, seed=40 + m, rows=rows) <= TOL
+
+
+def test_gemm_is_linear_in_x_at_full_size(hip):
+    """Size-independent property at the full north-star shape: Y(a x1 + x2) = a Y(x1) + Y(x2) up to
+    the fp16 rounding of the activations."""
+    n, k, m = 14336, 4096, 64
+    wq = hip.Tensor.from_numpy(synth.quant_weights(Q4_K, n, k, 5, 1))
+    x1, x2 = synth.activations(m, k, 5, 2), synth.activations(m, k, 5, 3)
+    y = lambda x: hip.mul_mat_q(Q4_K, wq, n, k, hip.Tensor.from_numpy(x)).numpy()
+    assert rel_l2(y(2.0 * x1 + x2), 2.0 * y(x1) + y(x2)) <= TOL
+
+
+@pytest.mark.parametrize("fmt", [Q4_0, Q4_K])
+def test_prefill_through_the_matrix_cores(hip, oracle, fmt):
+    """The runtime's multi-row pass with fp16 matmul operands: logits stay within the matmul bar
+    of the checker's f32 pass per layer (looser after three blocks), the cache matches, and decoding
+    continues from it."""
+    cfg = synth.tiny_llama(fmt, block_count=3, d_model=512, heads=4, kv_heads=2, ff=1024, vocab=777)
+    toks = synth.prompt_tokens(cfg, 40, 2)
+    ref = oracle_model(oracle, cfg, 2, kv_f16=True)
+    dev = hip_model(hip, cfg, 2)
+    want = ref.eval(toks[:32])
+    got = dev.eval(toks[:32], precise=False)
+    assert rel_l2(got, want) < 5e-3
+    kd, vd = dev.get_kv(2)
+    kr, vr = ref.get_kv(2)
+    assert rel_l2(kd, kr) < 5e-3 and rel_l2(vd, vr) < 5e-3
+    for t in toks[32:]:
+        assert rel_l2(dev.eval([t])[0], ref.eval([t])[0]) < 5e-3
