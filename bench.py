@@ -148,11 +148,14 @@ def bench_gemm(ln, hiprt, fmt, n, k, m, iters=40, n_buffers=8, seed=7):
     return ms
 
 
-def bench_prefill_gemm(ln, hiprt):
+def bench_prefill_gemm(ln, hiprt, only=None):
+    """only: "FORMAT:M" restricts the run to one case (profiling)."""
     from litenn_amd.formats import Q4_K, Q6_K, row_bytes
     out = []
     for name, fmt, n, k in (("Q4_K", Q4_K, 14336, 4096), ("Q6_K", Q6_K, 4096, 4096)):
         for m in (16, 64, 512):
+            if only and only != f"{name}:{m}":
+                continue
             ms = bench_gemm(ln, hiprt, fmt, n, k, m)
             flops = 2.0 * m * n * k
             bytes_ = n * row_bytes(fmt, k) + 4 * m * k + 4 * m * n
@@ -227,6 +230,7 @@ def main() -> int:
     ap.add_argument("--decode-new", type=int, default=256, help="tokens generated by the decode run")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill (batched matmul) measurements")
+    ap.add_argument("--gemm-case", default=None, help="run only this prefill case, e.g. Q4_K:512")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch a known-size streaming kernel (profiler counter calibration)")
     args = ap.parse_args()
@@ -293,7 +297,7 @@ def main() -> int:
         }
         log(f"[bench] CPU baseline: {s_per_call * 1e3:.1f} ms/call over {calls} calls")
     if not args.no_gemm:
-        line["prefill_gemm"] = bench_prefill_gemm(ln, hiprt)
+        line["prefill_gemm"] = bench_prefill_gemm(ln, hiprt, args.gemm_case)
     if not args.no_decode:
         line["decode"] = bench_decode(ln, args.decode_prompt, args.decode_new)
         log(f"[bench] decode: {line['decode']['tokens_per_s']} tok/s")

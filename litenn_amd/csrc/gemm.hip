@@ -10,7 +10,8 @@
 // range first (and its results scaled back), so the range of the activations does not matter;
 // LITENN_HIP_MATMUL_PRECISE selects the f32 GEMV path instead.
 //
-// Work split: a workgroup (4 wavefronts) owns 64 * NG weight rows and BM activation rows; a
+// Work split: a workgroup (WAVES wavefronts) owns 16 * WAVES * NG weight rows and BM activation
+// rows; a
 // wavefront owns NG groups of 16 weight rows and walks K in chunks of 256 (one K-quant
 // super-block, eight 32-element blocks).  Lane (r, g) = (lane % 16, lane / 16) decodes 64 of
 // the 256 elements of row r of each of its groups per chunk, eight per MFMA step, in whatever
@@ -34,7 +35,8 @@ namespace litenn_hip
 		typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 		constexpr int kChunk = 256;          // K elements per step of the outer loop
-		constexpr int kTileStride = 256 + 8; // halves per activation row in LDS (pad: 4 banks per row)
+		// halves per activation row in LDS: rows stay 16-byte aligned and shift by 4 banks each
+		constexpr int kTileStride = 256 + 8;
 
 		__device__ __forceinline__ uint32_t pack_f16(float a, float b)
 		{
@@ -60,6 +62,52 @@ namespace litenn_hip
 		// frag  : the 8 fp16 values of MFMA step s (0..7) as 4 packed dwords
 		// koff  : offsets (in elements, within the chunk) of the two runs of 4 activations
 		//         that pair with frag(s): elements 0..3 <-> k0 .. k0+3, 4..7 <-> k1 .. k1+3
+		//
+		// Small unsigned integers enter the arithmetic as binary16 SUBNORMALS: a 16-bit lane
+		// holding 0..1023 read as a half is exactly value * 2^-24, so a masked nibble or byte is a
+		// ready-made operand of v_fma_mix_f32 (half widened to f32 inside the multiply-add) and no
+		// integer -> float conversion is issued; the 2^24 rides in the f32 scale.
+
+		typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+		constexpr float kTwo24 = 16777216.0f, kTwo20 = 1048576.0f;
+
+		// lo16(pair) * scale + bias and hi16(pair) * scale + bias, halves taken as subnormal binary16
+		__device__ __forceinline__ void scale_pair(uint32_t pair, float scale, float bias, float& a, float& b)
+		{
+			const half2_t h = __builtin_bit_cast(half2_t, pair);
+			a = __builtin_fmaf(static_cast<float>(h.x), scale, bias);
+			b = __builtin_fmaf(static_cast<float>(h.y), scale, bias);
+		}
+
+		// One dword of packed nibbles -> 8 values: out[0..3] = low nibbles of bytes 0..3 (scale/bias
+		// lo), out[4..7] = high nibbles (scale/bias hi; the nibble sits 4 bits up, scale_hi carries
+		// 2^20 instead of 2^24)
+		__device__ __forceinline__ void nibbles8(uint32_t v, float s_lo, float b_lo, float s_hi, float b_hi,
+		                                          uint32_t (&out)[4])
+		{
+			const uint32_t t = v >> 8;
+			float f0, f1, f2, f3;
+			scale_pair(v & 0x000f000fu, s_lo, b_lo, f0, f2); // bytes 0, 2
+			scale_pair(t & 0x000f000fu, s_lo, b_lo, f1, f3); // bytes 1, 3
+			out[0] = pack_f16(f0, f1);
+			out[1] = pack_f16(f2, f3);
+			scale_pair(v & 0x00f000f0u, s_hi, b_hi, f0, f2);
+			scale_pair(t & 0x00f000f0u, s_hi, b_hi, f1, f3);
+			out[2] = pack_f16(f0, f1);
+			out[3] = pack_f16(f2, f3);
+		}
+
+		// One dword of unsigned bytes -> 4 values u * scale + bias as two packed dwords
+		__device__ __forceinline__ void bytes4(uint32_t v, float scale, float bias, uint32_t& p01, uint32_t& p23)
+		{
+			const uint32_t even = __builtin_amdgcn_perm(0u, v, 0x0c020c00u); // {b0, b2} as 16-bit lanes
+			const uint32_t odd = __builtin_amdgcn_perm(0u, v, 0x0c030c01u);  // {b1, b3}
+			float f0, f1, f2, f3;
+			scale_pair(even, scale, bias, f0, f2);
+			scale_pair(odd, scale, bias, f1, f3);
+			p01 = pack_f16(f0, f1);
+			p23 = pack_f16(f2, f3);
+		}
 
 		struct Q4_0Frag
 		{
@@ -90,23 +138,12 @@ namespace litenn_hip
 				}
 				return r.w[5 + t]; // bytes 20 + 4t ..
 			}
+			// (q - 8) * d: elements 4t .. 4t+3 (low nibbles) and 16 + 4t .. (high nibbles) of block b
 			static __device__ __forceinline__ void frag(const Raw& r, const Scale& sc, int s, uint32_t (&out)[4])
 			{
 				const int b = s >> 2, t = s & 3;
-				const uint32_t v = qs(r, b, t);
 				const float d = b == 0 ? sc.d0 : sc.d1;
-				float f[8];
-#pragma unroll
-				for (int e = 0; e < 4; ++e)
-				{
-					f[e] = (static_cast<float>((v >> (8 * e)) & 0xFu) - 8.0f) * d;         // element 4t + e
-					f[4 + e] = (static_cast<float>((v >> (8 * e + 4)) & 0xFu) - 8.0f) * d; // element 16 + 4t + e
-				}
-#pragma unroll
-				for (int i = 0; i < 4; ++i)
-				{
-					out[i] = pack_f16(f[2 * i], f[2 * i + 1]);
-				}
+				nibbles8(qs(r, b, t), d * kTwo24, -8.0f * d, d * kTwo20, -8.0f * d, out);
 			}
 			static __device__ __forceinline__ void koff(int g, int s, int& k0, int& k1)
 			{
@@ -152,19 +189,10 @@ namespace litenn_hip
 					lo = r.w[9 + 2 * t];
 					hi = r.w[10 + 2 * t];
 				}
+				// int8 q -> unsigned byte q + 128; the bias leaves through the -128 d term
 				const float d = b == 0 ? sc.d0 : sc.d1;
-				float f[8];
-#pragma unroll
-				for (int e = 0; e < 4; ++e)
-				{
-					f[e] = static_cast<float>(static_cast<int8_t>(lo >> (8 * e))) * d;
-					f[4 + e] = static_cast<float>(static_cast<int8_t>(hi >> (8 * e))) * d;
-				}
-#pragma unroll
-				for (int i = 0; i < 4; ++i)
-				{
-					out[i] = pack_f16(f[2 * i], f[2 * i + 1]);
-				}
+				bytes4(lo ^ 0x80808080u, d * kTwo24, -128.0f * d, out[0], out[1]);
+				bytes4(hi ^ 0x80808080u, d * kTwo24, -128.0f * d, out[2], out[3]);
 			}
 			static __device__ __forceinline__ void koff(int g, int s, int& k0, int& k1)
 			{
@@ -177,7 +205,7 @@ namespace litenn_hip
 		{
 			static constexpr int kChunkBytes = 144;
 			struct Raw { u32x4 h; uint32_t q[8]; }; // header (d, dmin, 12 scale bytes) + the 32 nibble bytes of group g
-			struct Scale { float s0, m0, s1, m1; }; // d*sc and dmin*m of sub-blocks 2g and 2g+1
+			struct Scale { float s0, m0, s1, m1; }; // d*sc*2^24, -dmin*m of sub-block 2g; d*sc*2^20, -dmin*m of 2g+1
 			static __device__ __forceinline__ Raw load(const uint8_t* chunk, int g)
 			{
 				Raw r;
@@ -188,50 +216,36 @@ namespace litenn_hip
 				r.q[4] = b.x, r.q[5] = b.y, r.q[6] = b.z, r.q[7] = b.w;
 				return r;
 			}
-			static __device__ __forceinline__ uint32_t scale_byte(const u32x4& h, int i) // byte i of scales[12]
-			{
-				const uint32_t w = i < 4 ? h.y : (i < 8 ? h.z : h.w);
-				return (w >> (8 * (i & 3))) & 0xffu;
-			}
-			static __device__ __forceinline__ void scale_min(const u32x4& h, int j, float& sc, float& mn)
-			{
-				uint32_t s, m;
-				if (j < 4)
-				{
-					s = scale_byte(h, j) & 63u;
-					m = scale_byte(h, j + 4) & 63u;
-				}
-				else
-				{
-					s = (scale_byte(h, j + 4) & 0xFu) | ((scale_byte(h, j - 4) >> 6) << 4);
-					m = (scale_byte(h, j + 4) >> 4) | ((scale_byte(h, j) >> 6) << 4);
-				}
-				sc = static_cast<float>(s);
-				mn = static_cast<float>(m);
-			}
+			// 6-bit (scale, min) of sub-blocks 2g and 2g+1 (get_scale_min_k4 of the ggml block
+			// definition): for g < 2 bytes 2g, 2g+1 (scales) and 2g+4, 2g+5 (mins) masked to 6 bits;
+			// for g >= 2 low/high nibbles of bytes 2g+4, 2g+5 with bits 6..7 of bytes 2g-4, 2g-3
+			// (scales) and 2g, 2g+1 (mins) on top.
 			static __device__ __forceinline__ Scale prep(const Raw& r, int g)
 			{
 				const float d = f16_bits_to_f32(r.h.x), dmin = f16_bits_to_f32(r.h.x >> 16);
-				float s0, m0, s1, m1;
-				scale_min(r.h, 2 * g, s0, m0);
-				scale_min(r.h, 2 * g + 1, s1, m1);
-				return { d * s0, dmin * m0, d * s1, dmin * m1 };
+				const int sh = (g & 1) * 16;
+				const uint32_t w0 = (r.h.y >> sh) & 0xffffu; // scale bytes 2g', 2g'+1 with g' = g & 1
+				const uint32_t w1 = (r.h.z >> sh) & 0xffffu; // bytes 4 + 2g', 5 + 2g'
+				const uint32_t w2 = (r.h.w >> sh) & 0xffffu; // bytes 8 + 2g', 9 + 2g'
+				uint32_t sc, mn; // two values each, in 16-bit... byte lanes 0 and 1
+				if (g < 2)
+				{
+					sc = w0 & 0x3f3fu;
+					mn = w1 & 0x3f3fu;
+				}
+				else
+				{
+					sc = (w2 & 0x0f0fu) | ((w0 >> 2) & 0x3030u);
+					mn = ((w2 >> 4) & 0x0f0fu) | ((w1 >> 2) & 0x3030u);
+				}
+				const float s0 = static_cast<float>(sc & 0xffu), s1 = static_cast<float>(sc >> 8);
+				const float m0 = static_cast<float>(mn & 0xffu), m1 = static_cast<float>(mn >> 8);
+				return { d * s0 * kTwo24, -(dmin * m0), d * s1 * kTwo20, -(dmin * m1) };
 			}
 			static __device__ __forceinline__ void frag(const Raw& r, const Scale& sc, int s, uint32_t (&out)[4])
 			{
-				const uint32_t v = r.q[s];
-				float f[8];
-#pragma unroll
-				for (int e = 0; e < 4; ++e)
-				{
-					f[e] = static_cast<float>((v >> (8 * e)) & 0xFu) * sc.s0 - sc.m0;         // sub-block 2g, element 4s + e
-					f[4 + e] = static_cast<float>((v >> (8 * e + 4)) & 0xFu) * sc.s1 - sc.m1; // sub-block 2g+1
-				}
-#pragma unroll
-				for (int i = 0; i < 4; ++i)
-				{
-					out[i] = pack_f16(f[2 * i], f[2 * i + 1]);
-				}
+				// low nibbles: sub-block 2g, elements 4s ..; high nibbles: sub-block 2g+1
+				nibbles8(r.q[s], sc.s0, sc.m0, sc.s1, sc.m1, out);
 			}
 			static __device__ __forceinline__ void koff(int g, int s, int& k0, int& k1)
 			{
@@ -246,7 +260,7 @@ namespace litenn_hip
 			// lane g = 2h + j covers l in [16j, 16j + 16) of half h: 16 bytes of each ql half-row,
 			// 16 bytes of qh, the four scales 8h + j + 2i and d
 			struct Raw { uint32_t la[4], lb[4], qh[4]; uint32_t sc[4]; uint32_t d; };
-			struct Scale { float s[4]; };
+			struct Scale { float s[4], b[4]; }; // d*scale*2^24 and -32*d*scale per quarter
 			static __device__ __forceinline__ Raw load(const uint8_t* chunk, int g)
 			{
 				const int h = g >> 1, j = g & 1;
@@ -276,34 +290,24 @@ namespace litenn_hip
 #pragma unroll
 				for (int i = 0; i < 4; ++i)
 				{
-					s.s[i] = d * static_cast<float>(static_cast<int8_t>(r.sc[i]));
+					const float ds = d * static_cast<float>(static_cast<int8_t>(r.sc[i]));
+					s.s[i] = ds * kTwo24;
+					s.b[i] = -32.0f * ds;
 				}
 				return s;
 			}
-			// step s: quarter i = s / 2 (q1..q4 of the reference decoder), elements 8 (s % 2) .. + 7 of the
-			// lane's 16
+			// step s: quarter i = s / 2 (q1..q4 of the ggml block definition), elements 8 (s % 2) .. + 7
+			// of the lane's 16; 6-bit value = nibble | two bits of qh << 4, minus 32
 			static __device__ __forceinline__ void frag(const Raw& r, const Scale& sc, int s, uint32_t (&out)[4])
 			{
 				const int i = s >> 1, u = s & 1;
-				float f[8];
 #pragma unroll
 				for (int w = 0; w < 2; ++w)
 				{
 					const uint32_t lw = (i & 1) ? r.lb[2 * u + w] : r.la[2 * u + w];
-					const uint32_t hw = r.qh[2 * u + w];
-#pragma unroll
-					for (int e = 0; e < 4; ++e)
-					{
-						const uint32_t lo = (lw >> (8 * e + (i >= 2 ? 4 : 0))) & 0xFu;
-						const uint32_t hi = (hw >> (8 * e + 2 * i)) & 3u;
-						const int q = static_cast<int>(lo | (hi << 4)) - 32;
-						f[4 * w + e] = static_cast<float>(q) * sc.s[i];
-					}
-				}
-#pragma unroll
-				for (int k = 0; k < 4; ++k)
-				{
-					out[k] = pack_f16(f[2 * k], f[2 * k + 1]);
+					const uint32_t nib = (i >= 2 ? lw >> 4 : lw) & 0x0f0f0f0fu;
+					const uint32_t top = ((r.qh[2 * u + w] >> (2 * i)) & 0x03030303u) << 4;
+					bytes4(nib | top, sc.s[i], sc.b[i], out[2 * w], out[2 * w + 1]);
 				}
 			}
 			static __device__ __forceinline__ void koff(int g, int s, int& k0, int& k1)
@@ -371,21 +375,26 @@ namespace litenn_hip
 		}
 
 		// ---- the GEMM ---------------------------------------------------------------------------
-		// grid (ceil(N / (64 NG)), ceil(M_pad / BM)); block 256.
-		template <typename F, int BM, int NG>
-		__global__ __launch_bounds__(256) void gemm_q_kernel(const uint8_t* __restrict__ w, const _Float16* __restrict__ xh,
-		                                                      const float* __restrict__ unscale, float* __restrict__ y,
-		                                                      const float* __restrict__ residual, int n, int k, int m,
-		                                                      int m_pad, size_t row_bytes)
+		// grid (ceil(N / (16 WAVES NG)), ceil(M_pad / BM)); block 64 WAVES.
+		template <typename F, int BM, int NG, int WAVES>
+		__global__ __launch_bounds__(64 * WAVES) void gemm_q_kernel(const uint8_t* __restrict__ w,
+		                                                             const _Float16* __restrict__ xh,
+		                                                             const float* __restrict__ unscale,
+		                                                             float* __restrict__ y,
+		                                                             const float* __restrict__ residual, int n, int k,
+		                                                             int m, int m_pad, size_t row_bytes)
 		{
-			constexpr int MT = BM / 16;                      // 16-row activation tiles
-			constexpr int kTileHalves = BM * kTileStride;    // one buffer of the LDS tile
-			constexpr int kStageLoads = (BM * 32) / 256;     // 16-byte loads per thread per chunk (BM rows x 512 B)
+			constexpr int kThreads = 64 * WAVES;
+			constexpr int MT = BM / 16;                   // 16-row activation tiles
+			constexpr int tile_stride = kTileStride;
+			constexpr int kTileHalves = BM * tile_stride; // one buffer of the LDS tile
+			constexpr int kPieces = BM * 32;              // 16-byte pieces of one BM x 512 B tile
+			constexpr int kStageLoads = (kPieces + kThreads - 1) / kThreads;
 			extern __shared__ __attribute__((aligned(16))) _Float16 tile[]; // [2][BM][kTileStride]
 			const int lane = threadIdx.x & 63;
 			const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 			const int r = lane & 15, g = lane >> 4;
-			const int n_base = (blockIdx.x * 4 + wave) * 16 * NG;
+			const int n_base = (blockIdx.x * WAVES + wave) * 16 * NG;
 			const int m_base = blockIdx.y * BM;
 			const int chunks = k / kChunk;
 
@@ -397,25 +406,32 @@ namespace litenn_hip
 				rows[q] = w + static_cast<size_t>(min(n_base + 16 * q + r, n - 1)) * row_bytes;
 			}
 
-			// activation staging: thread t moves 16-byte pieces p = t, t + 256, ... of the BM x 512 B tile
+			// activation staging: thread t moves 16-byte pieces p = t, t + kThreads, ... of the tile
 			u32x4 stage[kStageLoads];
 			const auto stage_load = [&](int c) {
 #pragma unroll
 				for (int i = 0; i < kStageLoads; ++i)
 				{
-					const int p = threadIdx.x + 256 * i;
-					const int row = p >> 5, piece = p & 31;
-					const int mm = min(m_base + row, m_pad - 1);
-					stage[i] = *reinterpret_cast<const u32x4*>(xh + static_cast<size_t>(mm) * k + c * kChunk + piece * 8);
+					const int p = threadIdx.x + kThreads * i;
+					if (kPieces % kThreads == 0 || p < kPieces)
+					{
+						const int row = p >> 5, piece = p & 31;
+						const int mm = min(m_base + row, m_pad - 1);
+						stage[i] =
+						    *reinterpret_cast<const u32x4*>(xh + static_cast<size_t>(mm) * k + c * kChunk + piece * 8);
+					}
 				}
 			};
 			const auto stage_store = [&](int buf) {
 #pragma unroll
 				for (int i = 0; i < kStageLoads; ++i)
 				{
-					const int p = threadIdx.x + 256 * i;
-					const int row = p >> 5, piece = p & 31;
-					*reinterpret_cast<u32x4*>(tile + buf * kTileHalves + row * kTileStride + piece * 8) = stage[i];
+					const int p = threadIdx.x + kThreads * i;
+					if (kPieces % kThreads == 0 || p < kPieces)
+					{
+						const int row = p >> 5, piece = p & 31;
+						*reinterpret_cast<u32x4*>(tile + buf * kTileHalves + row * tile_stride + piece * 8) = stage[i];
+					}
 				}
 			};
 
@@ -430,36 +446,15 @@ namespace litenn_hip
 				}
 			}
 
-			typename F::Raw raw[NG], raw_next[NG];
-#pragma unroll
-			for (int q = 0; q < NG; ++q)
-			{
-				raw[q] = F::load(rows[q], g);
-			}
-			stage_load(0);
-			stage_store(0);
-			__syncthreads();
-
-			for (int c = 0; c < chunks; ++c)
-			{
-				const int buf = c & 1;
-				const bool more = c + 1 < chunks;
-				if (more)
-				{
-#pragma unroll
-					for (int q = 0; q < NG; ++q)
-					{
-						raw_next[q] = F::load(rows[q] + static_cast<size_t>(c + 1) * F::kChunkBytes, g);
-					}
-					stage_load(c + 1);
-				}
+			// one 256-wide chunk: decode the lane's weights step by step, multiply against the tile
+			const auto multiply = [&](const typename F::Raw (&raw)[NG], int buf) {
 				typename F::Scale sc[NG];
 #pragma unroll
 				for (int q = 0; q < NG; ++q)
 				{
 					sc[q] = F::prep(raw[q], g);
 				}
-				const _Float16* xt = tile + buf * kTileHalves + r * kTileStride;
+				const _Float16* xt = tile + buf * kTileHalves + r * tile_stride;
 #pragma unroll
 				for (int s = 0; s < 8; ++s)
 				{
@@ -477,7 +472,7 @@ namespace litenn_hip
 #pragma unroll
 					for (int t = 0; t < MT; ++t)
 					{
-						const _Float16* xr = xt + t * 16 * kTileStride;
+						const _Float16* xr = xt + t * 16 * tile_stride;
 						const u32x2 b0 = *reinterpret_cast<const u32x2*>(xr + k0);
 						const u32x2 b1 = *reinterpret_cast<const u32x2*>(xr + k1);
 						const u32x4 bv = { b0.x, b0.y, b1.x, b1.y };
@@ -489,15 +484,57 @@ namespace litenn_hip
 							acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[q], b, acc[q][t], 0, 0, 0);
 						}
 					}
+					// keep the steps apart: left alone the scheduler hoists every LDS read of the chunk
+					// to the top and spills the accumulators
+					__builtin_amdgcn_sched_barrier(0);
 				}
-				if (more)
-				{
-					stage_store(buf ^ 1);
+			};
+			const auto load_raw = [&](typename F::Raw (&raw)[NG], int c) {
 #pragma unroll
-					for (int q = 0; q < NG; ++q)
-					{
-						raw[q] = raw_next[q];
-					}
+				for (int q = 0; q < NG; ++q)
+				{
+					raw[q] = F::load(rows[q] + static_cast<size_t>(c) * F::kChunkBytes, g);
+				}
+			};
+
+			// Two register sets of raw weight bytes alternate, so no set is copied; within a phase
+			// the next activation tile is requested first and the next weights after it: the tile
+			// must be in LDS before the barrier, the weights only when the next phase starts.
+			typename F::Raw raw_a[NG], raw_b[NG];
+			load_raw(raw_a, 0);
+			stage_load(0);
+			stage_store(0);
+			__syncthreads();
+			// s_waitcnt vmcnt(0) (expcnt and lgkmcnt left at their maxima).  Placed before a phase
+			// requests anything new, it makes the phase's own weights (requested one phase earlier)
+			// the only loads waited for; without it the compiler waits for them after the new
+			// requests are queued, and the in-order counter then drains those too.
+			constexpr int kWaitAllLoads = 0x0F70;
+			for (int c = 0; c < chunks; c += 2)
+			{
+				__builtin_amdgcn_s_waitcnt(kWaitAllLoads);
+				if (c + 1 < chunks)
+				{
+					stage_load(c + 1);
+					load_raw(raw_b, c + 1);
+				}
+				multiply(raw_a, 0);
+				if (c + 1 >= chunks)
+				{
+					break;
+				}
+				stage_store(1);
+				__syncthreads();
+				__builtin_amdgcn_s_waitcnt(kWaitAllLoads);
+				if (c + 2 < chunks)
+				{
+					stage_load(c + 2);
+					load_raw(raw_a, c + 2);
+				}
+				multiply(raw_b, 1);
+				if (c + 2 < chunks)
+				{
+					stage_store(0);
 				}
 				__syncthreads();
 			}
@@ -530,64 +567,54 @@ namespace litenn_hip
 			}
 		}
 
-		template <typename F, int BM, int NG>
+		template <typename F, int BM, int NG, int WAVES>
 		void launch_variant(const uint8_t* w, const _Float16* xh, const float* unscale, float* y, const float* residual,
 		                    int n, int k, int m, int m_pad, size_t row_bytes, hipStream_t stream)
 		{
 			constexpr size_t lds = sizeof(_Float16) * 2 * BM * kTileStride;
 			static const hipError_t attr =
-			    hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_q_kernel<F, BM, NG>),
+			    hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_q_kernel<F, BM, NG, WAVES>),
 			                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
 			(void)attr;
-			const dim3 grid((n + 64 * NG - 1) / (64 * NG), (m_pad + BM - 1) / BM);
-			gemm_q_kernel<F, BM, NG><<<grid, dim3(256), lds, stream>>>(w, xh, unscale, y, residual, n, k, m, m_pad,
-			                                                         row_bytes);
+			constexpr int bn = 16 * WAVES * NG;
+			const dim3 grid((n + bn - 1) / bn, (m_pad + BM - 1) / BM);
+			gemm_q_kernel<F, BM, NG, WAVES><<<grid, dim3(64 * WAVES), lds, stream>>>(w, xh, unscale, y, residual, n, k, m,
+			                                                                        m_pad, row_bytes);
 		}
 
-		// Tile choice: the activation tile as tall as the batch allows (each weight byte is
-		// decoded once per activation tile), then as many row groups per wavefront as still
-		// leave at least one workgroup per CU.
+		// Tile choice, from measurement on the MI355X (K = 4096; N = 14336 and 4096; M = 16 .. 512):
+		// the kernel is bound by the LDS reads of the activation operand and by latency, not by the
+		// matrix cores, so what pays is several small workgroups per CU (64-row activation tiles at
+		// most) and two row groups per wavefront (each activation fragment feeds two MFMAs) once the
+		// batch is large enough to keep every CU busy that way.
 		template <typename F>
 		void launch_format(const uint8_t* w, const _Float16* xh, const float* unscale, float* y, const float* residual,
 		                   int n, int k, int m, int m_pad, size_t row_bytes, int cus, hipStream_t stream)
 		{
-			const auto blocks = [&](int bm, int ng) {
-				return static_cast<long>((n + 64 * ng - 1) / (64 * ng)) * ((m_pad + bm - 1) / bm);
+			const auto blocks = [&](int bm, int bn) {
+				return static_cast<long>((n + bn - 1) / bn) * ((m_pad + bm - 1) / bm);
 			};
+#define LITENN_GEMM_ARGS w, xh, unscale, y, residual, n, k, m, m_pad, row_bytes, stream
 			if (m_pad >= 128)
 			{
-				if (blocks(128, 4) >= cus)
+				if (blocks(64, 128) >= 2 * cus)
 				{
-					launch_variant<F, 128, 4>(w, xh, unscale, y, residual, n, k, m, m_pad, row_bytes, stream);
-				}
-				else if (blocks(128, 2) >= cus)
-				{
-					launch_variant<F, 128, 2>(w, xh, unscale, y, residual, n, k, m, m_pad, row_bytes, stream);
+					launch_variant<F, 64, 2, 4>(LITENN_GEMM_ARGS);
 				}
 				else
 				{
-					launch_variant<F, 128, 1>(w, xh, unscale, y, residual, n, k, m, m_pad, row_bytes, stream);
-				}
-			}
-			else if (m_pad >= 64)
-			{
-				if (blocks(64, 2) >= cus)
-				{
-					launch_variant<F, 64, 2>(w, xh, unscale, y, residual, n, k, m, m_pad, row_bytes, stream);
-				}
-				else
-				{
-					launch_variant<F, 64, 1>(w, xh, unscale, y, residual, n, k, m, m_pad, row_bytes, stream);
+					launch_variant<F, 64, 1, 4>(LITENN_GEMM_ARGS);
 				}
 			}
 			else if (m_pad >= 32)
 			{
-				launch_variant<F, 32, 1>(w, xh, unscale, y, residual, n, k, m, m_pad, row_bytes, stream);
+				launch_variant<F, 32, 1, 4>(LITENN_GEMM_ARGS);
 			}
 			else
 			{
-				launch_variant<F, 16, 1>(w, xh, unscale, y, residual, n, k, m, m_pad, row_bytes, stream);
+				launch_variant<F, 16, 1, 4>(LITENN_GEMM_ARGS);
 			}
+#undef LITENN_GEMM_ARGS
 		}
 	} // namespace
 
