@@ -102,3 +102,36 @@ def test_error_paths(hip):
         m.set_tensor("attn_q", 0, Q4_0, np.zeros(18, np.uint8), 1, 32)
     with pytest.raises(hip.LiteNNHipError, match="head counts"):
         hip.LLaMA(1, 64, 4, 3, 64, 10, 8)
+
+
+def test_llama7b_q4_0_greedy_matches_committed_fixture(hip):
+    """BASELINE config 4 at full size: the 7B-shape Q4_0 model, prompt 128, 256 greedy tokens, fp16
+    KV cache, against tests/golden/llama7b_q4_0_tokens.json (written from the CPU checker by
+    tests/golden/make_llama7b_tokens.py; the model and the prompt are rebuilt from the seed).
+    Tokens must be identical; the top-2 logit margin of the first step must agree to 1e-3 relative,
+    which is what makes the identity meaningful for this random-init model (its margins are ~1.9)."""
+    import json
+    import os
+    fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "llama7b_q4_0_tokens.json")))
+    assert fx["complete"] and fx["new_tokens"] == 256
+    cfg = synth.llama_7b_q4_0(context_length=fx["context_length"])
+    assert cfg.name == fx["model"]
+    prompt = synth.prompt_tokens(cfg, fx["prompt_length"], fx["seed"])
+    assert prompt[:8].tolist() == fx["prompt_head"]
+    dev = hip_model(hip, cfg, fx["seed"])
+    # f32-operand prefill (GEMV path), then the captured single-token step
+    got, _, _ = dev.generate(prompt, 256)
+    assert got.tolist() == fx["tokens"]
+    # prefill on the matrix cores (fp16 operands), same continuation
+    dev.reset()
+    again, _, _ = dev.generate(prompt, 256, precise=False)
+    assert again.tolist() == fx["tokens"]
+    # margins: first generated step, from the logits of the last prompt position
+    dev.reset()
+    logits = dev.eval(prompt, all_logits=False)
+    best = int(np.argmax(logits))
+    rest = logits.copy()
+    rest[best] = -np.inf
+    assert best == fx["tokens"][0]
+    assert abs(float(logits[best] - rest.max()) - fx["margins"][0]) <= 1e-3 * abs(fx["margins"][0])
+    dev.close()
