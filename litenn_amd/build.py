@@ -61,5 +61,24 @@ def build(verbose: bool = True, jobs: int = 6) -> str:
     return LIB_PATH
 
 
+CPP_TEST_SRC = os.path.join(os.path.dirname(HERE), "tests", "cpp", "device_traits_test.cpp")
+CPP_TEST_BIN = os.path.join(os.path.dirname(HERE), "tests", "cpp", "device_traits_test")
+
+
+def build_cpp_host_test(verbose: bool = True) -> str:
+    """Compile the C++ host-side test of include/LiteNN/Device/HIP.h against the built library
+    (plain g++, C++20; no GPU code in it)."""
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if not cxx:
+        raise RuntimeError("g++ not found; the C++ host test cannot be built")
+    cmd = [cxx, "-std=c++20", "-O1", "-Wall", "-I", os.path.join(os.path.dirname(HERE), "include"), CPP_TEST_SRC,
+           "-L", LIB_DIR, "-llitenn_hip", "-Wl,-rpath,$ORIGIN/../../litenn_amd/lib", "-o", CPP_TEST_BIN]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return CPP_TEST_BIN
+
+
 if __name__ == "__main__":
     build()
+    build_cpp_host_test()
