@@ -189,15 +189,18 @@ def bench_cpu_baseline(fmt, n, k, budget_s=12.0):
     return dt / calls, calls
 
 
-def bench_decode(ln, n_prompt=128, n_new=256, seed=4):
+def bench_decode(ln, n_prompt=128, n_new=256, seed=4, model_name="7b"):
     from litenn_amd import synth
     from litenn_amd.formats import DT_F16
-    cfg = synth.llama_7b_q4_0(context_length=n_prompt + n_new)
+    if model_name == "8b":
+        cfg = synth.llama_8b_gqa_mixed(context_length=n_prompt + n_new)
+    else:
+        cfg = synth.llama_7b_q4_0(context_length=n_prompt + n_new)
     t0 = time.perf_counter()
     model = ln.LLaMA.from_config(cfg, kv_dtype=DT_F16)
     for item in synth.llama_tensors(cfg, seed):
         model.set_tensor(*item)
-    log(f"[bench] 7B-shape Q4_0 model resident after {time.perf_counter() - t0:.1f} s")
+    log(f"[bench] {cfg.name} resident after {time.perf_counter() - t0:.1f} s")
     prompt = synth.prompt_tokens(cfg, n_prompt, seed)
     model.generate(prompt, 8, precise=False)  # warm-up: captures the step graph
     model.reset()
@@ -230,6 +233,8 @@ def main() -> int:
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--decode-prompt", type=int, default=128, help="prompt length of the decode run")
     ap.add_argument("--decode-new", type=int, default=256, help="tokens generated by the decode run")
+    ap.add_argument("--decode-model", choices=["7b", "8b"], default="7b",
+                    help="7b: 7B-shape Q4_0 (the headline decode); 8b: 8B GQA shape, Q4_K + Q6_K")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill (batched matmul) measurements")
     ap.add_argument("--gemm-case", default=None, help="run only this prefill case, e.g. Q4_K:512")
@@ -301,7 +306,7 @@ def main() -> int:
     if not args.no_gemm:
         line["prefill_gemm"] = bench_prefill_gemm(ln, hiprt, args.gemm_case)
     if not args.no_decode:
-        line["decode"] = bench_decode(ln, args.decode_prompt, args.decode_new)
+        line["decode"] = bench_decode(ln, args.decode_prompt, args.decode_new, model_name=args.decode_model)
         log(f"[bench] decode: {line['decode']['tokens_per_s']} tok/s")
     print(json.dumps(line), flush=True)
     return 0
