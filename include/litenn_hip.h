@@ -229,6 +229,55 @@ int litenn_hip_llama_generate(litenn_hip_llama* model, const int32_t* prompt, si
 /* Copies the first `past` cache rows of one layer to host as f32 [past, n_kv_head*head_dim]. */
 int litenn_hip_llama_get_kv(litenn_hip_llama* model, int layer, float* k, float* v);
 
+/* ---- group 4: GGUF container reader (host side) ------------------------ */
+
+/* A dependency-free reader of the GGUF container (versions 2 and 3), producing what
+ * ImportGGUFArchive produces (tools/gguf/GGUFImporter.cpp:644-678) without ggml: metadata
+ * widened to u64 / i64 / f64 / bool / string (:339-437), tensors as (type, shape with the
+ * slowest dimension first, :206-221, raw payload, :457-502), LLaMA hyper-parameters with the
+ * defaults and checks of ParseLLaMAHyperparameters (:505-642).  The file is mapped read-only;
+ * pointers handed out stay valid until litenn_gguf_close.  Error texts are the reference's. */
+typedef struct litenn_gguf litenn_gguf;
+
+typedef struct litenn_gguf_tensor {
+	const char* name;
+	int ggml_type;      /* id of the published ggml_type enum */
+	int fmt;            /* QuantizedBlockFormat this backend executes, or -1 */
+	int dtype;          /* DataType of a plain tensor, or -1 */
+	int quantized;      /* non-zero for block formats */
+	size_t rank;
+	size_t shape[4];    /* slowest dimension first: a [N, K] weight has shape {N, K} */
+	size_t file_offset; /* of the payload, from the start of the file */
+	size_t bytes;
+	const void* data;   /* the payload inside the mapping */
+} litenn_gguf_tensor;
+
+int litenn_gguf_open(const char* path, litenn_gguf** out);
+void litenn_gguf_close(litenn_gguf* file);
+unsigned litenn_gguf_version(const litenn_gguf* file);
+size_t litenn_gguf_tensor_count(const litenn_gguf* file);
+size_t litenn_gguf_metadata_count(const litenn_gguf* file);
+int litenn_gguf_tensor_info(const litenn_gguf* file, size_t index, litenn_gguf_tensor* out);
+int litenn_gguf_find_tensor(const litenn_gguf* file, const char* name, litenn_gguf_tensor* out);
+const char* litenn_gguf_metadata_key(const litenn_gguf* file, size_t index);
+/* ReadSizeValue / ReadDoubleValue / ReadStringValue / ReadBoolValue,
+ * tools/gguf/GGUFImporter.cpp:66-147: any integer type for sizes (negative values refused),
+ * any numeric type for doubles. */
+int litenn_gguf_metadata_u64(const litenn_gguf* file, const char* key, uint64_t* out);
+int litenn_gguf_metadata_f64(const litenn_gguf* file, const char* key, double* out);
+int litenn_gguf_metadata_str(const litenn_gguf* file, const char* key, const char** out);
+int litenn_gguf_metadata_bool(const litenn_gguf* file, const char* key, int* out);
+int litenn_gguf_metadata_array(const litenn_gguf* file, const char* key, unsigned* elem_type, size_t* count);
+/* Fills every field but kv_dtype; vocab_size comes from token_embd.weight
+ * (tools/gguf/LLaMABuilder.cpp:685-703). */
+int litenn_gguf_llama_params(const litenn_gguf* file, litenn_hip_llama_params* out);
+/* Reads the file, uploads the tensors of the decoder (token_embd, output_norm, optional output,
+ * and per block attn_norm, attn_q/k/v/output, ffn_norm, ffn_gate/up/down: the names of
+ * tools/gguf/LLaMABuilder.cpp:171-178,466-500) and returns a resident model that owns them.
+ * context_length > 0 overrides the file's; kv_dtype is F16 or F32. */
+int litenn_hip_llama_load_gguf(int dev, const char* path, int kv_dtype, int32_t context_length,
+                               litenn_hip_llama** out);
+
 #ifdef __cplusplus
 }
 #endif

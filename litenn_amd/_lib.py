@@ -27,6 +27,14 @@ class LlamaParams(C.Structure):
     ]
 
 
+class GgufTensor(C.Structure):
+    _fields_ = [
+        ("name", C.c_char_p), ("ggml_type", C.c_int), ("fmt", C.c_int), ("dtype", C.c_int), ("quantized", C.c_int),
+        ("rank", C.c_size_t), ("shape", C.c_size_t * 4), ("file_offset", C.c_size_t), ("bytes", C.c_size_t),
+        ("data", C.c_void_p),
+    ]
+
+
 _vp, _sz, _i, _u, _d = C.c_void_p, C.c_size_t, C.c_int, C.c_uint, C.c_double
 _szp = C.POINTER(C.c_size_t)
 _ex = C.POINTER(Exec)
@@ -69,8 +77,27 @@ SIGNATURES = {
     "litenn_hip_llama_eval": [_vp, _vp, _sz, _vp, _vp, _u],
     "litenn_hip_llama_generate": [_vp, _vp, _sz, _sz, _vp, _u, C.POINTER(_d), C.POINTER(_d)],
     "litenn_hip_llama_get_kv": [_vp, _i, _vp, _vp],
+    "litenn_gguf_open": [C.c_char_p, C.POINTER(_vp)],
+    "litenn_gguf_close": [_vp],
+    "litenn_gguf_version": [_vp],
+    "litenn_gguf_tensor_count": [_vp],
+    "litenn_gguf_metadata_count": [_vp],
+    "litenn_gguf_tensor_info": [_vp, _sz, C.POINTER(GgufTensor)],
+    "litenn_gguf_find_tensor": [_vp, C.c_char_p, C.POINTER(GgufTensor)],
+    "litenn_gguf_metadata_key": [_vp, _sz],
+    "litenn_gguf_metadata_u64": [_vp, C.c_char_p, C.POINTER(C.c_uint64)],
+    "litenn_gguf_metadata_f64": [_vp, C.c_char_p, C.POINTER(_d)],
+    "litenn_gguf_metadata_str": [_vp, C.c_char_p, C.POINTER(C.c_char_p)],
+    "litenn_gguf_metadata_bool": [_vp, C.c_char_p, C.POINTER(_i)],
+    "litenn_gguf_metadata_array": [_vp, C.c_char_p, C.POINTER(_u), C.POINTER(_sz)],
+    "litenn_gguf_llama_params": [_vp, C.POINTER(LlamaParams)],
+    "litenn_hip_llama_load_gguf": [_i, C.c_char_p, _i, C.c_int32, C.POINTER(_vp)],
 }
-_RESTYPES = {"litenn_hip_last_error": C.c_char_p, "litenn_hip_mul_mat_q_workspace_bytes": C.c_size_t}
+_RESTYPES = {
+    "litenn_hip_last_error": C.c_char_p, "litenn_hip_mul_mat_q_workspace_bytes": C.c_size_t,
+    "litenn_gguf_close": None, "litenn_gguf_version": C.c_uint, "litenn_gguf_tensor_count": C.c_size_t,
+    "litenn_gguf_metadata_count": C.c_size_t, "litenn_gguf_metadata_key": C.c_char_p,
+}
 
 _lib = None
 

@@ -101,6 +101,7 @@ struct litenn_hip_llama
 	float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *gate = nullptr,
 	      *gate2 = nullptr, *up = nullptr, *logits = nullptr;
 	void* xh = nullptr; // fp16 copy of a matmul's activations (multi-row path), 16-row padded
+	std::vector<void*> owned; // device buffers freed with the model (tensors uploaded by the GGUF loader)
 	int32_t* d_tokens = nullptr;
 	int32_t* d_next = nullptr; // token produced by the last arg-max
 	int32_t* d_out = nullptr;  // generated tokens
@@ -481,6 +482,17 @@ extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* p
 	return 0;
 }
 
+// Hands a device allocation to the model: it is released by litenn_hip_llama_free.
+extern "C" int litenn_hip_llama_adopt(litenn_hip_llama* m, void* device_ptr)
+{
+	if (!m || !device_ptr)
+	{
+		return fail(kAction, "null argument");
+	}
+	m->owned.push_back(device_ptr);
+	return 0;
+}
+
 extern "C" int litenn_hip_llama_free(litenn_hip_llama* m)
 {
 	if (!m)
@@ -504,6 +516,10 @@ extern "C" int litenn_hip_llama_free(litenn_hip_llama* m)
 		{
 			(void)hipFree(L.vcache);
 		}
+	}
+	for (void* ptr : m->owned)
+	{
+		(void)hipFree(ptr);
 	}
 	void* singles[] = { m->cos_t, m->sin_t,      m->logits,       m->d_next,       m->d_out,
 	                    m->d_counters, m->d_err, m->attn_partial, m->attn_counters };

@@ -37,6 +37,23 @@ class LLaMA:
                    cfg.feed_forward_length, cfg.vocab, cfg.context_length, cfg.rms_eps, cfg.rope_freq_base,
                    kv_dtype=kv_dtype, device=device)
 
+    @classmethod
+    def from_gguf(cls, path: str, kv_dtype=DT_F16, context_length: int = 0, device: HIP = HIP()) -> "LLaMA":
+        """Read a GGUF file, upload its decoder tensors and return the resident model (the library
+        owns the uploaded buffers).  context_length > 0 overrides the file's."""
+        from .gguf import GGUFFile
+        with GGUFFile(path) as f:
+            p = f.llama_params()
+        self = cls.__new__(cls)
+        self.device = device
+        self.vocab_size = p.vocab_size
+        self.kv_width = p.head_count_kv * (p.embedding_length // max(p.head_count, 1))
+        self._tensors = []
+        self._h = C.c_void_p()
+        check(_lib.load().litenn_hip_llama_load_gguf(device.deviceIndex, str(path).encode(), kv_dtype, context_length,
+                                                     C.byref(self._h)))
+        return self
+
     def close(self) -> None:
         if self._h:
             _lib.load().litenn_hip_llama_free(self._h)

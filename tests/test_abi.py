@@ -10,7 +10,7 @@ from litenn_amd import _lib
 def declared_symbols():
     text = open(_lib.HEADER_PATH).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(litenn_hip_[a-z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(litenn_(?:hip|gguf)_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_library_is_built_in_tree():

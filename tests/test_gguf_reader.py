@@ -1,0 +1,135 @@
+"""The GGUF container reader (host code in the library, no GPU): files written by the
+independent writer in tests/gguf_writer.py are parsed back; behaviour follows the reference's
+importer (tools/gguf/GGUFImporter.cpp) -- shape reversal (:206-221, pinned by
+tests/GGUFImporterTest.cpp:513-519), raw payload import (:457-502, the 18-byte Q4_0 fixture of
+tests/GGUFImporterTest.cpp:173-178,521-534), metadata widening (:339-437), hyper-parameter defaults,
+checks and messages (:505-642)."""
+import numpy as np
+import pytest
+
+import gguf_writer as gw
+from litenn_amd import synth
+from litenn_amd._lib import LiteNNHipError
+from litenn_amd.formats import Q4_0, Q4_K, Q6_K, Q8_0
+from litenn_amd.gguf import GGUFFile
+
+Q4_0_FIXTURE = bytes([0x10, 0x00, 0x22, 0x44, 0x66, 0x88, 0xaa, 0xcc, 0xee, 0x11, 0x33, 0x55, 0x77, 0x99, 0xbb, 0xdd,
+                      0xff, 0x7f])
+
+
+def test_q4_0_payload_fixture_round_trips(tmp_path):
+    """The reference's raw-import fixture: one Q4_0 block, shape [32], bytes kept verbatim."""
+    path = gw.write_gguf(tmp_path / "one.gguf", [("general.architecture", gw.STRING, "llama")],
+                         [("blk.0.attn_q.weight", "q4_0", (32,), np.frombuffer(Q4_0_FIXTURE, np.uint8))])
+    with GGUFFile(path) as f:
+        assert f.version == 3 and f.tensor_count == 1 and f.metadata_count == 1
+        t = f.tensor("blk.0.attn_q.weight")
+        assert t.shape == (32,) and t.quantized and t.fmt == Q4_0 and t.dtype == -1 and t.bytes == 18
+        raw = f.payload(0)
+        assert raw[0] == 0x10 and raw[17] == 0x7f  # what the reference's test asserts
+        assert raw.tobytes() == Q4_0_FIXTURE
+        assert t.file_offset % 32 == 0
+
+
+def test_shapes_are_reversed_and_payloads_aligned(tmp_path):
+    rng = np.random.default_rng(0)
+    a = rng.standard_normal((3, 5)).astype(np.float32)           # stored as ne = [5, 3]
+    q = synth.quant_weights(Q6_K, 7, 512, 1)
+    path = gw.write_gguf(tmp_path / "s.gguf", [], [("a", "f32", (3, 5), a), ("q", "q6_k", (7, 512), q),
+                                                    ("v", "f32", (4,), np.arange(4, dtype=np.float32))], alignment=64,
+                         declare_alignment=True)
+    with GGUFFile(path) as f:
+        ta, tq, tv = f.tensor("a"), f.tensor("q"), f.tensor(2)
+        assert ta.shape == (3, 5) and ta.dtype == 0 and not ta.quantized and ta.fmt == -1
+        assert np.array_equal(f.payload("a").view(np.float32).reshape(3, 5), a)
+        assert tq.shape == (7, 512) and tq.fmt == Q6_K and tq.bytes == 7 * 2 * 210
+        assert np.array_equal(f.payload("q"), q.reshape(-1))
+        assert tv.name == "v" and tv.shape == (4,)
+        assert all(t.file_offset % 64 == 0 for t in f.tensors())
+        assert f.get_size("general.alignment") == 64
+
+
+def test_metadata_is_widened_like_the_reference(tmp_path):
+    md = [("u8", gw.U8, 200), ("i8", gw.I8, -5), ("u16", gw.U16, 60000), ("i16", gw.I16, -300), ("u32", gw.U32, 7),
+          ("i32", gw.I32, 12), ("f32", gw.F32, 0.5), ("b", gw.BOOL, 1), ("s", gw.STRING, "hello"),
+          ("u64", gw.U64, 2 ** 40), ("i64", gw.I64, -2 ** 40), ("f64", gw.F64, 1e-300),
+          ("arr", gw.ARRAY, (gw.I32, [1, 2, 3])), ("names", gw.ARRAY, (gw.STRING, ["a", "bc"]))]
+    path = gw.write_gguf(tmp_path / "m.gguf", md, [])
+    with GGUFFile(path) as f:
+        assert f.keys() == [k for k, _, _ in md]
+        assert f.get_size("u8") == 200 and f.get_size("u16") == 60000 and f.get_size("i32") == 12
+        assert f.get_size("u64") == 2 ** 40
+        assert f.get_double("f32") == 0.5 and f.get_double("f64") == 1e-300 and f.get_double("i8") == -5.0
+        assert f.get_string("s") == "hello" and f.get_bool("b") is True
+        assert f.get_array_info("arr") == (gw.I32, 3) and f.get_array_info("names") == (gw.STRING, 2)
+        for key, msg in [("i8", "must be non-negative"), ("f32", "must be an integer"), ("s", "must be an integer")]:
+            with pytest.raises(LiteNNHipError, match=f"GGUF metadata key '{key}' {msg}"):
+                f.get_size(key)
+        with pytest.raises(LiteNNHipError, match="GGUF metadata key 's' must be numeric"):
+            f.get_double("s")
+        with pytest.raises(LiteNNHipError, match="GGUF metadata key 'u8' must be a string"):
+            f.get_string("u8")
+        with pytest.raises(LiteNNHipError, match="Missing GGUF metadata key 'nope'"):
+            f.get_size("nope")
+        with pytest.raises(LiteNNHipError, match="Missing GGUF tensor 'nope'"):
+            f.tensor("nope")
+
+
+def test_llama_hyperparameters_defaults_and_checks(tmp_path):
+    cfg = synth.tiny_llama(Q4_K, block_count=1, d_model=256, heads=4, kv_heads=2, ff=512, vocab=300, context_length=77)
+    with GGUFFile(gw.llama_gguf(tmp_path / "t.gguf", cfg, 1)) as f:
+        p = f.llama_params()
+        assert (p.block_count, p.embedding_length, p.head_count, p.head_count_kv, p.feed_forward_length) == \
+               (1, 256, 4, 2, 512)
+        assert p.vocab_size == 300 and p.context_length == 77
+        assert p.rope_dimension_count == 64  # defaults to the head dimension
+        assert p.rms_norm_epsilon == float(np.float32(cfg.rms_eps))  # f32 key widened to double
+        assert p.rope_freq_base == cfg.rope_freq_base and p.rope_freq_scale == 1.0
+        assert f.get_string("general.architecture") == "llama"
+
+    # linear rope scaling: freq_scale = 1 / factor; another architecture prefix works the same way
+    extra = [("qwen2.rope.scaling.type", gw.STRING, "LINEAR"), ("qwen2.rope.scaling.factor", gw.F32, 4.0)]
+    with GGUFFile(gw.llama_gguf(tmp_path / "l.gguf", cfg, 1, extra_metadata=extra, arch="qwen2")) as f:
+        assert f.llama_params().rope_freq_scale == 0.25
+
+    bad = [
+        ([("llama.rope.scaling.type", gw.STRING, "yarn")], "only executes none/linear scaling, got 'yarn'"),
+        ([("llama.rope.scaling.type", gw.STRING, "weird")], "Unsupported LLaMA rope.scaling.type 'weird'"),
+        ([("llama.rope.dimension_count", gw.U32, 63)], "rope.dimension_count must be an even value"),
+        ([("llama.rope.scaling.factor", gw.F32, -1.0)], "rope.scaling.factor must be non-negative"),
+    ]
+    for i, (extra, msg) in enumerate(bad):
+        with GGUFFile(gw.llama_gguf(tmp_path / f"bad{i}.gguf", cfg, 1, extra_metadata=extra)) as f:
+            with pytest.raises(LiteNNHipError, match=msg):
+                f.llama_params()
+    cfg_bad = synth.tiny_llama(Q4_0, block_count=1, d_model=256, heads=4, kv_heads=3, ff=512, vocab=300)
+    with GGUFFile(gw.llama_gguf(tmp_path / "kv.gguf", cfg_bad, 1, skip=("attn_k", "attn_v"))) as f:
+        with pytest.raises(LiteNNHipError, match="attention.head_count 4 must be divisible by attention.head_count_kv 3"):
+            f.llama_params()
+
+
+def test_broken_files_are_refused(tmp_path):
+    with pytest.raises(LiteNNHipError, match="Failed to open GGUF file"):
+        GGUFFile(tmp_path / "missing.gguf")
+    p = tmp_path / "junk.gguf"
+    p.write_bytes(b"GGUX" + b"\0" * 64)
+    with pytest.raises(LiteNNHipError, match="Failed to open GGUF file"):
+        GGUFFile(p)
+    good = gw.write_gguf(tmp_path / "g.gguf", [], [("a", "f32", (64,), np.zeros(64, np.float32))])
+    raw = open(good, "rb").read()
+    cut = tmp_path / "cut.gguf"
+    cut.write_bytes(raw[:-100])  # payload truncated
+    with pytest.raises(LiteNNHipError, match="Failed to read 256 bytes for GGUF tensor 'a'"):
+        GGUFFile(cut)
+    odd = gw.write_gguf(tmp_path / "odd.gguf", [], [("q", "q4_k", (2, 256), np.zeros(288, np.uint8))])
+    with GGUFFile(odd) as f:
+        assert f.tensor("q").bytes == 288
+    # an unknown ggml type id
+    patched = bytearray(open(odd, "rb").read())
+    idx = patched.find(b"q" + (2).to_bytes(4, "little"))  # name 'q' followed by rank 2
+    type_pos = idx + 1 + 4 + 16
+    patched[type_pos:type_pos + 4] = (99).to_bytes(4, "little")
+    bad = tmp_path / "type.gguf"
+    bad.write_bytes(bytes(patched))
+    with pytest.raises(LiteNNHipError, match="Unsupported ggml tensor type '99' for tensor 'q'"):
+        GGUFFile(bad)

@@ -135,3 +135,40 @@ def test_llama7b_q4_0_greedy_matches_committed_fixture(hip):
     assert best == fx["tokens"][0]
     assert abs(float(logits[best] - rest.max()) - fx["margins"][0]) <= 1e-3 * abs(fx["margins"][0])
     dev.close()
+
+
+def test_model_loaded_from_a_gguf_file(hip, oracle, tmp_path):
+    """GGUF file -> resident decoder through the library's own reader: same logits as the model built
+    tensor by tensor (bit for bit) and as the CPU checker; absent output.weight ties the head to the
+    embedding (tools/gguf/LLaMABuilder.cpp:719-733); problems are reported with the reference's texts."""
+    import gguf_writer as gw
+    from litenn_amd._lib import LiteNNHipError
+    cfg = synth.tiny_llama(Q4_K, block_count=2, d_model=512, heads=4, kv_heads=2, ff=768, vocab=333, context_length=48,
+                           formats={"default": Q4_K, "attn_v": Q6_K, "ffn_down": Q6_K, "token_embd": Q8_0})
+    path = gw.llama_gguf(tmp_path / "m.gguf", cfg, 11)
+    toks = synth.prompt_tokens(cfg, 7, 3)
+    loaded = hip.LLaMA.from_gguf(str(path))
+    built = hip_model(hip, cfg, 11)
+    got = loaded.eval(toks)
+    assert np.array_equal(got, built.eval(toks))
+    assert rel_l2(got, oracle_model(oracle, cfg, 11).eval(toks)) < 1e-4
+    assert loaded.past == 7
+    loaded.reset()
+    built.reset()
+    tokens, _, _ = loaded.generate(toks, 5)
+    assert tokens.tolist() == built.generate(toks, 5)[0].tolist()
+    loaded.close()
+
+    # context override, tied head
+    tied_path = gw.llama_gguf(tmp_path / "tied.gguf", cfg, 11, skip=("output",))
+    tied = hip.LLaMA.from_gguf(str(tied_path), context_length=16)
+    ref_tied = oracle_model(oracle, cfg, 11, skip=("output",))
+    assert rel_l2(tied.eval(toks), ref_tied.eval(toks)) < 1e-4
+    with pytest.raises(LiteNNHipError):
+        tied.eval(list(toks) * 2)  # 7 + 14 > 16 positions
+    tied.close()
+
+    with pytest.raises(LiteNNHipError, match="Missing GGUF tensor 'blk.0.ffn_up.weight'"):
+        hip.LLaMA.from_gguf(str(gw.llama_gguf(tmp_path / "miss.gguf", cfg, 11, skip=("ffn_up",))))
+    with pytest.raises(LiteNNHipError, match="Failed to open GGUF file"):
+        hip.LLaMA.from_gguf(str(tmp_path / "absent.gguf"))
