@@ -702,6 +702,87 @@ namespace litenn_hip
 			}
 		}
 
+		// ---- arg-max of one long row in two launches (the decoder's vocabulary) -------------------
+		// Many workgroups scan a chunk each; one wavefront merges their (value, index) pairs, stores
+		// the token and advances the decoder's device-side counters {past length, tokens emitted}.
+		constexpr int kArgmaxChunk = 2048;
+
+		__device__ __forceinline__ void argmax_take(float ov, int oi, float& best, int& best_i)
+		{
+			if (ov > best || (ov == best && oi < best_i))
+			{
+				best = ov;
+				best_i = oi;
+			}
+		}
+
+		__global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ x, int n,
+		                                                              float* __restrict__ pv, int* __restrict__ pi)
+		{
+			__shared__ float bv[4];
+			__shared__ int bi[4];
+			const int begin = blockIdx.x * kArgmaxChunk, end = min(n, begin + kArgmaxChunk);
+			float best = -INFINITY;
+			int best_i = 0x7fffffff;
+			for (int i = begin + threadIdx.x; i < end; i += 256)
+			{
+				const float v = x[i];
+				if (v > best || best_i == 0x7fffffff)
+				{
+					best = v;
+					best_i = i;
+				}
+			}
+			for (int off = 32; off > 0; off >>= 1)
+			{
+				argmax_take(__shfl_xor(best, off, 64), __shfl_xor(best_i, off, 64), best, best_i);
+			}
+			if ((threadIdx.x & 63) == 0)
+			{
+				bv[threadIdx.x >> 6] = best;
+				bi[threadIdx.x >> 6] = best_i;
+			}
+			__syncthreads();
+			if (threadIdx.x == 0)
+			{
+				for (int wv = 1; wv < 4; ++wv)
+				{
+					argmax_take(bv[wv], bi[wv], best, best_i);
+				}
+				pv[blockIdx.x] = best;
+				pi[blockIdx.x] = best_i;
+			}
+		}
+
+		// one wavefront; counters = {past length, tokens emitted}, out may be null
+		__global__ __launch_bounds__(64) void argmax_merge_step_kernel(const float* __restrict__ pv,
+		                                                                const int* __restrict__ pi, int blocks,
+		                                                                int32_t* __restrict__ next, int* counters,
+		                                                                int past_inc, int32_t* __restrict__ out)
+		{
+			float best = -INFINITY;
+			int best_i = 0x7fffffff;
+			for (int b = threadIdx.x; b < blocks; b += 64)
+			{
+				argmax_take(pv[b], pi[b], best, best_i);
+			}
+			for (int off = 32; off > 0; off >>= 1)
+			{
+				argmax_take(__shfl_xor(best, off, 64), __shfl_xor(best_i, off, 64), best, best_i);
+			}
+			if (threadIdx.x == 0)
+			{
+				const int32_t token = best_i == 0x7fffffff ? 0 : best_i;
+				*next = token;
+				if (out)
+				{
+					out[counters[1]] = token;
+					counters[1] += 1;
+				}
+				counters[0] += past_inc;
+			}
+		}
+
 		__global__ void add_int_kernel(int* p, int v) { *p += v; }
 		__global__ void set_int_kernel(int* p, int v) { *p = v; }
 	} // namespace
@@ -858,6 +939,24 @@ namespace litenn_hip
 	void launch_argmax(const float* x, size_t rows, size_t n, int32_t* out, hipStream_t s)
 	{
 		argmax_kernel<<<dim3(rows), dim3(1024), 0, s>>>(x, static_cast<int>(n), out);
+	}
+
+	// bytes of scratch launch_argmax_step needs for a row of n values
+	size_t argmax_step_scratch_bytes(size_t n)
+	{
+		return ((n + kArgmaxChunk - 1) / kArgmaxChunk) * (sizeof(float) + sizeof(int));
+	}
+
+	// next = arg-max of x[0 .. n) (first maximal index); out[counters[1]++] = next (when out is given);
+	// counters[0] += past_inc
+	void launch_argmax_step(const float* x, size_t n, void* scratch, int32_t* next, int* counters, int past_inc,
+	                        int32_t* out, hipStream_t s)
+	{
+		const int blocks = static_cast<int>((n + kArgmaxChunk - 1) / kArgmaxChunk);
+		float* pv = static_cast<float*>(scratch);
+		int* pi = reinterpret_cast<int*>(pv + blocks);
+		argmax_partial_kernel<<<dim3(blocks), dim3(256), 0, s>>>(x, static_cast<int>(n), pv, pi);
+		argmax_merge_step_kernel<<<dim3(1), dim3(64), 0, s>>>(pv, pi, blocks, next, counters, past_inc, out);
 	}
 
 	void launch_add_int(int* p, int v, hipStream_t s) { add_int_kernel<<<1, 1, 0, s>>>(p, v); }

@@ -44,21 +44,14 @@ namespace litenn_hip
 	                        float* out, size_t splits, float* partial, int* counters, hipStream_t s);
 	void launch_silu_mul(const float* gate, const float* up, float* y, size_t n, hipStream_t s);
 	void launch_argmax(const float* x, size_t rows, size_t n, int32_t* out, hipStream_t s);
+	size_t argmax_step_scratch_bytes(size_t n);
+	void launch_argmax_step(const float* x, size_t n, void* scratch, int32_t* next, int* counters, int past_inc,
+	                        int32_t* out, hipStream_t s);
 	bool launch_convert(int src_dtype, const void* src, size_t n, int dst_dtype, void* dst, hipStream_t s);
 
 	namespace
 	{
 		// counters[0] = past length, counters[1] = tokens emitted so far
-		__global__ void advance_kernel(int* counters, int past_inc, const int32_t* next, int32_t* out)
-		{
-			if (out)
-			{
-				out[counters[1]] = *next;
-				counters[1] += 1;
-			}
-			counters[0] += past_inc;
-		}
-
 		__global__ void set_counters_kernel(int* counters, int past, int emitted)
 		{
 			counters[0] = past;
@@ -101,6 +94,7 @@ struct litenn_hip_llama
 	float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *gate = nullptr,
 	      *gate2 = nullptr, *up = nullptr, *logits = nullptr;
 	void* xh = nullptr; // fp16 copy of a matmul's activations (multi-row path), 16-row padded
+	void* argmax_scratch = nullptr; // per-chunk (value, index) pairs of the vocabulary arg-max
 	std::vector<void*> owned; // device buffers freed with the model (tensors uploaded by the GGUF loader)
 	int32_t* d_tokens = nullptr;
 	int32_t* d_next = nullptr; // token produced by the last arg-max
@@ -466,6 +460,10 @@ extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* p
 	{
 		return bail(e);
 	}
+	if ((e = hipMalloc(&m->argmax_scratch, argmax_step_scratch_bytes(static_cast<size_t>(p.vocab_size)))) != hipSuccess)
+	{
+		return bail(e);
+	}
 	m->attn_splits = attn_splits(1, static_cast<size_t>(p.context_length), static_cast<size_t>(p.head_count));
 	if (m->attn_splits > 1)
 	{
@@ -522,7 +520,8 @@ extern "C" int litenn_hip_llama_free(litenn_hip_llama* m)
 		(void)hipFree(ptr);
 	}
 	void* singles[] = { m->cos_t, m->sin_t,      m->logits,       m->d_next,       m->d_out,
-	                    m->d_counters, m->d_err, m->attn_partial, m->attn_counters };
+	                    m->d_counters, m->d_err, m->attn_partial, m->attn_counters,
+	                    m->argmax_scratch };
 	for (void* ptr : singles)
 	{
 		if (ptr)
@@ -756,8 +755,8 @@ extern "C" int litenn_hip_llama_generate(litenn_hip_llama* m, const int32_t* pro
 	set_counters_kernel<<<1, 1, 0, s>>>(m->d_counters, m->past, 0);
 	GEN_TRY(hipEventRecord(ev[0], s));
 	forward(m, m->d_tokens, n_prompt, 1, flags);
-	launch_argmax(m->logits, 1, m->p.vocab_size, m->d_next, s);
-	advance_kernel<<<1, 1, 0, s>>>(m->d_counters, static_cast<int>(n_prompt), m->d_next, m->d_out);
+	launch_argmax_step(m->logits, m->p.vocab_size, m->argmax_scratch, m->d_next, m->d_counters,
+	                   static_cast<int>(n_prompt), m->d_out, s);
 	GEN_TRY(hipEventRecord(ev[1], s));
 	GEN_TRY(hipGetLastError());
 
@@ -774,8 +773,7 @@ extern "C" int litenn_hip_llama_generate(litenn_hip_llama* m, const int32_t* pro
 			if (ce == hipSuccess)
 			{
 				forward(m, m->d_next, 1, 1, flags);
-				launch_argmax(m->logits, 1, m->p.vocab_size, m->d_next, s);
-				advance_kernel<<<1, 1, 0, s>>>(m->d_counters, 1, m->d_next, m->d_out);
+				launch_argmax_step(m->logits, m->p.vocab_size, m->argmax_scratch, m->d_next, m->d_counters, 1, m->d_out, s);
 				ce = hipStreamEndCapture(s, &m->step_graph);
 			}
 			if (ce == hipSuccess)
@@ -798,8 +796,7 @@ extern "C" int litenn_hip_llama_generate(litenn_hip_llama* m, const int32_t* pro
 			else
 			{
 				forward(m, m->d_next, 1, 1, flags);
-				launch_argmax(m->logits, 1, m->p.vocab_size, m->d_next, s);
-				advance_kernel<<<1, 1, 0, s>>>(m->d_counters, 1, m->d_next, m->d_out);
+				launch_argmax_step(m->logits, m->p.vocab_size, m->argmax_scratch, m->d_next, m->d_counters, 1, m->d_out, s);
 			}
 		}
 	}
