@@ -171,3 +171,26 @@ def test_linear_group_residual_and_errors(hip, oracle):
         hip.linear_group(Q4_0, [wt, wt, wt], [n, n, n], k, hip.Tensor.from_numpy(x), silu_mul=True)
     with pytest.raises(hip.LiteNNHipError, match="single matrix"):
         hip.linear_group(Q4_0, [wt, wt], [n, n], k, hip.Tensor.from_numpy(x), residual=hip.Tensor.from_numpy(res))
+
+
+@pytest.mark.parametrize("fmt,n", [(Q6_K, 128256), (Q4_0, 32000)])
+def test_lm_head_shapes(hip, oracle, fmt, n):
+    """The vocabulary projections of BASELINE configs 5 and 4 at full size (431 MB / 74 MB)."""
+    assert run_case(hip, oracle, fmt, n, 4096, seed=n) <= TOL
+
+
+def test_gemv_properties_at_full_size(hip):
+    """Size-independent checks at the north-star shape: linearity in x, and y(e_k) = column k of the
+    dequantised matrix (so y over all one-hot inputs of a block reproduces litenn_hip_dequantize)."""
+    n, k = 14336, 4096
+    wq = hip.Tensor.from_numpy(synth.quant_weights(Q4_K, n, k, 8, 1))
+    y = lambda x: hip.mul_mat_q(Q4_K, wq, n, k, hip.Tensor.from_numpy(np.ascontiguousarray(x, np.float32))).numpy()
+    x1, x2 = synth.activations(1, k, 8, 2), synth.activations(1, k, 8, 3)
+    assert rel_l2(y(3.0 * x1 - x2), 3.0 * y(x1) - y(x2)) <= 1e-5
+    deq = hip.dequantize(Q4_K, wq, n, k).numpy()
+    for col in (0, 31, 32, 255, 256, 4095):
+        e = np.zeros((1, k), np.float32)
+        e[0, col] = 1.0
+        assert np.array_equal(y(e)[0], deq[:, col]), col
+    # all-ones input: row sums (f32 summation order differs: tolerance, not equality)
+    assert rel_l2(y(np.ones((1, k), np.float32))[0], deq.astype(np.float64).sum(axis=1).astype(np.float32)) <= 1e-5
