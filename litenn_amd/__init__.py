@@ -10,7 +10,8 @@ from .device import (HIP, DeviceTraits, HIPDeviceCount, IsHIPDeviceAvailable, Te
                      dequantize, get_rows_q, kv_append, linear_group, mul_mat_q, rmsnorm, rope_interleaved, silu_mul,
                      MATMUL_PRECISE)
 from .llama import LLaMA
+from .gguf import GGUFFile
 
 __all__ = ["formats", "synth", "LiteNNHipError", "LIB_PATH", "HIP", "DeviceTraits", "HIPDeviceCount",
            "IsHIPDeviceAvailable", "Tensor", "argmax", "attn_decode", "dequantize", "get_rows_q", "kv_append",
-           "mul_mat_q", "linear_group", "rmsnorm", "rope_interleaved", "silu_mul", "MATMUL_PRECISE", "LLaMA"]
+           "mul_mat_q", "linear_group", "rmsnorm", "rope_interleaved", "silu_mul", "MATMUL_PRECISE", "LLaMA", "GGUFFile"]
