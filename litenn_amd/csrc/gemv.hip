@@ -552,7 +552,10 @@ namespace litenn_hip
 		constexpr int kLdsUnitStride = 68;  // floats between the staged activations of consecutive units
 		constexpr int kXPerThread = 8;      // most 128-bit activation loads a thread issues while staging
 		constexpr int kMaxStreamRows = 64;  // most rows a wavefront of the streaming kernel owns (one per lane)
-		constexpr int kPrefetchRows = 3;    // rows a wavefront keeps in flight (= its LDS row slots)
+		// Rows a wavefront keeps in flight (= its LDS row slots).  Two rows of eight wavefronts on
+		// each of 256 CUs are about 9 MB, the card's bandwidth x latency product; deeper rings were
+		// measured slower, each extra slot by 5 - 8 % on a 33 MB launch.
+		constexpr int kPrefetchRows = 2;
 		constexpr size_t kStreamLdsLimit = 160 * 1024;
 
 #ifdef LITENN_GEMV_TRACE
