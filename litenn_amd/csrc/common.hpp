@@ -7,12 +7,20 @@
 #include <cstddef>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <string>
 
 #include "../../include/litenn_hip.h"
 
 namespace litenn_hip
 {
+	// integer tuning knob from the environment
+	inline int env_int(const char* name, int fallback)
+	{
+		const char* v = getenv(name);
+		return (v && *v) ? atoi(v) : fallback;
+	}
+
 	// ---- error reporting: status code + thread-local message ---------------
 	void set_error(const std::string& message);
 	int fail(const char* action, const std::string& message);

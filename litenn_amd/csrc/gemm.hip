@@ -10,18 +10,19 @@
 // range first (and its results scaled back), so the range of the activations does not matter;
 // LITENN_HIP_MATMUL_PRECISE selects the f32 GEMV path instead.
 //
-// Work split: a workgroup (WAVES wavefronts) owns 16 * WAVES * NG weight rows and BM activation
-// rows; a
-// wavefront owns NG groups of 16 weight rows and walks K in chunks of 256 (one K-quant
-// super-block, eight 32-element blocks).  Lane (r, g) = (lane % 16, lane / 16) decodes 64 of
-// the 256 elements of row r of each of its groups per chunk, eight per MFMA step, in whatever
-// order is cheapest for the format; the activation operand is read from LDS in the same order,
-// so the contraction is complete and no weight byte is decoded twice or staged in LDS.
-// The weights of chunk c + 1 are loaded while chunk c is multiplied; the fp16 activation tile
-// of the next chunk is staged into the second half of a double-buffered LDS tile.
+// Work split: a workgroup (WAVES wavefronts) owns 16 * WAVES * NG weight rows and 16 * MT
+// activation rows; a wavefront owns NG groups of 16 weight rows and walks K in chunks of 256 (one
+// K-quant super-block, eight 32-element blocks).  Lane (r, g) = (lane % 16, lane / 16) decodes 64
+// of the 256 elements of row r of each of its groups per chunk, eight per MFMA step, in whatever
+// order is cheapest for the format.  The activations are stored by the pre-pass in exactly that
+// order, as ready-made 1 KB MFMA fragments, so the contraction is complete, no weight byte is
+// decoded twice or staged in LDS, and an activation fragment is one lane-linear 128-bit access
+// everywhere.  Chunk c + 1 (activation tile by direct-to-LDS loads, weights into a second
+// register set) is fetched while chunk c is multiplied.
 #include "common.hpp"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace litenn_hip
 {
@@ -34,9 +35,14 @@ namespace litenn_hip
 		typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 		typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-		constexpr int kChunk = 256;          // K elements per step of the outer loop
-		// halves per activation row in LDS: rows stay 16-byte aligned and shift by 4 banks each
-		constexpr int kTileStride = 256 + 8;
+// Timing instrumentation, never set in a product build: -DLITENN_GEMM_KNOCKOUT=<bits> compiles a
+// kernel with parts switched off (its results are then wrong) so that what the remaining parts
+// cost can be measured: 1 activation staging, 2 weight loads, 4 the per-chunk barrier, 8 the
+// decode arithmetic, 16 the LDS fragment reads.
+#ifndef LITENN_GEMM_KNOCKOUT
+#define LITENN_GEMM_KNOCKOUT 0
+#endif
+		constexpr int kChunk = 256; // K elements per step of the outer loop
 
 		__device__ __forceinline__ uint32_t pack_f16(float a, float b)
 		{
@@ -112,6 +118,8 @@ namespace litenn_hip
 		struct Q4_0Frag
 		{
 			static constexpr int kChunkBytes = 8 * 18;
+			static constexpr int kFragValu = 19; // VALU instructions of one frag(), roughly
+			static constexpr bool kWideTile = true; // two row groups x eight activation tiles fit the registers
 			struct Raw { uint32_t w[9]; }; // blocks 2g and 2g+1: 36 bytes
 			struct Scale { float d0, d1; };
 			static __device__ __forceinline__ Raw load(const uint8_t* chunk, int g)
@@ -156,6 +164,8 @@ namespace litenn_hip
 		struct Q8_0Frag
 		{
 			static constexpr int kChunkBytes = 8 * 34;
+			static constexpr int kFragValu = 24;
+			static constexpr bool kWideTile = false;
 			struct Raw { uint32_t w[17]; }; // blocks 2g and 2g+1: 68 bytes
 			struct Scale { float d0, d1; };
 			static __device__ __forceinline__ Raw load(const uint8_t* chunk, int g)
@@ -204,6 +214,8 @@ namespace litenn_hip
 		struct Q4_KFrag
 		{
 			static constexpr int kChunkBytes = 144;
+			static constexpr int kFragValu = 17;
+			static constexpr bool kWideTile = true;
 			struct Raw { u32x4 h; uint32_t q[8]; }; // header (d, dmin, 12 scale bytes) + the 32 nibble bytes of group g
 			struct Scale { float s0, m0, s1, m1; }; // d*sc*2^24, -dmin*m of sub-block 2g; d*sc*2^20, -dmin*m of 2g+1
 			static __device__ __forceinline__ Raw load(const uint8_t* chunk, int g)
@@ -257,6 +269,8 @@ namespace litenn_hip
 		struct Q6_KFrag
 		{
 			static constexpr int kChunkBytes = 210;
+			static constexpr int kFragValu = 28;
+			static constexpr bool kWideTile = false;
 			// lane g = 2h + j covers l in [16j, 16j + 16) of half h: 16 bytes of each ql half-row,
 			// 16 bytes of qh, the four scales 8h + j + 2i and d
 			struct Raw { uint32_t la[4], lb[4], qh[4]; uint32_t sc[4]; uint32_t d; };
@@ -318,22 +332,35 @@ namespace litenn_hip
 			}
 		};
 
-		// ---- activations to fp16 -------------------------------------------------------------------
+		// ---- activations to fp16, in fragment order ----------------------------------------------------
 		// One workgroup per row.  Every row is scaled by a power of two so that its largest magnitude
 		// lands in [2^14, 2^15): nothing overflows fp16 whatever the activations' range, small rows keep
 		// full fp16 precision, and the scaling itself is exact; the GEMM multiplies the row's results by
 		// the inverse factor.  Rows m .. m_pad - 1 are zero padding.
-		__global__ __launch_bounds__(256) void to_half_kernel(const float* __restrict__ x, _Float16* __restrict__ xh,
+		//
+		// The fp16 rows are not stored row-major but as the GEMM consumes them: for every 16-row tile
+		// mt and 256-element chunk c, eight 1 KB fragments (one per MFMA step s), each holding for lane
+		// (r, g) the 8 halves of row 16 mt + r that pair with the format's weight fragment of that step
+		// (F::koff).  A fragment is then one lane-linear 128-bit read, in global memory and in LDS.
+		constexpr int kFragBytes = 1024;                // 64 lanes x 8 halves
+		constexpr int kChunkTileBytes = 8 * kFragBytes; // one 16-row tile of one chunk
+
+		template <typename F>
+		__global__ __launch_bounds__(256) void to_half_kernel(const float* __restrict__ x, uint8_t* __restrict__ xf,
 		                                                       float* __restrict__ unscale, int m, int k)
 		{
 			__shared__ float red[4];
 			const int row = blockIdx.x;
-			_Float16* dst = xh + static_cast<size_t>(row) * k;
+			const int chunks = k / kChunk;
+			const int mt = row >> 4, r = row & 15;
+			uint8_t* tile_row = xf + static_cast<size_t>(mt) * chunks * kChunkTileBytes + r * 16;
+			const int items = chunks * 32; // (chunk, step, lane group) triples of this row
 			if (row >= m)
 			{
-				for (int i = threadIdx.x * 8; i < k; i += 256 * 8)
+				for (int it = threadIdx.x; it < items; it += 256)
 				{
-					*reinterpret_cast<u32x4*>(dst + i) = u32x4{ 0u, 0u, 0u, 0u };
+					const int c = it >> 5, st = (it >> 2) & 7, g = it & 3;
+					*reinterpret_cast<u32x4*>(tile_row + (c * 8 + st) * kFragBytes + g * 256) = u32x4{ 0u, 0u, 0u, 0u };
 				}
 				if (threadIdx.x == 0)
 				{
@@ -360,13 +387,19 @@ namespace litenn_hip
 			{
 				shift = 14 - ilogbf(mx);
 			}
-			for (int i = threadIdx.x * 4; i < k; i += 256 * 4)
+			for (int it = threadIdx.x; it < items; it += 256)
 			{
-				const float4 v = *reinterpret_cast<const float4*>(src + i);
-				u32x2 out;
-				out.x = pack_f16(ldexpf(v.x, shift), ldexpf(v.y, shift));
-				out.y = pack_f16(ldexpf(v.z, shift), ldexpf(v.w, shift));
-				*reinterpret_cast<u32x2*>(dst + i) = out;
+				const int c = it >> 5, st = (it >> 2) & 7, g = it & 3;
+				int k0, k1;
+				F::koff(g, st, k0, k1);
+				const float4 v0 = *reinterpret_cast<const float4*>(src + c * kChunk + k0);
+				const float4 v1 = *reinterpret_cast<const float4*>(src + c * kChunk + k1);
+				u32x4 out;
+				out.x = pack_f16(ldexpf(v0.x, shift), ldexpf(v0.y, shift));
+				out.y = pack_f16(ldexpf(v0.z, shift), ldexpf(v0.w, shift));
+				out.z = pack_f16(ldexpf(v1.x, shift), ldexpf(v1.y, shift));
+				out.w = pack_f16(ldexpf(v1.z, shift), ldexpf(v1.w, shift));
+				*reinterpret_cast<u32x4*>(tile_row + (c * 8 + st) * kFragBytes + g * 256) = out;
 			}
 			if (threadIdx.x == 0)
 			{
@@ -375,27 +408,38 @@ namespace litenn_hip
 		}
 
 		// ---- the GEMM ---------------------------------------------------------------------------
-		// grid (ceil(N / (16 WAVES NG)), ceil(M_pad / BM)); block 64 WAVES.
-		template <typename F, int BM, int NG, int WAVES>
+		// grid (ceil(N / (16 WAVES NG)), ceil(M_tiles / MT)); block 64 WAVES; MT 16-row activation
+		// tiles and NG 16-row weight groups per wavefront.
+		//
+		// Per 256-element chunk the workgroup's MT activation tiles (MT x 8 KB, already in fragment
+		// order) are copied global -> LDS by direct loads, into the half of a double buffer the
+		// previous chunk is not using; the wavefront's weights of the next chunk are loaded into the
+		// idle one of two register sets at the same time.  Inside a chunk the eight MFMA steps are
+		// software-pipelined: while the NG x MT MFMAs of step s run, the activation fragments of step
+		// s + 1 are read from LDS and the weight fragments of step s + 1 are decoded, the three
+		// instruction streams interleaved by scheduling directives.  One barrier per chunk, before
+		// the last step reads the first fragments of the next chunk.
+		typedef __attribute__((address_space(3))) void* gemm_lds_ptr_t;
+		typedef const __attribute__((address_space(1))) void* gemm_global_ptr_t;
+
+		template <typename F, int MT, int NG, int WAVES>
 		__global__ __launch_bounds__(64 * WAVES) void gemm_q_kernel(const uint8_t* __restrict__ w,
-		                                                             const _Float16* __restrict__ xh,
+		                                                             const uint8_t* __restrict__ xf,
 		                                                             const float* __restrict__ unscale,
 		                                                             float* __restrict__ y,
 		                                                             const float* __restrict__ residual, int n, int k,
-		                                                             int m, int m_pad, size_t row_bytes)
+		                                                             int m, int m_tiles, size_t row_bytes)
 		{
 			constexpr int kThreads = 64 * WAVES;
-			constexpr int MT = BM / 16;                   // 16-row activation tiles
-			constexpr int tile_stride = kTileStride;
-			constexpr int kTileHalves = BM * tile_stride; // one buffer of the LDS tile
-			constexpr int kPieces = BM * 32;              // 16-byte pieces of one BM x 512 B tile
-			constexpr int kStageLoads = (kPieces + kThreads - 1) / kThreads;
-			extern __shared__ __attribute__((aligned(16))) _Float16 tile[]; // [2][BM][kTileStride]
+			constexpr int kTileBytes = MT * kChunkTileBytes; // one chunk of the workgroup's activations
+			constexpr int kStageLoads = kTileBytes / (kThreads * 16);
+			static_assert(kStageLoads >= 1 && kStageLoads * kThreads * 16 == kTileBytes, "tile / thread split");
+			extern __shared__ __attribute__((aligned(16))) uint8_t tile[]; // [2][kTileBytes]
 			const int lane = threadIdx.x & 63;
 			const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 			const int r = lane & 15, g = lane >> 4;
 			const int n_base = (blockIdx.x * WAVES + wave) * 16 * NG;
-			const int m_base = blockIdx.y * BM;
+			const int mt_base = blockIdx.y * MT;
 			const int chunks = k / kChunk;
 
 			const uint8_t* rows[NG];
@@ -406,32 +450,34 @@ namespace litenn_hip
 				rows[q] = w + static_cast<size_t>(min(n_base + 16 * q + r, n - 1)) * row_bytes;
 			}
 
-			// activation staging: thread t moves 16-byte pieces p = t, t + kThreads, ... of the tile
-			u32x4 stage[kStageLoads];
-			const auto stage_load = [&](int c) {
+			// activation staging: load i of wavefront `wave` moves the 1 KB piece i * WAVES + wave of
+			// the tile, lane l its bytes 16 l ..; tiles past the end re-read the last one.  The piece
+			// offsets are wavefront-uniform (scalar registers), only the lane offset is per lane.
+			uint32_t stage_off[kStageLoads];
+#pragma unroll
+			for (int i = 0; i < kStageLoads; ++i)
+			{
+				const int piece = i * WAVES + wave; // 1 KB pieces, 8 per 16-row tile
+				const int t = min(mt_base + (piece >> 3), m_tiles - 1);
+				stage_off[i] = static_cast<uint32_t>(t * chunks) * kChunkTileBytes + (piece & 7) * kFragBytes;
+			}
+			// Issued outside the compiler's view: it would otherwise treat the pending direct-to-LDS
+			// loads as possibly out-of-order returns and turn every later LDS wait of the chunk into a
+			// wait for everything.  The explicit vmcnt(0) before the chunk's barrier covers them.
+			const uint32_t lane_off = lane * 16;
+			const uint32_t tile_lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+			    (__attribute__((address_space(3))) const uint8_t*)(tile)));
+			const auto stage_issue = [&](int c, int buf) {
 #pragma unroll
 				for (int i = 0; i < kStageLoads; ++i)
 				{
-					const int p = threadIdx.x + kThreads * i;
-					if (kPieces % kThreads == 0 || p < kPieces)
-					{
-						const int row = p >> 5, piece = p & 31;
-						const int mm = min(m_base + row, m_pad - 1);
-						stage[i] =
-						    *reinterpret_cast<const u32x4*>(xh + static_cast<size_t>(mm) * k + c * kChunk + piece * 8);
-					}
-				}
-			};
-			const auto stage_store = [&](int buf) {
-#pragma unroll
-				for (int i = 0; i < kStageLoads; ++i)
-				{
-					const int p = threadIdx.x + kThreads * i;
-					if (kPieces % kThreads == 0 || p < kPieces)
-					{
-						const int row = p >> 5, piece = p & 31;
-						*reinterpret_cast<u32x4*>(tile + buf * kTileHalves + row * tile_stride + piece * 8) = stage[i];
-					}
+					const int piece = i * WAVES + wave;
+					const uint8_t* src = xf + (stage_off[i] + static_cast<uint32_t>(c) * kChunkTileBytes);
+					const uint32_t dst = tile_lds + buf * kTileBytes + piece * kFragBytes;
+					asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+					             :
+					             : "s"(dst), "v"(lane_off), "s"(src)
+					             : "memory", "m0");
 				}
 			};
 
@@ -446,48 +492,61 @@ namespace litenn_hip
 				}
 			}
 
-			// one 256-wide chunk: decode the lane's weights step by step, multiply against the tile
-			const auto multiply = [&](const typename F::Raw (&raw)[NG], int buf) {
-				typename F::Scale sc[NG];
+			half8 a_cur[NG], a_nxt[NG];
+			u32x4 b[MT]; // fragment t of the current step until its MFMAs are issued, then of the next
+			const uint8_t* lane_tile = tile + lane * 16;
+			const auto read_b = [&](int t, int buf, int s) {
+				b[t] = *reinterpret_cast<const u32x4*>(lane_tile + buf * kTileBytes + t * kChunkTileBytes + s * kFragBytes);
+			};
+			const auto decode = [&](half8 (&a)[NG], const typename F::Raw (&raw)[NG], const typename F::Scale (&sc)[NG],
+			                        int s) {
 #pragma unroll
 				for (int q = 0; q < NG; ++q)
 				{
-					sc[q] = F::prep(raw[q], g);
+					uint32_t pk[4];
+					F::frag(raw[q], sc[q], s, pk);
+					const u32x4 v = { pk[0], pk[1], pk[2], pk[3] };
+					a[q] = __builtin_bit_cast(half8, v);
 				}
-				const _Float16* xt = tile + buf * kTileHalves + r * tile_stride;
+			};
+			// the MFMAs of the current step; fragment t is refilled for step (buf, s) right after its
+			// last use (refill = false on the very last step)
+			const auto mfma_step = [&](bool refill, int buf, int s) {
 #pragma unroll
-				for (int s = 0; s < 8; ++s)
+				for (int t = 0; t < MT; ++t)
 				{
-					half8 a[NG];
+					const half8 bt = __builtin_bit_cast(half8, b[t]);
 #pragma unroll
 					for (int q = 0; q < NG; ++q)
 					{
-						uint32_t pk[4];
-						F::frag(raw[q], sc[q], s, pk);
-						const u32x4 v = { pk[0], pk[1], pk[2], pk[3] };
-						a[q] = __builtin_bit_cast(half8, v);
+						// D[i = weight row][j = activation row] += A[i][k] * B[k][j]
+						acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur[q], bt, acc[q][t], 0, 0, 0);
 					}
-					int k0, k1;
-					F::koff(g, s, k0, k1);
-#pragma unroll
-					for (int t = 0; t < MT; ++t)
+					if (refill)
 					{
-						const _Float16* xr = xt + t * 16 * tile_stride;
-						const u32x2 b0 = *reinterpret_cast<const u32x2*>(xr + k0);
-						const u32x2 b1 = *reinterpret_cast<const u32x2*>(xr + k1);
-						const u32x4 bv = { b0.x, b0.y, b1.x, b1.y };
-						const half8 b = __builtin_bit_cast(half8, bv);
-#pragma unroll
-						for (int q = 0; q < NG; ++q)
-						{
-							// D[i = weight row][j = activation row] += A[i][k] * B[k][j]
-							acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[q], b, acc[q][t], 0, 0, 0);
-						}
+						read_b(t, buf, s);
 					}
-					// keep the steps apart: left alone the scheduler hoists every LDS read of the chunk
-					// to the top and spills the accumulators
-					__builtin_amdgcn_sched_barrier(0);
 				}
+			};
+			const auto rotate = [&]() {
+#pragma unroll
+				for (int q = 0; q < NG; ++q)
+				{
+					a_cur[q] = a_nxt[q];
+				}
+			};
+			// spread the LDS reads and the decode arithmetic of a step between its MFMAs
+			const auto interleave = [&]() {
+				constexpr int kMfma = NG * MT;
+				constexpr int kValuPerTile = (F::kFragValu * NG + MT - 1) / MT;
+#pragma unroll
+				for (int t = 0; t < MT; ++t)
+				{
+					__builtin_amdgcn_sched_group_barrier(0x008, NG, 0);           // the MFMAs of one activation fragment
+					__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);            // its refill from LDS
+					__builtin_amdgcn_sched_group_barrier(0x002, kValuPerTile, 0); // a share of the decode arithmetic
+				}
+				(void)kMfma;
 			};
 			const auto load_raw = [&](typename F::Raw (&raw)[NG], int c) {
 #pragma unroll
@@ -496,50 +555,105 @@ namespace litenn_hip
 					raw[q] = F::load(rows[q] + static_cast<size_t>(c) * F::kChunkBytes, g);
 				}
 			};
+			const auto prep_all = [&](typename F::Scale (&sc)[NG], const typename F::Raw (&raw)[NG]) {
+#pragma unroll
+				for (int q = 0; q < NG; ++q)
+				{
+					sc[q] = F::prep(raw[q], g);
+				}
+			};
+			constexpr int kWaitAllLoads = 0x0F70; // s_waitcnt vmcnt(0), the other counters at their maxima
 
-			// Two register sets of raw weight bytes alternate, so no set is copied; within a phase
-			// the next activation tile is requested first and the next weights after it: the tile
-			// must be in LDS before the barrier, the weights only when the next phase starts.
+			// one chunk out of `cur`, fetching the next into `nxt`
+			const auto chunk = [&](auto has_next_tag, const typename F::Raw (&raw_cur)[NG],
+			                       const typename F::Scale (&sc_cur)[NG], typename F::Raw (&raw_nxt)[NG],
+			                       typename F::Scale (&sc_nxt)[NG], int c, int buf) {
+				constexpr bool has_next = decltype(has_next_tag)::value;
+				if (has_next)
+				{
+#if !(LITENN_GEMM_KNOCKOUT & 1)
+					stage_issue(c + 1, buf ^ 1);
+#endif
+#if !(LITENN_GEMM_KNOCKOUT & 2)
+					load_raw(raw_nxt, c + 1);
+#endif
+				}
+#pragma unroll
+				for (int s = 0; s < 7; ++s)
+				{
+#if !(LITENN_GEMM_KNOCKOUT & 8)
+					decode(a_nxt, raw_cur, sc_cur, s + 1);
+#endif
+					mfma_step(!(LITENN_GEMM_KNOCKOUT & 16), buf, s + 1);
+					interleave();
+					__builtin_amdgcn_sched_barrier(0);
+					rotate();
+				}
+				// Everything this wavefront requested at the top of the chunk has landed, every
+				// wavefront's LDS reads of this chunk have returned: after the barrier the next tile is
+				// complete and this one may be overwritten.
+				__builtin_amdgcn_s_waitcnt(kWaitAllLoads);
+#if !(LITENN_GEMM_KNOCKOUT & 4)
+				__syncthreads();
+#endif
+				if (has_next)
+				{
+#if !(LITENN_GEMM_KNOCKOUT & 2)
+					prep_all(sc_nxt, raw_nxt);
+#endif
+#if !(LITENN_GEMM_KNOCKOUT & 8)
+					decode(a_nxt, raw_nxt, sc_nxt, 0);
+#endif
+				}
+				mfma_step(has_next && !(LITENN_GEMM_KNOCKOUT & 16), buf ^ 1, 0);
+				if (has_next)
+				{
+					interleave();
+				}
+				__builtin_amdgcn_sched_barrier(0);
+				rotate();
+			};
+
 			typename F::Raw raw_a[NG], raw_b[NG];
+			typename F::Scale sc_a[NG], sc_b[NG];
+			stage_issue(0, 0);
 			load_raw(raw_a, 0);
-			stage_load(0);
-			stage_store(0);
+			__builtin_amdgcn_s_waitcnt(kWaitAllLoads);
 			__syncthreads();
-			// s_waitcnt vmcnt(0) (expcnt and lgkmcnt left at their maxima).  Placed before a phase
-			// requests anything new, it makes the phase's own weights (requested one phase earlier)
-			// the only loads waited for; without it the compiler waits for them after the new
-			// requests are queued, and the in-order counter then drains those too.
-			constexpr int kWaitAllLoads = 0x0F70;
-			for (int c = 0; c < chunks; c += 2)
+			prep_all(sc_a, raw_a);
+#pragma unroll
+			for (int t = 0; t < MT; ++t)
 			{
-				__builtin_amdgcn_s_waitcnt(kWaitAllLoads);
-				if (c + 1 < chunks)
-				{
-					stage_load(c + 1);
-					load_raw(raw_b, c + 1);
-				}
-				multiply(raw_a, 0);
-				if (c + 1 >= chunks)
-				{
-					break;
-				}
-				stage_store(1);
-				__syncthreads();
-				__builtin_amdgcn_s_waitcnt(kWaitAllLoads);
-				if (c + 2 < chunks)
-				{
-					stage_load(c + 2);
-					load_raw(raw_a, c + 2);
-				}
-				multiply(raw_b, 1);
-				if (c + 2 < chunks)
-				{
-					stage_store(0);
-				}
-				__syncthreads();
+				read_b(t, 0, 0);
+			}
+			decode(a_cur, raw_a, sc_a, 0);
+#if LITENN_GEMM_KNOCKOUT
+			load_raw(raw_b, 0);
+			prep_all(sc_b, raw_b);
+			decode(a_nxt, raw_a, sc_a, 1);
+#endif
+			// chunks come in pairs (one per register set and LDS half); the last one fetches nothing
+			using std::false_type;
+			using std::true_type;
+			int c = 0;
+			for (; c + 2 < chunks; c += 2)
+			{
+				chunk(true_type{}, raw_a, sc_a, raw_b, sc_b, c, 0);
+				chunk(true_type{}, raw_b, sc_b, raw_a, sc_a, c + 1, 1);
+			}
+			if (c + 2 == chunks)
+			{
+				chunk(true_type{}, raw_a, sc_a, raw_b, sc_b, c, 0);
+				chunk(false_type{}, raw_b, sc_b, raw_a, sc_a, c + 1, 1);
+			}
+			else
+			{
+				chunk(false_type{}, raw_a, sc_a, raw_b, sc_b, c, 0);
 			}
 
 			// D layout: lane holds activation row j = lane % 16 and weight rows 4 (lane / 16) + 0..3
+			const bool vec_ok = (n & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 &&
+			                    (!residual || (reinterpret_cast<uintptr_t>(residual) & 15) == 0);
 #pragma unroll
 			for (int q = 0; q < NG; ++q)
 			{
@@ -547,19 +661,32 @@ namespace litenn_hip
 #pragma unroll
 				for (int t = 0; t < MT; ++t)
 				{
-					const int mm = m_base + 16 * t + r;
+					const int mm = (mt_base + t) * 16 + r;
 					if (mm < m)
 					{
 						float* dst = y + static_cast<size_t>(mm) * n + n0;
 						const float* res = residual ? residual + static_cast<size_t>(mm) * n + n0 : nullptr;
 						const float us = unscale[mm];
 						const float vals[4] = { acc[q][t].x * us, acc[q][t].y * us, acc[q][t].z * us, acc[q][t].w * us };
-#pragma unroll
-						for (int e = 0; e < 4; ++e)
+						if (vec_ok && n0 + 3 < n)
 						{
-							if (n0 + e < n)
+							float4 out = { vals[0], vals[1], vals[2], vals[3] };
+							if (res)
 							{
-								dst[e] = res ? res[e] + vals[e] : vals[e];
+								const float4 rv = *reinterpret_cast<const float4*>(res);
+								out.x += rv.x, out.y += rv.y, out.z += rv.z, out.w += rv.w;
+							}
+							*reinterpret_cast<float4*>(dst) = out;
+						}
+						else
+						{
+#pragma unroll
+							for (int e = 0; e < 4; ++e)
+							{
+								if (n0 + e < n)
+								{
+									dst[e] = res ? res[e] + vals[e] : vals[e];
+								}
 							}
 						}
 					}
@@ -567,53 +694,74 @@ namespace litenn_hip
 			}
 		}
 
-		template <typename F, int BM, int NG, int WAVES>
-		void launch_variant(const uint8_t* w, const _Float16* xh, const float* unscale, float* y, const float* residual,
-		                    int n, int k, int m, int m_pad, size_t row_bytes, hipStream_t stream)
+		template <typename F, int MT, int NG, int WAVES>
+		void launch_variant(const uint8_t* w, const uint8_t* xf, const float* unscale, float* y, const float* residual,
+		                    int n, int k, int m, int m_tiles, size_t row_bytes, hipStream_t stream)
 		{
-			constexpr size_t lds = sizeof(_Float16) * 2 * BM * kTileStride;
+			constexpr size_t lds = 2 * MT * kChunkTileBytes;
 			static const hipError_t attr =
-			    hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_q_kernel<F, BM, NG, WAVES>),
+			    hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_q_kernel<F, MT, NG, WAVES>),
 			                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
 			(void)attr;
 			constexpr int bn = 16 * WAVES * NG;
-			const dim3 grid((n + bn - 1) / bn, (m_pad + BM - 1) / BM);
-			gemm_q_kernel<F, BM, NG, WAVES><<<grid, dim3(64 * WAVES), lds, stream>>>(w, xh, unscale, y, residual, n, k, m,
-			                                                                        m_pad, row_bytes);
+			const dim3 grid((n + bn - 1) / bn, (m_tiles + MT - 1) / MT);
+			gemm_q_kernel<F, MT, NG, WAVES><<<grid, dim3(64 * WAVES), lds, stream>>>(w, xf, unscale, y, residual, n, k, m,
+			                                                                        m_tiles, row_bytes);
 		}
 
-		// Tile choice, from measurement on the MI355X (K = 4096; N = 14336 and 4096; M = 16 .. 512):
-		// the kernel is bound by the LDS reads of the activation operand and by latency, not by the
-		// matrix cores, so what pays is several small workgroups per CU (64-row activation tiles at
-		// most) and two row groups per wavefront (each activation fragment feeds two MFMAs) once the
-		// batch is large enough to keep every CU busy that way.
+		// Tile choice: MT activation tiles per workgroup so that a weight is decoded as few times as
+		// possible (MT = 8 takes 128 KB of LDS, so eight wavefronts share it); two weight groups per
+		// wavefront (each activation fragment read from LDS feeds two MFMAs) when that still leaves
+		// every CU a workgroup.
 		template <typename F>
-		void launch_format(const uint8_t* w, const _Float16* xh, const float* unscale, float* y, const float* residual,
-		                   int n, int k, int m, int m_pad, size_t row_bytes, int cus, hipStream_t stream)
+		void launch_format(const uint8_t* w, const uint8_t* xf, const float* unscale, float* y, const float* residual,
+		                   int n, int k, int m, int m_tiles, size_t row_bytes, int cus, hipStream_t stream)
 		{
-			const auto blocks = [&](int bm, int bn) {
-				return static_cast<long>((n + bn - 1) / bn) * ((m_pad + bm - 1) / bm);
+			const auto blocks = [&](int mt, int bn) {
+				return static_cast<long>((n + bn - 1) / bn) * ((m_tiles + mt - 1) / mt);
 			};
-#define LITENN_GEMM_ARGS w, xh, unscale, y, residual, n, k, m, m_pad, row_bytes, stream
-			if (m_pad >= 128)
+			static const int forced = env_int("LITENN_HIP_GEMM_TILE", 0); // MT * 100 + NG * 10 + WAVES
+#define LITENN_GEMM_ARGS w, xf, unscale, y, residual, n, k, m, m_tiles, row_bytes, stream
+#define LITENN_GEMM_CASE(MT_, NG_, WV_)                                                                              \
+	if (pick == MT_ * 100 + NG_ * 10 + WV_)                                                                        \
+	{                                                                                                              \
+		launch_variant<F, MT_, NG_, WV_>(LITENN_GEMM_ARGS);                                                        \
+		return;                                                                                                    \
+	}
+			int pick = forced;
+			if (pick == 0)
 			{
-				if (blocks(64, 128) >= 2 * cus)
+				// measured on the MI355X (K = 4096, N = 4096 and 14336, M = 16 .. 512): the widest tile
+				// wins once it nearly fills the card, otherwise the tallest single-group tile that
+				// still gives every CU a workgroup
+				if (m_tiles >= 8 && F::kWideTile && 5 * blocks(8, 256) >= 4 * cus)
 				{
-					launch_variant<F, 64, 2, 4>(LITENN_GEMM_ARGS);
+					pick = 828;
+				}
+				else if (m_tiles >= 8 && blocks(8, 128) >= cus)
+				{
+					pick = 818;
+				}
+				else if (m_tiles >= 4 && blocks(4, 64) >= cus)
+				{
+					pick = 414;
+				}
+				else if (m_tiles >= 2 && blocks(2, 64) >= cus)
+				{
+					pick = 214;
 				}
 				else
 				{
-					launch_variant<F, 64, 1, 4>(LITENN_GEMM_ARGS);
+					pick = 114;
 				}
 			}
-			else if (m_pad >= 32)
-			{
-				launch_variant<F, 32, 1, 4>(LITENN_GEMM_ARGS);
-			}
-			else
-			{
-				launch_variant<F, 16, 1, 4>(LITENN_GEMM_ARGS);
-			}
+			LITENN_GEMM_CASE(8, 2, 8)
+			LITENN_GEMM_CASE(8, 1, 8)
+			LITENN_GEMM_CASE(4, 1, 4)
+			LITENN_GEMM_CASE(2, 1, 4)
+			LITENN_GEMM_CASE(1, 1, 4)
+			launch_variant<F, 1, 1, 4>(LITENN_GEMM_ARGS);
+#undef LITENN_GEMM_CASE
 #undef LITENN_GEMM_ARGS
 		}
 	} // namespace
@@ -640,7 +788,7 @@ namespace litenn_hip
 		const uintptr_t w_align = fmt == LITENN_FMT_Q6_K ? 2 : 16;
 		if (k % kChunk != 0 || rb == 0 || reinterpret_cast<uintptr_t>(wq) % w_align != 0 ||
 		    reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(scratch_halves) % 16 != 0 ||
-		    !scratch_halves)
+		    !scratch_halves || 2 * ((m + 15) / 16 * 16) * k >= (size_t{ 1 } << 32)) // 32-bit tile offsets
 		{
 			return false;
 		}
@@ -654,19 +802,30 @@ namespace litenn_hip
 			return prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
 		}();
 		const size_t m_pad = (m + 15) / 16 * 16;
-		_Float16* xh = static_cast<_Float16*>(scratch_halves);
-		float* unscale = reinterpret_cast<float*>(xh + m_pad * k); // 4-byte aligned: m_pad * k is even
-		to_half_kernel<<<dim3(static_cast<unsigned>(m_pad)), dim3(256), 0, stream>>>(x, xh, unscale, static_cast<int>(m),
-		                                                                            static_cast<int>(k));
+		uint8_t* xf = static_cast<uint8_t*>(scratch_halves);
+		float* unscale = reinterpret_cast<float*>(xf + 2 * m_pad * k); // after the fp16 tiles
 		const uint8_t* w = static_cast<const uint8_t*>(wq);
 		const int ni = static_cast<int>(n), ki = static_cast<int>(k), mi = static_cast<int>(m),
-		          mp = static_cast<int>(m_pad);
+		          mt = static_cast<int>(m_pad / 16);
+		const dim3 rows_grid(static_cast<unsigned>(m_pad));
 		switch (fmt)
 		{
-		case LITENN_FMT_Q4_0: launch_format<Q4_0Frag>(w, xh, unscale, y, residual, ni, ki, mi, mp, rb, cus, stream); break;
-		case LITENN_FMT_Q8_0: launch_format<Q8_0Frag>(w, xh, unscale, y, residual, ni, ki, mi, mp, rb, cus, stream); break;
-		case LITENN_FMT_Q4_K: launch_format<Q4_KFrag>(w, xh, unscale, y, residual, ni, ki, mi, mp, rb, cus, stream); break;
-		default: launch_format<Q6_KFrag>(w, xh, unscale, y, residual, ni, ki, mi, mp, rb, cus, stream); break;
+		case LITENN_FMT_Q4_0:
+			to_half_kernel<Q4_0Frag><<<rows_grid, dim3(256), 0, stream>>>(x, xf, unscale, mi, ki);
+			launch_format<Q4_0Frag>(w, xf, unscale, y, residual, ni, ki, mi, mt, rb, cus, stream);
+			break;
+		case LITENN_FMT_Q8_0:
+			to_half_kernel<Q8_0Frag><<<rows_grid, dim3(256), 0, stream>>>(x, xf, unscale, mi, ki);
+			launch_format<Q8_0Frag>(w, xf, unscale, y, residual, ni, ki, mi, mt, rb, cus, stream);
+			break;
+		case LITENN_FMT_Q4_K:
+			to_half_kernel<Q4_KFrag><<<rows_grid, dim3(256), 0, stream>>>(x, xf, unscale, mi, ki);
+			launch_format<Q4_KFrag>(w, xf, unscale, y, residual, ni, ki, mi, mt, rb, cus, stream);
+			break;
+		default:
+			to_half_kernel<Q6_KFrag><<<rows_grid, dim3(256), 0, stream>>>(x, xf, unscale, mi, ki);
+			launch_format<Q6_KFrag>(w, xf, unscale, y, residual, ni, ki, mi, mt, rb, cus, stream);
+			break;
 		}
 		return true;
 	}

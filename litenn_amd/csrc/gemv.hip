@@ -963,7 +963,7 @@ namespace litenn_hip
 			}
 			for (; r < count; ++r) // the last rows: nothing left to request
 			{
-				wait_rows_outstanding_dyn<PD - 2>(count - 1 - r, loads_per_row);
+				wait_rows_outstanding_dyn<(PD >= 2 ? PD - 2 : 0)>(count - 1 - r, loads_per_row);
 				consume(r);
 				slot_off = slot_off + U::kSliceBytes == PD * U::kSliceBytes ? 0u : slot_off + U::kSliceBytes;
 			}
@@ -1247,12 +1247,6 @@ namespace litenn_hip
 			{
 				out[static_cast<size_t>(blockIdx.x) * k + i] = generic_elem(fmt, rp, i);
 			}
-		}
-
-		int env_int(const char* name, int fallback)
-		{
-			const char* v = getenv(name);
-			return (v && *v) ? atoi(v) : fallback;
 		}
 
 		int compute_units()
