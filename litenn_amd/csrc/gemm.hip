@@ -35,13 +35,6 @@ namespace litenn_hip
 		typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 		typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-// Timing instrumentation, never set in a product build: -DLITENN_GEMM_KNOCKOUT=<bits> compiles a
-// kernel with parts switched off (its results are then wrong) so that what the remaining parts
-// cost can be measured: 1 activation staging, 2 weight loads, 4 the per-chunk barrier, 8 the
-// decode arithmetic, 16 the LDS fragment reads.
-#ifndef LITENN_GEMM_KNOCKOUT
-#define LITENN_GEMM_KNOCKOUT 0
-#endif
 		constexpr int kChunk = 256; // K elements per step of the outer loop
 
 		__device__ __forceinline__ uint32_t pack_f16(float a, float b)
@@ -51,15 +44,23 @@ namespace litenn_hip
 			return __builtin_bit_cast(uint32_t, h);
 		}
 
-		// unaligned little-endian reads from global memory (blocks are only 2-byte aligned)
-		__device__ __forceinline__ uint32_t ld_u32(const uint8_t* p)
+		// the weight bytes reach the decoders through LDS
+		typedef const __attribute__((address_space(3))) uint8_t* lds_bytes_t;
+		typedef const __attribute__((address_space(3))) u32x4* lds_u32x4_t;
+
+		// little-endian reads at 2-byte alignment (K-quant blocks are only that aligned)
+		__device__ __forceinline__ uint32_t ld_u32(lds_bytes_t p)
 		{
 			typedef uint32_t u32_a2 __attribute__((aligned(2)));
-			return *reinterpret_cast<const u32_a2*>(p);
+			return *(const __attribute__((address_space(3))) u32_a2*)(p);
 		}
-		__device__ __forceinline__ uint32_t ld_u16(const uint8_t* p)
+		__device__ __forceinline__ uint32_t ld_u32_aligned(lds_bytes_t p)
 		{
-			return *reinterpret_cast<const uint16_t*>(p);
+			return *(const __attribute__((address_space(3))) uint32_t*)(p);
+		}
+		__device__ __forceinline__ uint32_t ld_u16(lds_bytes_t p)
+		{
+			return *(const __attribute__((address_space(3))) uint16_t*)(p);
 		}
 
 		// ---- per-format decoders -----------------------------------------------------------
@@ -119,17 +120,18 @@ namespace litenn_hip
 		{
 			static constexpr int kChunkBytes = 8 * 18;
 			static constexpr int kFragValu = 19; // VALU instructions of one frag(), roughly
-			static constexpr bool kWideTile = true; // two row groups x eight activation tiles fit the registers
+			static constexpr bool kAligned16 = true; // chunks start on 16-byte boundaries
+			static constexpr bool kWideTile = true;  // two row groups x eight activation tiles fit the registers
 			struct Raw { uint32_t w[9]; }; // blocks 2g and 2g+1: 36 bytes
 			struct Scale { float d0, d1; };
-			static __device__ __forceinline__ Raw load(const uint8_t* chunk, int g)
+			static __device__ __forceinline__ Raw load(lds_bytes_t chunk, int g)
 			{
 				Raw r;
-				const uint8_t* p = chunk + 36 * g; // 4-byte aligned: rows are 16-byte aligned
+				lds_bytes_t p = chunk + 36 * g; // 4-byte aligned: rows are 16-byte aligned
 #pragma unroll
 				for (int i = 0; i < 9; ++i)
 				{
-					r.w[i] = ld_u32(p + 4 * i);
+					r.w[i] = ld_u32_aligned(p + 4 * i);
 				}
 				return r;
 			}
@@ -165,17 +167,18 @@ namespace litenn_hip
 		{
 			static constexpr int kChunkBytes = 8 * 34;
 			static constexpr int kFragValu = 24;
+			static constexpr bool kAligned16 = true;
 			static constexpr bool kWideTile = false;
 			struct Raw { uint32_t w[17]; }; // blocks 2g and 2g+1: 68 bytes
 			struct Scale { float d0, d1; };
-			static __device__ __forceinline__ Raw load(const uint8_t* chunk, int g)
+			static __device__ __forceinline__ Raw load(lds_bytes_t chunk, int g)
 			{
 				Raw r;
-				const uint8_t* p = chunk + 68 * g;
+				lds_bytes_t p = chunk + 68 * g;
 #pragma unroll
 				for (int i = 0; i < 17; ++i)
 				{
-					r.w[i] = ld_u32(p + 4 * i);
+					r.w[i] = ld_u32_aligned(p + 4 * i);
 				}
 				return r;
 			}
@@ -215,15 +218,16 @@ namespace litenn_hip
 		{
 			static constexpr int kChunkBytes = 144;
 			static constexpr int kFragValu = 17;
+			static constexpr bool kAligned16 = true;
 			static constexpr bool kWideTile = true;
 			struct Raw { u32x4 h; uint32_t q[8]; }; // header (d, dmin, 12 scale bytes) + the 32 nibble bytes of group g
 			struct Scale { float s0, m0, s1, m1; }; // d*sc*2^24, -dmin*m of sub-block 2g; d*sc*2^20, -dmin*m of 2g+1
-			static __device__ __forceinline__ Raw load(const uint8_t* chunk, int g)
+			static __device__ __forceinline__ Raw load(lds_bytes_t chunk, int g)
 			{
 				Raw r;
-				r.h = *reinterpret_cast<const u32x4*>(chunk);
-				const u32x4 a = *reinterpret_cast<const u32x4*>(chunk + 16 + 32 * g);
-				const u32x4 b = *reinterpret_cast<const u32x4*>(chunk + 32 + 32 * g);
+				r.h = *(lds_u32x4_t)(chunk);
+				const u32x4 a = *(lds_u32x4_t)(chunk + 16 + 32 * g);
+				const u32x4 b = *(lds_u32x4_t)(chunk + 32 + 32 * g);
 				r.q[0] = a.x, r.q[1] = a.y, r.q[2] = a.z, r.q[3] = a.w;
 				r.q[4] = b.x, r.q[5] = b.y, r.q[6] = b.z, r.q[7] = b.w;
 				return r;
@@ -270,17 +274,18 @@ namespace litenn_hip
 		{
 			static constexpr int kChunkBytes = 210;
 			static constexpr int kFragValu = 28;
+			static constexpr bool kAligned16 = false; // 210-byte blocks: 2-byte aligned
 			static constexpr bool kWideTile = false;
 			// lane g = 2h + j covers l in [16j, 16j + 16) of half h: 16 bytes of each ql half-row,
 			// 16 bytes of qh, the four scales 8h + j + 2i and d
 			struct Raw { uint32_t la[4], lb[4], qh[4]; uint32_t sc[4]; uint32_t d; };
 			struct Scale { float s[4], b[4]; }; // d*scale*2^24 and -32*d*scale per quarter
-			static __device__ __forceinline__ Raw load(const uint8_t* chunk, int g)
+			static __device__ __forceinline__ Raw load(lds_bytes_t chunk, int g)
 			{
 				const int h = g >> 1, j = g & 1;
 				Raw r;
-				const uint8_t* ql = chunk + 64 * h + 16 * j;
-				const uint8_t* qh = chunk + 128 + 32 * h + 16 * j;
+				lds_bytes_t ql = chunk + 64 * h + 16 * j;
+				lds_bytes_t qh = chunk + 128 + 32 * h + 16 * j;
 #pragma unroll
 				for (int i = 0; i < 4; ++i)
 				{
@@ -288,7 +293,7 @@ namespace litenn_hip
 					r.lb[i] = ld_u32(ql + 32 + 4 * i);
 					r.qh[i] = ld_u32(qh + 4 * i);
 				}
-				const uint8_t* sc = chunk + 192 + 8 * h + j;
+				lds_bytes_t sc = chunk + 192 + 8 * h + j;
 #pragma unroll
 				for (int i = 0; i < 4; ++i)
 				{
@@ -369,11 +374,36 @@ namespace litenn_hip
 				return;
 			}
 			const float* src = x + static_cast<size_t>(row) * k;
+			// The thread's share of the row stays in registers between the maximum and the conversion
+			// (up to kHeld items of 8 elements; longer rows re-read the rest).
+			constexpr int kHeld = 8;
+			float4 held[kHeld][2];
 			float mx = 0.0f;
-			for (int i = threadIdx.x * 4; i < k; i += 256 * 4)
+#pragma unroll
+			for (int u = 0; u < kHeld; ++u)
 			{
-				const float4 v = *reinterpret_cast<const float4*>(src + i);
-				mx = fmaxf(fmaxf(mx, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
+				const int it = threadIdx.x + 256 * u;
+				if (it < items)
+				{
+					const int c = it >> 5, st = (it >> 2) & 7, g = it & 3;
+					int k0, k1;
+					F::koff(g, st, k0, k1);
+					held[u][0] = *reinterpret_cast<const float4*>(src + c * kChunk + k0);
+					held[u][1] = *reinterpret_cast<const float4*>(src + c * kChunk + k1);
+					const float4 a = held[u][0], b = held[u][1];
+					mx = fmaxf(mx, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
+					mx = fmaxf(mx, fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w))));
+				}
+			}
+			for (int it = threadIdx.x + 256 * kHeld; it < items; it += 256)
+			{
+				const int c = it >> 5, st = (it >> 2) & 7, g = it & 3;
+				int k0, k1;
+				F::koff(g, st, k0, k1);
+				const float4 a = *reinterpret_cast<const float4*>(src + c * kChunk + k0);
+				const float4 b = *reinterpret_cast<const float4*>(src + c * kChunk + k1);
+				mx = fmaxf(mx, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
+				mx = fmaxf(mx, fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w))));
 			}
 			mx = wave_max(mx);
 			if ((threadIdx.x & 63) == 0)
@@ -387,19 +417,31 @@ namespace litenn_hip
 			{
 				shift = 14 - ilogbf(mx);
 			}
-			for (int it = threadIdx.x; it < items; it += 256)
-			{
+			const auto emit = [&](int it, const float4& v0, const float4& v1) {
 				const int c = it >> 5, st = (it >> 2) & 7, g = it & 3;
-				int k0, k1;
-				F::koff(g, st, k0, k1);
-				const float4 v0 = *reinterpret_cast<const float4*>(src + c * kChunk + k0);
-				const float4 v1 = *reinterpret_cast<const float4*>(src + c * kChunk + k1);
 				u32x4 out;
 				out.x = pack_f16(ldexpf(v0.x, shift), ldexpf(v0.y, shift));
 				out.y = pack_f16(ldexpf(v0.z, shift), ldexpf(v0.w, shift));
 				out.z = pack_f16(ldexpf(v1.x, shift), ldexpf(v1.y, shift));
 				out.w = pack_f16(ldexpf(v1.z, shift), ldexpf(v1.w, shift));
 				*reinterpret_cast<u32x4*>(tile_row + (c * 8 + st) * kFragBytes + g * 256) = out;
+			};
+#pragma unroll
+			for (int u = 0; u < kHeld; ++u)
+			{
+				const int it = threadIdx.x + 256 * u;
+				if (it < items)
+				{
+					emit(it, held[u][0], held[u][1]);
+				}
+			}
+			for (int it = threadIdx.x + 256 * kHeld; it < items; it += 256)
+			{
+				const int c = it >> 5, st = (it >> 2) & 7, g = it & 3;
+				int k0, k1;
+				F::koff(g, st, k0, k1);
+				emit(it, *reinterpret_cast<const float4*>(src + c * kChunk + k0),
+				     *reinterpret_cast<const float4*>(src + c * kChunk + k1));
 			}
 			if (threadIdx.x == 0)
 			{
@@ -411,16 +453,39 @@ namespace litenn_hip
 		// grid (ceil(N / (16 WAVES NG)), ceil(M_tiles / MT)); block 64 WAVES; MT 16-row activation
 		// tiles and NG 16-row weight groups per wavefront.
 		//
-		// Per 256-element chunk the workgroup's MT activation tiles (MT x 8 KB, already in fragment
-		// order) are copied global -> LDS by direct loads, into the half of a double buffer the
-		// previous chunk is not using; the wavefront's weights of the next chunk are loaded into the
-		// idle one of two register sets at the same time.  Inside a chunk the eight MFMA steps are
-		// software-pipelined: while the NG x MT MFMAs of step s run, the activation fragments of step
-		// s + 1 are read from LDS and the weight fragments of step s + 1 are decoded, the three
-		// instruction streams interleaved by scheduling directives.  One barrier per chunk, before
-		// the last step reads the first fragments of the next chunk.
-		typedef __attribute__((address_space(3))) void* gemm_lds_ptr_t;
-		typedef const __attribute__((address_space(1))) void* gemm_global_ptr_t;
+		// Everything reaches the CU by direct-to-LDS loads, issued with inline assembly and waited for
+		// with explicit vmcnt counts (the compiler, seeing such loads, would turn every later LDS wait
+		// into a wait for everything outstanding):
+		//   * activations: half a chunk (four MFMA steps, MT x 4 KB, already in fragment order) per
+		//     buffer, three buffers, so the half needed next but one is requested while the current
+		//     one is multiplied;
+		//   * weights: each wavefront has one private slot holding the raw blocks of its 16 NG rows for
+		//     one chunk (rows back to back, as 16-byte pieces from a 16-byte aligned start), requested
+		//     for chunk c + 1 as soon as chunk c's bytes have been moved to registers.
+		// Inside a chunk the eight MFMA steps are software-pipelined: while the NG x MT MFMAs of step s
+		// run, every activation fragment is refilled from LDS for step s + 1 right after its last use
+		// and the weight fragments of step s + 1 are decoded, the three instruction streams
+		// interleaved by scheduling directives.  One barrier per half chunk: it publishes the next
+		// half's activations and frees the buffer of the previous one.
+		template <int N>
+		__device__ __forceinline__ void vm_wait()
+		{
+			asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+		}
+
+		template <typename F>
+		constexpr int weight_pieces() // 16-byte pieces per row and chunk in the LDS slot
+		{
+			return F::kAligned16 ? F::kChunkBytes / 16 : (F::kChunkBytes + 14 + 15) / 16;
+		}
+
+		constexpr size_t kLdsLimit = 160 * 1024;
+
+		template <typename F, int MT, int NG, int WAVES>
+		constexpr size_t gemm_lds_bytes()
+		{
+			return 3 * MT * 4 * kFragBytes + static_cast<size_t>(WAVES) * NG * 16 * 16 * weight_pieces<F>();
+		}
 
 		template <typename F, int MT, int NG, int WAVES>
 		__global__ __launch_bounds__(64 * WAVES) void gemm_q_kernel(const uint8_t* __restrict__ w,
@@ -430,56 +495,92 @@ namespace litenn_hip
 		                                                             const float* __restrict__ residual, int n, int k,
 		                                                             int m, int m_tiles, size_t row_bytes)
 		{
-			constexpr int kThreads = 64 * WAVES;
-			constexpr int kTileBytes = MT * kChunkTileBytes; // one chunk of the workgroup's activations
-			constexpr int kStageLoads = kTileBytes / (kThreads * 16);
-			static_assert(kStageLoads >= 1 && kStageLoads * kThreads * 16 == kTileBytes, "tile / thread split");
-			extern __shared__ __attribute__((aligned(16))) uint8_t tile[]; // [2][kTileBytes]
+			constexpr int kHalfBytes = MT * 4 * kFragBytes; // one activation buffer: four steps of MT tiles
+			constexpr int kXLoads = MT * 4 / WAVES;         // 1 KB pieces a wavefront moves per half
+			static_assert(kXLoads >= 1 && kXLoads * WAVES == MT * 4, "activation pieces / wavefront split");
+			constexpr int P = weight_pieces<F>();
+			constexpr int kRowStride = 16 * P;              // bytes of one row's chunk in the slot
+			constexpr int kSlotBytes = NG * 16 * kRowStride;
+			constexpr int kWLoads = (NG * 16 * P + 63) / 64;
+			extern __shared__ __attribute__((aligned(16))) uint8_t lds[]; // [3][kHalfBytes][WAVES][kSlotBytes]
 			const int lane = threadIdx.x & 63;
 			const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 			const int r = lane & 15, g = lane >> 4;
 			const int n_base = (blockIdx.x * WAVES + wave) * 16 * NG;
 			const int mt_base = blockIdx.y * MT;
 			const int chunks = k / kChunk;
-
-			const uint8_t* rows[NG];
-#pragma unroll
-			for (int q = 0; q < NG; ++q)
-			{
-				// rows past the end re-read the last row; their results are never stored
-				rows[q] = w + static_cast<size_t>(min(n_base + 16 * q + r, n - 1)) * row_bytes;
-			}
-
-			// activation staging: load i of wavefront `wave` moves the 1 KB piece i * WAVES + wave of
-			// the tile, lane l its bytes 16 l ..; tiles past the end re-read the last one.  The piece
-			// offsets are wavefront-uniform (scalar registers), only the lane offset is per lane.
-			uint32_t stage_off[kStageLoads];
-#pragma unroll
-			for (int i = 0; i < kStageLoads; ++i)
-			{
-				const int piece = i * WAVES + wave; // 1 KB pieces, 8 per 16-row tile
-				const int t = min(mt_base + (piece >> 3), m_tiles - 1);
-				stage_off[i] = static_cast<uint32_t>(t * chunks) * kChunkTileBytes + (piece & 7) * kFragBytes;
-			}
-			// Issued outside the compiler's view: it would otherwise treat the pending direct-to-LDS
-			// loads as possibly out-of-order returns and turn every later LDS wait of the chunk into a
-			// wait for everything.  The explicit vmcnt(0) before the chunk's barrier covers them.
+			const uint32_t lds_base =
+			    static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const uint8_t*)(lds)));
+			const uint32_t slot_lds = lds_base + 3 * kHalfBytes + wave * kSlotBytes;
 			const uint32_t lane_off = lane * 16;
-			const uint32_t tile_lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
-			    (__attribute__((address_space(3))) const uint8_t*)(tile)));
-			const auto stage_issue = [&](int c, int buf) {
+
+			// ---- activation requests: piece i * WAVES + wave of the half (tile t = piece / 4, step
+			// piece % 4); tiles past the end re-read the last one.  Offsets are wavefront-uniform.
+			uint32_t x_off[kXLoads];
 #pragma unroll
-				for (int i = 0; i < kStageLoads; ++i)
+			for (int i = 0; i < kXLoads; ++i)
+			{
+				const int piece = i * WAVES + wave;
+				const int t = min(mt_base + (piece >> 2), m_tiles - 1);
+				x_off[i] = static_cast<uint32_t>(t * chunks) * kChunkTileBytes + (piece & 3) * kFragBytes;
+			}
+			const auto issue_x = [&](int half, int buf_off) {
+#pragma unroll
+				for (int i = 0; i < kXLoads; ++i)
 				{
 					const int piece = i * WAVES + wave;
-					const uint8_t* src = xf + (stage_off[i] + static_cast<uint32_t>(c) * kChunkTileBytes);
-					const uint32_t dst = tile_lds + buf * kTileBytes + piece * kFragBytes;
+					const uint8_t* src = xf + (x_off[i] + static_cast<uint32_t>(half) * (4 * kFragBytes));
+					const uint32_t dst = lds_base + buf_off + piece * kFragBytes;
 					asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
 					             :
 					             : "s"(dst), "v"(lane_off), "s"(src)
 					             : "memory", "m0");
 				}
 			};
+
+			// ---- weight requests: piece p = 64 i + lane of the slot is piece p % P of row p / P; a
+			// row's pieces start at the 16-byte boundary at or below its chunk.  Rows past the end
+			// re-read the last row; their results are never stored.
+			const uint8_t* w_src[kWLoads]; // the row's chunk 0
+			int w_piece[kWLoads];          // 16 j
+#pragma unroll
+			for (int i = 0; i < kWLoads; ++i)
+			{
+				const int piece = min(64 * i + lane, NG * 16 * P - 1);
+				const int row = piece / P;
+				w_piece[i] = 16 * (piece - row * P);
+				w_src[i] = w + static_cast<size_t>(min(n_base + row, n - 1)) * row_bytes;
+			}
+			const auto issue_w = [&](int c) {
+#pragma unroll
+				for (int i = 0; i < kWLoads; ++i)
+				{
+					if (64 * (i + 1) <= NG * 16 * P || 64 * i + lane < NG * 16 * P)
+					{
+						const uintptr_t chunk = reinterpret_cast<uintptr_t>(w_src[i] + static_cast<size_t>(c) * F::kChunkBytes);
+						const uint8_t* src =
+						    reinterpret_cast<const uint8_t*>((F::kAligned16 ? chunk : (chunk & ~uintptr_t{ 15 })) + w_piece[i]);
+						const uint32_t dst = slot_lds + i * 1024;
+						asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+						             :
+						             : "s"(dst), "v"(src)
+						             : "memory", "m0");
+					}
+				}
+			};
+			// this lane's row of group q inside the slot
+			lds_bytes_t slot_rows[NG];
+#pragma unroll
+			for (int q = 0; q < NG; ++q)
+			{
+				slot_rows[q] = (lds_bytes_t)(lds) + 3 * kHalfBytes + wave * kSlotBytes + (16 * q + r) * kRowStride;
+			}
+			const uint8_t* lane_rows[NG]; // for the misalignment of a chunk start
+#pragma unroll
+			for (int q = 0; q < NG; ++q)
+			{
+				lane_rows[q] = w + static_cast<size_t>(min(n_base + 16 * q + r, n - 1)) * row_bytes;
+			}
 
 			floatx4 acc[NG][MT];
 #pragma unroll
@@ -494,12 +595,13 @@ namespace litenn_hip
 
 			half8 a_cur[NG], a_nxt[NG];
 			u32x4 b[MT]; // fragment t of the current step until its MFMAs are issued, then of the next
-			const uint8_t* lane_tile = tile + lane * 16;
-			const auto read_b = [&](int t, int buf, int s) {
-				b[t] = *reinterpret_cast<const u32x4*>(lane_tile + buf * kTileBytes + t * kChunkTileBytes + s * kFragBytes);
+			typename F::Raw raw[NG];
+			typename F::Scale sc[NG];
+			const auto lane_x = (lds_bytes_t)(lds) + lane * 16;
+			const auto read_b = [&](int t, int buf_off, int s4) {
+				b[t] = *(lds_u32x4_t)(lane_x + buf_off + t * (4 * kFragBytes) + s4 * kFragBytes);
 			};
-			const auto decode = [&](half8 (&a)[NG], const typename F::Raw (&raw)[NG], const typename F::Scale (&sc)[NG],
-			                        int s) {
+			const auto decode = [&](half8 (&a)[NG], int s) {
 #pragma unroll
 				for (int q = 0; q < NG; ++q)
 				{
@@ -509,9 +611,21 @@ namespace litenn_hip
 					a[q] = __builtin_bit_cast(half8, v);
 				}
 			};
-			// the MFMAs of the current step; fragment t is refilled for step (buf, s) right after its
-			// last use (refill = false on the very last step)
-			const auto mfma_step = [&](bool refill, int buf, int s) {
+			const auto load_raw = [&](int c) {
+#pragma unroll
+				for (int q = 0; q < NG; ++q)
+				{
+					const int mis =
+					    F::kAligned16
+					        ? 0
+					        : static_cast<int>(reinterpret_cast<uintptr_t>(lane_rows[q] + static_cast<size_t>(c) * F::kChunkBytes) & 15);
+					raw[q] = F::load(slot_rows[q] + mis, g);
+					sc[q] = F::prep(raw[q], g);
+				}
+			};
+			// the MFMAs of the current step; fragment t is refilled from (buf_off, s4) right after its
+			// last use
+			const auto mfma_step = [&](bool refill, int buf_off, int s4) {
 #pragma unroll
 				for (int t = 0; t < MT; ++t)
 				{
@@ -524,7 +638,7 @@ namespace litenn_hip
 					}
 					if (refill)
 					{
-						read_b(t, buf, s);
+						read_b(t, buf_off, s4);
 					}
 				}
 			};
@@ -536,120 +650,108 @@ namespace litenn_hip
 				}
 			};
 			// spread the LDS reads and the decode arithmetic of a step between its MFMAs
-			const auto interleave = [&]() {
-				constexpr int kMfma = NG * MT;
-				constexpr int kValuPerTile = (F::kFragValu * NG + MT - 1) / MT;
+			const auto interleave = [&](auto extra_valu_tag) {
+				constexpr int valu_per_tile = (F::kFragValu * NG + decltype(extra_valu_tag)::value + MT - 1) / MT;
 #pragma unroll
 				for (int t = 0; t < MT; ++t)
 				{
-					__builtin_amdgcn_sched_group_barrier(0x008, NG, 0);           // the MFMAs of one activation fragment
-					__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);            // its refill from LDS
-					__builtin_amdgcn_sched_group_barrier(0x002, kValuPerTile, 0); // a share of the decode arithmetic
-				}
-				(void)kMfma;
-			};
-			const auto load_raw = [&](typename F::Raw (&raw)[NG], int c) {
-#pragma unroll
-				for (int q = 0; q < NG; ++q)
-				{
-					raw[q] = F::load(rows[q] + static_cast<size_t>(c) * F::kChunkBytes, g);
+					__builtin_amdgcn_sched_group_barrier(0x008, NG, 0);            // the MFMAs of one activation fragment
+					__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // its refill from LDS
+					__builtin_amdgcn_sched_group_barrier(0x002, valu_per_tile, 0); // a share of the decode arithmetic
 				}
 			};
-			const auto prep_all = [&](typename F::Scale (&sc)[NG], const typename F::Raw (&raw)[NG]) {
-#pragma unroll
-				for (int q = 0; q < NG; ++q)
-				{
-					sc[q] = F::prep(raw[q], g);
-				}
-			};
-			constexpr int kWaitAllLoads = 0x0F70; // s_waitcnt vmcnt(0), the other counters at their maxima
-
-			// one chunk out of `cur`, fetching the next into `nxt`
-			const auto chunk = [&](auto has_next_tag, const typename F::Raw (&raw_cur)[NG],
-			                       const typename F::Scale (&sc_cur)[NG], typename F::Raw (&raw_nxt)[NG],
-			                       typename F::Scale (&sc_nxt)[NG], int c, int buf) {
-				constexpr bool has_next = decltype(has_next_tag)::value;
-				if (has_next)
-				{
-#if !(LITENN_GEMM_KNOCKOUT & 1)
-					stage_issue(c + 1, buf ^ 1);
-#endif
-#if !(LITENN_GEMM_KNOCKOUT & 2)
-					load_raw(raw_nxt, c + 1);
-#endif
-				}
-#pragma unroll
-				for (int s = 0; s < 7; ++s)
-				{
-#if !(LITENN_GEMM_KNOCKOUT & 8)
-					decode(a_nxt, raw_cur, sc_cur, s + 1);
-#endif
-					mfma_step(!(LITENN_GEMM_KNOCKOUT & 16), buf, s + 1);
-					interleave();
-					__builtin_amdgcn_sched_barrier(0);
-					rotate();
-				}
-				// Everything this wavefront requested at the top of the chunk has landed, every
-				// wavefront's LDS reads of this chunk have returned: after the barrier the next tile is
-				// complete and this one may be overwritten.
-				__builtin_amdgcn_s_waitcnt(kWaitAllLoads);
-#if !(LITENN_GEMM_KNOCKOUT & 4)
-				__syncthreads();
-#endif
-				if (has_next)
-				{
-#if !(LITENN_GEMM_KNOCKOUT & 2)
-					prep_all(sc_nxt, raw_nxt);
-#endif
-#if !(LITENN_GEMM_KNOCKOUT & 8)
-					decode(a_nxt, raw_nxt, sc_nxt, 0);
-#endif
-				}
-				mfma_step(has_next && !(LITENN_GEMM_KNOCKOUT & 16), buf ^ 1, 0);
-				if (has_next)
-				{
-					interleave();
-				}
+			const auto plain_step = [&](int buf_off, int s) { // steps 0..2 and 4..6: refill from the same half
+				decode(a_nxt, s + 1);
+				mfma_step(true, buf_off, (s + 1) & 3);
+				interleave(std::integral_constant<int, 0>{});
 				__builtin_amdgcn_sched_barrier(0);
 				rotate();
 			};
 
-			typename F::Raw raw_a[NG], raw_b[NG];
-			typename F::Scale sc_a[NG], sc_b[NG];
-			stage_issue(0, 0);
-			load_raw(raw_a, 0);
-			__builtin_amdgcn_s_waitcnt(kWaitAllLoads);
+			// Half h of the K walk lives in buffer h % 3.  `cur`, `nxt`, `far` are the byte offsets of
+			// the buffers of the current half, the next and the one after; they rotate per half.
+			int cur = 0, nxt = kHalfBytes, far = 2 * kHalfBytes;
+			const auto rotate_buffers = [&]() {
+				const int t = cur;
+				cur = nxt;
+				nxt = far;
+				far = t;
+			};
+			const auto chunk = [&](auto has_next_tag, int c) {
+				constexpr bool has_next = decltype(has_next_tag)::value;
+				// first half: steps 0..3 out of `cur`
+				if (has_next)
+				{
+					issue_x(2 * c + 2, far);
+					issue_w(c + 1);
+				}
+				plain_step(cur, 0);
+				plain_step(cur, 1);
+				plain_step(cur, 2);
+				// the second half of this chunk (requested one half ago) must be complete, in every
+				// wavefront's share; what was requested at the top of this half may stay in flight
+				if (has_next)
+				{
+					vm_wait<kXLoads + kWLoads>();
+				}
+				else
+				{
+					vm_wait<0>();
+				}
+				__syncthreads();
+				decode(a_nxt, 4);
+				mfma_step(true, nxt, 0);
+				interleave(std::integral_constant<int, 0>{});
+				__builtin_amdgcn_sched_barrier(0);
+				rotate();
+				rotate_buffers();
+				// second half: steps 4..7; the barrier above freed the buffer of the previous half
+				if (has_next)
+				{
+					issue_x(2 * c + 3, far);
+				}
+				plain_step(cur, 4);
+				plain_step(cur, 5);
+				plain_step(cur, 6);
+				if (has_next)
+				{
+					// next chunk: its first half and its weights have landed
+					vm_wait<kXLoads>();
+					__syncthreads();
+					load_raw(c + 1);
+					decode(a_nxt, 0);
+					mfma_step(true, nxt, 0);
+					interleave(std::integral_constant<int, 16 * NG>{});
+					__builtin_amdgcn_sched_barrier(0);
+					rotate();
+					rotate_buffers();
+				}
+				else
+				{
+					mfma_step(false, 0, 0);
+				}
+			};
+
+			issue_w(0);
+			issue_x(0, 0);
+			issue_x(1, kHalfBytes);
+			vm_wait<0>();
 			__syncthreads();
-			prep_all(sc_a, raw_a);
+			load_raw(0);
 #pragma unroll
 			for (int t = 0; t < MT; ++t)
 			{
 				read_b(t, 0, 0);
 			}
-			decode(a_cur, raw_a, sc_a, 0);
-#if LITENN_GEMM_KNOCKOUT
-			load_raw(raw_b, 0);
-			prep_all(sc_b, raw_b);
-			decode(a_nxt, raw_a, sc_a, 1);
-#endif
-			// chunks come in pairs (one per register set and LDS half); the last one fetches nothing
+			decode(a_cur, 0);
 			using std::false_type;
 			using std::true_type;
 			int c = 0;
-			for (; c + 2 < chunks; c += 2)
+			for (; c + 1 < chunks; ++c)
 			{
-				chunk(true_type{}, raw_a, sc_a, raw_b, sc_b, c, 0);
-				chunk(true_type{}, raw_b, sc_b, raw_a, sc_a, c + 1, 1);
+				chunk(true_type{}, c);
 			}
-			if (c + 2 == chunks)
-			{
-				chunk(true_type{}, raw_a, sc_a, raw_b, sc_b, c, 0);
-				chunk(false_type{}, raw_b, sc_b, raw_a, sc_a, c + 1, 1);
-			}
-			else
-			{
-				chunk(false_type{}, raw_a, sc_a, raw_b, sc_b, c, 0);
-			}
+			chunk(false_type{}, c);
 
 			// D layout: lane holds activation row j = lane % 16 and weight rows 4 (lane / 16) + 0..3
 			const bool vec_ok = (n & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 &&
@@ -698,7 +800,8 @@ namespace litenn_hip
 		void launch_variant(const uint8_t* w, const uint8_t* xf, const float* unscale, float* y, const float* residual,
 		                    int n, int k, int m, int m_tiles, size_t row_bytes, hipStream_t stream)
 		{
-			constexpr size_t lds = 2 * MT * kChunkTileBytes;
+			constexpr size_t lds = gemm_lds_bytes<F, MT, NG, WAVES>();
+			static_assert(lds <= kLdsLimit, "LDS budget");
 			static const hipError_t attr =
 			    hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_q_kernel<F, MT, NG, WAVES>),
 			                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
@@ -723,10 +826,13 @@ namespace litenn_hip
 			static const int forced = env_int("LITENN_HIP_GEMM_TILE", 0); // MT * 100 + NG * 10 + WAVES
 #define LITENN_GEMM_ARGS w, xf, unscale, y, residual, n, k, m, m_tiles, row_bytes, stream
 #define LITENN_GEMM_CASE(MT_, NG_, WV_)                                                                              \
-	if (pick == MT_ * 100 + NG_ * 10 + WV_)                                                                        \
+	if constexpr (gemm_lds_bytes<F, MT_, NG_, WV_>() <= kLdsLimit && (NG_ == 1 || F::kWideTile))                                              \
 	{                                                                                                              \
-		launch_variant<F, MT_, NG_, WV_>(LITENN_GEMM_ARGS);                                                        \
-		return;                                                                                                    \
+		if (pick == MT_ * 100 + NG_ * 10 + WV_)                                                                    \
+		{                                                                                                          \
+			launch_variant<F, MT_, NG_, WV_>(LITENN_GEMM_ARGS);                                                    \
+			return;                                                                                                \
+		}                                                                                                          \
 	}
 			int pick = forced;
 			if (pick == 0)
@@ -738,15 +844,15 @@ namespace litenn_hip
 				{
 					pick = 828;
 				}
-				else if (m_tiles >= 8 && blocks(8, 128) >= cus)
+				else if (m_tiles >= 8 && 5 * blocks(8, 128) >= 4 * cus)
 				{
 					pick = 818;
 				}
-				else if (m_tiles >= 4 && blocks(4, 64) >= cus)
+				else if (m_tiles >= 4 && 5 * blocks(4, 64) >= 4 * cus)
 				{
 					pick = 414;
 				}
-				else if (m_tiles >= 2 && blocks(2, 64) >= cus)
+				else if (m_tiles >= 2 && 5 * blocks(2, 64) >= 4 * cus)
 				{
 					pick = 214;
 				}
