@@ -1243,6 +1243,9 @@ namespace litenn_hip
 				return;
 			}
 			const uint8_t* rp = table + static_cast<size_t>(id) * row_bytes;
+			// several elements per thread in flight: the per-element decode is a chain of dependent
+			// byte loads, and a single-token step waits for this kernel
+#pragma unroll 4
 			for (int i = threadIdx.x; i < k; i += blockDim.x)
 			{
 				out[static_cast<size_t>(blockIdx.x) * k + i] = generic_elem(fmt, rp, i);
@@ -1526,7 +1529,7 @@ namespace litenn_hip
 	void launch_get_rows_q(int fmt, const void* table, size_t rows, size_t k, const int32_t* ids, size_t n_ids,
 	                       float* out, int* err_flag, hipStream_t stream)
 	{
-		get_rows_q_kernel<<<dim3(n_ids), dim3(256), 0, stream>>>(fmt, static_cast<const uint8_t*>(table),
+		get_rows_q_kernel<<<dim3(n_ids), dim3(k >= 4096 ? 1024 : 256), 0, stream>>>(fmt, static_cast<const uint8_t*>(table),
 		                                                          static_cast<int>(rows), static_cast<int>(k),
 		                                                          row_bytes(fmt, k), ids, out, err_flag);
 	}
