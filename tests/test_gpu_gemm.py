@@ -73,6 +73,18 @@ def test_config3_q6_k_4096x4096(hip, oracle, m):
     assert run_case(hip, oracle, Q6_K, m, 4096, 4096, seed=40 + m, rows=rows) <= TOL
 
 
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("m,n,k", [(144, 26400, 512),    # 128-row tiles, one row group per wavefront
+                                   (130, 52500, 256),    # 128-row tiles, two row groups (nibble formats)
+                                   (50, 13200, 768)])    # 64-row tiles
+def test_gemm_every_tile_shape(hip, oracle, fmt, m, n, k):
+    """Shapes chosen so that the launcher's tile choice reaches each of its variants for every
+    format (ragged in M and N, odd chunk counts); a 512-row sample of N is checked."""
+    rows = np.sort(np.random.default_rng(n).choice(n, 512, replace=False))
+    rows[0], rows[-1] = 0, n - 1
+    assert run_case(hip, oracle, fmt, m, n, k, seed=n % 97, rows=rows, residual=(k == 512)) <= TOL
+
+
 def test_gemm_is_linear_in_x_at_full_size(hip):
     """Size-independent property at the full north-star shape: Y(a x1 + x2) = a Y(x1) + Y(x2) up to
     the fp16 rounding of the activations."""
