@@ -350,11 +350,20 @@ namespace litenn_hip
 		constexpr int kFragBytes = 1024;                // 64 lanes x 8 halves
 		constexpr int kChunkTileBytes = 8 * kFragBytes; // one 16-row tile of one chunk
 
+		// Optional producers folded into the pre-pass (they would otherwise be a launch and a pass over
+		// the activations each): RMSNorm with f64 accumulation and the f32 result the stand-alone kernel
+		// gives (ComputePrimitives.h:792-817), or SwiGLU's silu(gate) * up with its separately rounded
+		// steps (Activation.h:22-35,56-63; SwiGLU.h:63-66).  The row stays in registers throughout.
+		constexpr int kHeldItems = 8; // 8-element items per thread held in registers: rows up to 16384 wide
+
 		template <typename F>
 		__global__ __launch_bounds__(256) void to_half_kernel(const float* __restrict__ x, uint8_t* __restrict__ xf,
-		                                                       float* __restrict__ unscale, int m, int k)
+		                                                       float* __restrict__ unscale, int m, int k,
+		                                                       const float* __restrict__ norm_w, double eps,
+		                                                       const float* __restrict__ up)
 		{
 			__shared__ float red[4];
+			__shared__ double red64[4];
 			const int row = blockIdx.x;
 			const int chunks = k / kChunk;
 			const int mt = row >> 4, r = row & 15;
@@ -374,36 +383,96 @@ namespace litenn_hip
 				return;
 			}
 			const float* src = x + static_cast<size_t>(row) * k;
-			// The thread's share of the row stays in registers between the maximum and the conversion
-			// (up to kHeld items of 8 elements; longer rows re-read the rest).
-			constexpr int kHeld = 8;
-			float4 held[kHeld][2];
-			float mx = 0.0f;
+			float held[kHeldItems][8];
+			// element offsets of item `it`: 0..3 at k0, 4..7 at k1
+			const auto offsets = [&](int it, int& o0, int& o1) {
+				const int c = it >> 5, st = (it >> 2) & 7, g = it & 3;
+				int k0, k1;
+				F::koff(g, st, k0, k1);
+				o0 = c * kChunk + k0;
+				o1 = c * kChunk + k1;
+			};
+			double ss = 0.0;
 #pragma unroll
-			for (int u = 0; u < kHeld; ++u)
+			for (int u = 0; u < kHeldItems; ++u)
 			{
 				const int it = threadIdx.x + 256 * u;
 				if (it < items)
 				{
-					const int c = it >> 5, st = (it >> 2) & 7, g = it & 3;
-					int k0, k1;
-					F::koff(g, st, k0, k1);
-					held[u][0] = *reinterpret_cast<const float4*>(src + c * kChunk + k0);
-					held[u][1] = *reinterpret_cast<const float4*>(src + c * kChunk + k1);
-					const float4 a = held[u][0], b = held[u][1];
-					mx = fmaxf(mx, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
-					mx = fmaxf(mx, fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w))));
+					int o0, o1;
+					offsets(it, o0, o1);
+					const float4 a = *reinterpret_cast<const float4*>(src + o0);
+					const float4 b = *reinterpret_cast<const float4*>(src + o1);
+					held[u][0] = a.x, held[u][1] = a.y, held[u][2] = a.z, held[u][3] = a.w;
+					held[u][4] = b.x, held[u][5] = b.y, held[u][6] = b.z, held[u][7] = b.w;
+					if (up)
+					{
+						const float4 ua = *reinterpret_cast<const float4*>(up + static_cast<size_t>(row) * k + o0);
+						const float4 ub = *reinterpret_cast<const float4*>(up + static_cast<size_t>(row) * k + o1);
+						const float uu[8] = { ua.x, ua.y, ua.z, ua.w, ub.x, ub.y, ub.z, ub.w };
+#pragma unroll
+						for (int e = 0; e < 8; ++e)
+						{
+							const float gv = held[u][e];
+							const float sig = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf(-gv)));
+							held[u][e] = __fmul_rn(__fmul_rn(gv, sig), uu[e]);
+						}
+					}
+					if (norm_w)
+					{
+#pragma unroll
+						for (int e = 0; e < 8; ++e)
+						{
+							const double v = static_cast<double>(held[u][e]);
+							ss += v * v;
+						}
+					}
 				}
 			}
-			for (int it = threadIdx.x + 256 * kHeld; it < items; it += 256)
+			if (norm_w)
 			{
-				const int c = it >> 5, st = (it >> 2) & 7, g = it & 3;
-				int k0, k1;
-				F::koff(g, st, k0, k1);
-				const float4 a = *reinterpret_cast<const float4*>(src + c * kChunk + k0);
-				const float4 b = *reinterpret_cast<const float4*>(src + c * kChunk + k1);
-				mx = fmaxf(mx, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
-				mx = fmaxf(mx, fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w))));
+				for (int off = 32; off > 0; off >>= 1)
+				{
+					ss += __shfl_xor(ss, off, 64);
+				}
+				if ((threadIdx.x & 63) == 0)
+				{
+					red64[threadIdx.x >> 6] = ss;
+				}
+				__syncthreads();
+				const double total = red64[0] + red64[1] + red64[2] + red64[3];
+				const double inv = 1.0 / sqrt(total / static_cast<double>(k) + eps);
+#pragma unroll
+				for (int u = 0; u < kHeldItems; ++u)
+				{
+					const int it = threadIdx.x + 256 * u;
+					if (it < items)
+					{
+						int o0, o1;
+						offsets(it, o0, o1);
+						const float4 wa = *reinterpret_cast<const float4*>(norm_w + o0);
+						const float4 wb = *reinterpret_cast<const float4*>(norm_w + o1);
+						const float ww[8] = { wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w };
+#pragma unroll
+						for (int e = 0; e < 8; ++e)
+						{
+							held[u][e] = static_cast<float>(static_cast<double>(held[u][e]) * inv * static_cast<double>(ww[e]));
+						}
+					}
+				}
+			}
+			float mx = 0.0f;
+#pragma unroll
+			for (int u = 0; u < kHeldItems; ++u)
+			{
+				if (threadIdx.x + 256 * u < items)
+				{
+#pragma unroll
+					for (int e = 0; e < 8; ++e)
+					{
+						mx = fmaxf(mx, fabsf(held[u][e]));
+					}
+				}
 			}
 			mx = wave_max(mx);
 			if ((threadIdx.x & 63) == 0)
@@ -417,31 +486,20 @@ namespace litenn_hip
 			{
 				shift = 14 - ilogbf(mx);
 			}
-			const auto emit = [&](int it, const float4& v0, const float4& v1) {
-				const int c = it >> 5, st = (it >> 2) & 7, g = it & 3;
-				u32x4 out;
-				out.x = pack_f16(ldexpf(v0.x, shift), ldexpf(v0.y, shift));
-				out.y = pack_f16(ldexpf(v0.z, shift), ldexpf(v0.w, shift));
-				out.z = pack_f16(ldexpf(v1.x, shift), ldexpf(v1.y, shift));
-				out.w = pack_f16(ldexpf(v1.z, shift), ldexpf(v1.w, shift));
-				*reinterpret_cast<u32x4*>(tile_row + (c * 8 + st) * kFragBytes + g * 256) = out;
-			};
 #pragma unroll
-			for (int u = 0; u < kHeld; ++u)
+			for (int u = 0; u < kHeldItems; ++u)
 			{
 				const int it = threadIdx.x + 256 * u;
 				if (it < items)
 				{
-					emit(it, held[u][0], held[u][1]);
+					const int c = it >> 5, st = (it >> 2) & 7, g = it & 3;
+					u32x4 out;
+					out.x = pack_f16(ldexpf(held[u][0], shift), ldexpf(held[u][1], shift));
+					out.y = pack_f16(ldexpf(held[u][2], shift), ldexpf(held[u][3], shift));
+					out.z = pack_f16(ldexpf(held[u][4], shift), ldexpf(held[u][5], shift));
+					out.w = pack_f16(ldexpf(held[u][6], shift), ldexpf(held[u][7], shift));
+					*reinterpret_cast<u32x4*>(tile_row + (c * 8 + st) * kFragBytes + g * 256) = out;
 				}
-			}
-			for (int it = threadIdx.x + 256 * kHeld; it < items; it += 256)
-			{
-				const int c = it >> 5, st = (it >> 2) & 7, g = it & 3;
-				int k0, k1;
-				F::koff(g, st, k0, k1);
-				emit(it, *reinterpret_cast<const float4*>(src + c * kChunk + k0),
-				     *reinterpret_cast<const float4*>(src + c * kChunk + k1));
 			}
 			if (threadIdx.x == 0)
 			{
@@ -467,6 +525,11 @@ namespace litenn_hip
 		// and the weight fragments of step s + 1 are decoded, the three instruction streams
 		// interleaved by scheduling directives.  One barrier per half chunk: it publishes the next
 		// half's activations and frees the buffer of the previous one.
+		// The direct-to-LDS loads below set M0 themselves and say so in their clobber lists; clang
+		// warns that it does not save a reserved register around such a statement.  Nothing else in
+		// this kernel lives in M0 (no other LDS-DMA, no register-indexed arrays).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 		template <int N>
 		__device__ __forceinline__ void vm_wait()
 		{
@@ -487,14 +550,28 @@ namespace litenn_hip
 			return 3 * MT * 4 * kFragBytes + static_cast<size_t>(WAVES) * NG * 16 * 16 * weight_pieces<F>();
 		}
 
-		template <typename F, int MT, int NG, int WAVES>
-		__global__ __launch_bounds__(64 * WAVES) void gemm_q_kernel(const uint8_t* __restrict__ w,
-		                                                             const uint8_t* __restrict__ xf,
-		                                                             const float* __restrict__ unscale,
-		                                                             float* __restrict__ y,
-		                                                             const float* __restrict__ residual, int n, int k,
-		                                                             int m, int m_tiles, size_t row_bytes)
+		// Up to three matrices of one format and width that share the activations (q/k/v, gate/up):
+		// their row blocks are laid side by side along grid x.
+		struct GemmMats
 		{
+			const uint8_t* w[3];
+			float* y[3];
+			int n[3];
+			int first_block[3]; // grid x index of each matrix's first row block (INT_MAX when unused)
+		};
+
+		template <typename F, int MT, int NG, int WAVES>
+		__global__ __launch_bounds__(64 * WAVES) void gemm_q_kernel(const GemmMats mats, const uint8_t* __restrict__ xf,
+		                                                             const float* __restrict__ unscale,
+		                                                             const float* __restrict__ residual, int k, int m,
+		                                                             int m_tiles, size_t row_bytes)
+		{
+			const int which = (static_cast<int>(blockIdx.x) >= mats.first_block[1]) +
+			                  (static_cast<int>(blockIdx.x) >= mats.first_block[2]);
+			const uint8_t* __restrict__ w = which == 0 ? mats.w[0] : (which == 1 ? mats.w[1] : mats.w[2]);
+			float* __restrict__ y = which == 0 ? mats.y[0] : (which == 1 ? mats.y[1] : mats.y[2]);
+			const int n = which == 0 ? mats.n[0] : (which == 1 ? mats.n[1] : mats.n[2]);
+			const int block_x = blockIdx.x - (which == 0 ? 0 : (which == 1 ? mats.first_block[1] : mats.first_block[2]));
 			constexpr int kHalfBytes = MT * 4 * kFragBytes; // one activation buffer: four steps of MT tiles
 			constexpr int kXLoads = MT * 4 / WAVES;         // 1 KB pieces a wavefront moves per half
 			static_assert(kXLoads >= 1 && kXLoads * WAVES == MT * 4, "activation pieces / wavefront split");
@@ -506,7 +583,7 @@ namespace litenn_hip
 			const int lane = threadIdx.x & 63;
 			const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 			const int r = lane & 15, g = lane >> 4;
-			const int n_base = (blockIdx.x * WAVES + wave) * 16 * NG;
+			const int n_base = (block_x * WAVES + wave) * 16 * NG;
 			const int mt_base = blockIdx.y * MT;
 			const int chunks = k / kChunk;
 			const uint32_t lds_base =
@@ -796,9 +873,24 @@ namespace litenn_hip
 			}
 		}
 
+#pragma clang diagnostic pop
+
+		struct GemmCall
+		{
+			int count;
+			const uint8_t* w[3];
+			float* y[3];
+			int n[3];
+			const uint8_t* xf;
+			const float* unscale;
+			const float* residual;
+			int k, m, m_tiles;
+			size_t row_bytes;
+			hipStream_t stream;
+		};
+
 		template <typename F, int MT, int NG, int WAVES>
-		void launch_variant(const uint8_t* w, const uint8_t* xf, const float* unscale, float* y, const float* residual,
-		                    int n, int k, int m, int m_tiles, size_t row_bytes, hipStream_t stream)
+		void launch_variant(const GemmCall& c)
 		{
 			constexpr size_t lds = gemm_lds_bytes<F, MT, NG, WAVES>();
 			static_assert(lds <= kLdsLimit, "LDS budget");
@@ -807,30 +899,42 @@ namespace litenn_hip
 			                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
 			(void)attr;
 			constexpr int bn = 16 * WAVES * NG;
-			const dim3 grid((n + bn - 1) / bn, (m_tiles + MT - 1) / MT);
-			gemm_q_kernel<F, MT, NG, WAVES><<<grid, dim3(64 * WAVES), lds, stream>>>(w, xf, unscale, y, residual, n, k, m,
-			                                                                        m_tiles, row_bytes);
+			GemmMats mats;
+			int blocks = 0;
+			for (int i = 0; i < 3; ++i)
+			{
+				mats.w[i] = i < c.count ? c.w[i] : nullptr;
+				mats.y[i] = i < c.count ? c.y[i] : nullptr;
+				mats.n[i] = i < c.count ? c.n[i] : 0;
+				mats.first_block[i] = i < c.count ? blocks : 0x7fffffff;
+				blocks += i < c.count ? (c.n[i] + bn - 1) / bn : 0;
+			}
+			const dim3 grid(blocks, (c.m_tiles + MT - 1) / MT);
+			gemm_q_kernel<F, MT, NG, WAVES><<<grid, dim3(64 * WAVES), lds, c.stream>>>(mats, c.xf, c.unscale, c.residual,
+			                                                                          c.k, c.m, c.m_tiles, c.row_bytes);
 		}
 
 		// Tile choice: MT activation tiles per workgroup so that a weight is decoded as few times as
-		// possible (MT = 8 takes 128 KB of LDS, so eight wavefronts share it); two weight groups per
-		// wavefront (each activation fragment read from LDS feeds two MFMAs) when that still leaves
-		// every CU a workgroup.
+		// possible; two weight groups per wavefront (each activation fragment read from LDS feeds two
+		// MFMAs) when that still nearly fills the card.
 		template <typename F>
-		void launch_format(const uint8_t* w, const uint8_t* xf, const float* unscale, float* y, const float* residual,
-		                   int n, int k, int m, int m_tiles, size_t row_bytes, int cus, hipStream_t stream)
+		void launch_format(const GemmCall& c, int cus)
 		{
 			const auto blocks = [&](int mt, int bn) {
-				return static_cast<long>((n + bn - 1) / bn) * ((m_tiles + mt - 1) / mt);
+				long nb = 0;
+				for (int i = 0; i < c.count; ++i)
+				{
+					nb += (c.n[i] + bn - 1) / bn;
+				}
+				return nb * ((c.m_tiles + mt - 1) / mt);
 			};
 			static const int forced = env_int("LITENN_HIP_GEMM_TILE", 0); // MT * 100 + NG * 10 + WAVES
-#define LITENN_GEMM_ARGS w, xf, unscale, y, residual, n, k, m, m_tiles, row_bytes, stream
 #define LITENN_GEMM_CASE(MT_, NG_, WV_)                                                                              \
-	if constexpr (gemm_lds_bytes<F, MT_, NG_, WV_>() <= kLdsLimit && (NG_ == 1 || F::kWideTile))                                              \
+	if constexpr (gemm_lds_bytes<F, MT_, NG_, WV_>() <= kLdsLimit && (NG_ == 1 || F::kWideTile))                   \
 	{                                                                                                              \
 		if (pick == MT_ * 100 + NG_ * 10 + WV_)                                                                    \
 		{                                                                                                          \
-			launch_variant<F, MT_, NG_, WV_>(LITENN_GEMM_ARGS);                                                    \
+			launch_variant<F, MT_, NG_, WV_>(c);                                                                   \
 			return;                                                                                                \
 		}                                                                                                          \
 	}
@@ -839,7 +943,8 @@ namespace litenn_hip
 			{
 				// measured on the MI355X (K = 4096, N = 4096 and 14336, M = 16 .. 512): the widest tile
 				// wins once it nearly fills the card, otherwise the tallest single-group tile that
-				// still gives every CU a workgroup
+				// still gives (nearly) every CU a workgroup
+				const int m_tiles = c.m_tiles;
 				if (m_tiles >= 8 && F::kWideTile && 5 * blocks(8, 256) >= 4 * cus)
 				{
 					pick = 828;
@@ -866,9 +971,17 @@ namespace litenn_hip
 			LITENN_GEMM_CASE(4, 1, 4)
 			LITENN_GEMM_CASE(2, 1, 4)
 			LITENN_GEMM_CASE(1, 1, 4)
-			launch_variant<F, 1, 1, 4>(LITENN_GEMM_ARGS);
+			launch_variant<F, 1, 1, 4>(c);
 #undef LITENN_GEMM_CASE
-#undef LITENN_GEMM_ARGS
+		}
+
+		template <typename F>
+		void launch_prepass_and_gemm(const GemmCall& c, const float* x, const float* norm_w, double eps, const float* up,
+		                             uint8_t* xf, float* unscale, int m_pad, int cus)
+		{
+			to_half_kernel<F><<<dim3(static_cast<unsigned>(m_pad)), dim3(256), 0, c.stream>>>(x, xf, unscale, c.m, c.k,
+			                                                                                 norm_w, eps, up);
+			launch_format<F>(c, cus);
 		}
 	} // namespace
 
@@ -879,22 +992,41 @@ namespace litenn_hip
 		return m_pad * k + 2 * m_pad; // fp16 rows, then one f32 factor per row
 	}
 
-	// Returns false when the shape is not one this kernel takes (the caller then uses the GEMV):
-	// K must be a whole number of 256-element chunks and the rows 16-byte aligned.
-	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
-	                 const float* residual, void* scratch_halves, hipStream_t stream)
+	// One activation matrix against up to three quantised matrices of one format and width:
+	//   y_i[M, n_i] = X'[M, K] . deq(W_i)^T   (+ residual, single matrix only)
+	// where X' = x, or RMSNorm(x) * norm_w when norm_w is given, or silu(x) * up when up is given (the
+	// producers run inside the fp16 pre-pass).  Returns false, launching nothing, when the shape is
+	// not one this kernel takes (the caller then composes the operators and uses the GEMV): K must be
+	// a whole number of 256-element chunks and at most 16384 (a thread of the pre-pass holds its share
+	// of a row in registers), and the rows 16-byte aligned (2-byte for Q6_K).
+	bool launch_gemm_group(int fmt, int count, const void* const* wq, const size_t* n, size_t k, const float* x,
+	                       size_t m, float* const* y, const float* residual, const float* norm_w, double eps,
+	                       const float* up, void* scratch_halves, hipStream_t stream)
 	{
 		const size_t rb = row_bytes(fmt, k);
 		if (fmt != LITENN_FMT_Q4_0 && fmt != LITENN_FMT_Q8_0 && fmt != LITENN_FMT_Q4_K && fmt != LITENN_FMT_Q6_K)
 		{
 			return false;
 		}
-		// Q6_K blocks (210 bytes) are read with 2-byte aligned accesses; the other decoders use
-		// 4- and 16-byte loads, which rows of whole 256-element chunks always allow
+		if (count < 1 || count > 3 || (count > 1 && residual) || (norm_w && up))
+		{
+			return false;
+		}
+		// Q6_K blocks (210 bytes) are fetched from the 16-byte boundary below them; the other formats'
+		// chunks must start on one
 		const uintptr_t w_align = fmt == LITENN_FMT_Q6_K ? 2 : 16;
-		if (k % kChunk != 0 || rb == 0 || reinterpret_cast<uintptr_t>(wq) % w_align != 0 ||
-		    reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(scratch_halves) % 16 != 0 ||
-		    !scratch_halves || 2 * ((m + 15) / 16 * 16) * k >= (size_t{ 1 } << 32)) // 32-bit tile offsets
+		for (int i = 0; i < count; ++i)
+		{
+			if (reinterpret_cast<uintptr_t>(wq[i]) % w_align != 0 || n[i] == 0 || n[i] > 0x7fffffffu)
+			{
+				return false;
+			}
+		}
+		if (k % kChunk != 0 || rb == 0 || (rb % w_align) != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0 ||
+		    reinterpret_cast<uintptr_t>(scratch_halves) % 16 != 0 || !scratch_halves ||
+		    2 * ((m + 15) / 16 * 16) * k >= (size_t{ 1 } << 32) || // 32-bit tile offsets
+		    k > static_cast<size_t>(kHeldItems) * 256 * 8 ||
+		    (norm_w && reinterpret_cast<uintptr_t>(norm_w) % 16 != 0) || (up && reinterpret_cast<uintptr_t>(up) % 16 != 0))
 		{
 			return false;
 		}
@@ -910,29 +1042,38 @@ namespace litenn_hip
 		const size_t m_pad = (m + 15) / 16 * 16;
 		uint8_t* xf = static_cast<uint8_t*>(scratch_halves);
 		float* unscale = reinterpret_cast<float*>(xf + 2 * m_pad * k); // after the fp16 tiles
-		const uint8_t* w = static_cast<const uint8_t*>(wq);
-		const int ni = static_cast<int>(n), ki = static_cast<int>(k), mi = static_cast<int>(m),
-		          mt = static_cast<int>(m_pad / 16);
-		const dim3 rows_grid(static_cast<unsigned>(m_pad));
+		GemmCall c{};
+		c.count = count;
+		for (int i = 0; i < count; ++i)
+		{
+			c.w[i] = static_cast<const uint8_t*>(wq[i]);
+			c.y[i] = y[i];
+			c.n[i] = static_cast<int>(n[i]);
+		}
+		c.xf = xf;
+		c.unscale = unscale;
+		c.residual = residual;
+		c.k = static_cast<int>(k);
+		c.m = static_cast<int>(m);
+		c.m_tiles = static_cast<int>(m_pad / 16);
+		c.row_bytes = rb;
+		c.stream = stream;
+		const int mp = static_cast<int>(m_pad);
 		switch (fmt)
 		{
-		case LITENN_FMT_Q4_0:
-			to_half_kernel<Q4_0Frag><<<rows_grid, dim3(256), 0, stream>>>(x, xf, unscale, mi, ki);
-			launch_format<Q4_0Frag>(w, xf, unscale, y, residual, ni, ki, mi, mt, rb, cus, stream);
-			break;
-		case LITENN_FMT_Q8_0:
-			to_half_kernel<Q8_0Frag><<<rows_grid, dim3(256), 0, stream>>>(x, xf, unscale, mi, ki);
-			launch_format<Q8_0Frag>(w, xf, unscale, y, residual, ni, ki, mi, mt, rb, cus, stream);
-			break;
-		case LITENN_FMT_Q4_K:
-			to_half_kernel<Q4_KFrag><<<rows_grid, dim3(256), 0, stream>>>(x, xf, unscale, mi, ki);
-			launch_format<Q4_KFrag>(w, xf, unscale, y, residual, ni, ki, mi, mt, rb, cus, stream);
-			break;
-		default:
-			to_half_kernel<Q6_KFrag><<<rows_grid, dim3(256), 0, stream>>>(x, xf, unscale, mi, ki);
-			launch_format<Q6_KFrag>(w, xf, unscale, y, residual, ni, ki, mi, mt, rb, cus, stream);
-			break;
+		case LITENN_FMT_Q4_0: launch_prepass_and_gemm<Q4_0Frag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
+		case LITENN_FMT_Q8_0: launch_prepass_and_gemm<Q8_0Frag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
+		case LITENN_FMT_Q4_K: launch_prepass_and_gemm<Q4_KFrag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
+		default: launch_prepass_and_gemm<Q6_KFrag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
 		}
 		return true;
+	}
+
+	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
+	                 const float* residual, void* scratch_halves, hipStream_t stream)
+	{
+		const void* w[1] = { wq };
+		float* ys[1] = { y };
+		return launch_gemm_group(fmt, 1, w, &n, k, x, m, ys, residual, nullptr, 0.0, nullptr, scratch_halves, stream);
 	}
 } // namespace litenn_hip

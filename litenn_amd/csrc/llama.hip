@@ -20,6 +20,9 @@ namespace litenn_hip
 	int launch_gemv(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
 	                const float* residual, hipStream_t stream);
 	size_t gemm_scratch_halves(size_t m, size_t k);
+	bool launch_gemm_group(int fmt, int count, const void* const* wq, const size_t* n, size_t k, const float* x,
+	                       size_t m, float* const* y, const float* residual, const float* norm_w, double eps,
+	                       const float* up, void* scratch_halves, hipStream_t stream);
 	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
 	                 const float* residual, void* scratch_halves, hipStream_t stream);
 	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
@@ -218,6 +221,53 @@ namespace
 		launch_gemv(w.fmt, w.data, w.n, w.k, x, rows, y, residual, s);
 	}
 
+	// Multi-row form of an operator group: y_i = X' . W_i^T (+ residual) with X' = x, RMSNorm(x) * norm_w
+	// or silu(x) * up.  On the matrix cores the producer runs inside the fp16 pre-pass and matrices of
+	// one format share a launch; otherwise it is composed from the stand-alone kernels (`tmp` takes
+	// the producer's result).
+	void matmul_group(litenn_hip_llama* m, int count, const Weight* const* ws, float* const* ys, const float* x,
+	                  size_t rows, const float* residual, const float* norm_w, const float* up, float* tmp,
+	                  unsigned flags, hipStream_t s)
+	{
+		const Weight& w0 = *ws[0];
+		bool same = true;
+		for (int i = 1; i < count; ++i)
+		{
+			same = same && ws[i]->fmt == w0.fmt && ws[i]->k == w0.k;
+		}
+		const bool quant = w0.fmt != LITENN_FMT_F16 && w0.fmt != LITENN_FMT_F32;
+		if (same && rows >= 16 && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && w0.k % 256 == 0)
+		{
+			const void* w[3] = { nullptr, nullptr, nullptr };
+			size_t n[3] = { 0, 0, 0 };
+			for (int i = 0; i < count; ++i)
+			{
+				w[i] = ws[i]->data;
+				n[i] = ws[i]->n;
+			}
+			if (launch_gemm_group(w0.fmt, count, w, n, w0.k, x, rows, ys, residual, norm_w, m->p.rms_norm_epsilon, up,
+			                      m->xh, s))
+			{
+				return;
+			}
+		}
+		const float* in = x;
+		if (norm_w)
+		{
+			launch_rmsnorm(x, norm_w, m->p.rms_norm_epsilon, rows, w0.k, tmp, s);
+			in = tmp;
+		}
+		else if (up)
+		{
+			launch_silu_mul(x, up, tmp, rows * w0.k, s);
+			in = tmp;
+		}
+		for (int i = 0; i < count; ++i)
+		{
+			matmul(m, *ws[i], in, rows, ys[i], residual, flags, s);
+		}
+	}
+
 	// One operator group of the single-token step (see launch_linear_group).
 	void group(litenn_hip_llama* m, int count, const Weight* const* ws, float* const* ys, const float* x,
 	           const float* residual, const float* norm_w, bool silu_mul, hipStream_t s)
@@ -313,25 +363,24 @@ namespace
 		hipStream_t s = m->stream;
 		const size_t d = m->p.embedding_length;
 		const size_t H = m->p.head_count, KH = m->p.head_count_kv, hd = m->head_dim;
-		const size_t ff = m->p.feed_forward_length;
 		const int* past_dev = m->d_counters;
 		launch_get_rows_q(m->tok_embd.fmt, m->tok_embd.data, m->tok_embd.n, d, ids, rows, m->x, m->d_err, s);
 		for (Layer& L : m->layers)
 		{
-			launch_rmsnorm(m->x, L.attn_norm, m->p.rms_norm_epsilon, rows, d, m->xn, s);
-			matmul(m, L.wq, m->xn, rows, m->q, nullptr, flags, s);
-			matmul(m, L.wk, m->xn, rows, m->k, nullptr, flags, s);
-			matmul(m, L.wv, m->xn, rows, m->v, nullptr, flags, s);
+			const Weight* qkv[3] = { &L.wq, &L.wk, &L.wv };
+			float* qkv_out[3] = { m->q, m->k, m->v };
+			matmul_group(m, 3, qkv, qkv_out, m->x, rows, nullptr, L.attn_norm, nullptr, m->xn, flags, s);
 			launch_rope_qkv_append(m->q, m->k, m->v, L.kcache, L.vcache, m->p.kv_dtype, past_dev, rows, H, KH, hd,
 			                       m->p.rope_dimension_count, m->cos_t, m->sin_t, s);
 			launch_attn_decode(m->q, L.kcache, L.vcache, m->p.kv_dtype, rows, past_dev, 0, H, KH, hd, m->attn,
 			                   rows == 1 ? m->attn_splits : 1, m->attn_partial, m->attn_counters, s);
 			matmul(m, L.wo, m->attn, rows, m->x, m->x, flags, s); // x = x + attn . Wo
-			launch_rmsnorm(m->x, L.ffn_norm, m->p.rms_norm_epsilon, rows, d, m->xn, s);
-			matmul(m, L.gate, m->xn, rows, m->gate, nullptr, flags, s);
-			matmul(m, L.up, m->xn, rows, m->up, nullptr, flags, s);
-			launch_silu_mul(m->gate, m->up, m->gate, rows * ff, s);
-			matmul(m, L.down, m->gate, rows, m->x, m->x, flags, s); // x = x + mlp
+			const Weight* gu[2] = { &L.gate, &L.up };
+			float* gu_out[2] = { m->gate, m->up };
+			matmul_group(m, 2, gu, gu_out, m->x, rows, nullptr, L.ffn_norm, nullptr, m->xn, flags, s);
+			const Weight* wd[1] = { &L.down };
+			float* xo[1] = { m->x };
+			matmul_group(m, 1, wd, xo, m->gate, rows, m->x, nullptr, m->up, m->gate2, flags, s); // x = x + mlp
 		}
 		const size_t first = rows - logit_rows;
 		launch_rmsnorm(m->x + first * d, m->output_norm, m->p.rms_norm_epsilon, logit_rows, d, m->xn, s);
