@@ -229,14 +229,22 @@ int litenn_hip_llama_generate(litenn_hip_llama* model, const int32_t* prompt, si
 /* Copies the first `past` cache rows of one layer to host as f32 [past, n_kv_head*head_dim]. */
 int litenn_hip_llama_get_kv(litenn_hip_llama* model, int layer, float* k, float* v);
 
-/* ---- group 4: GGUF container reader (host side) ------------------------ */
+/* ---- group 4: weight container readers (host side) --------------------- */
 
 /* A dependency-free reader of the GGUF container (versions 2 and 3), producing what
  * ImportGGUFArchive produces (tools/gguf/GGUFImporter.cpp:644-678) without ggml: metadata
  * widened to u64 / i64 / f64 / bool / string (:339-437), tensors as (type, shape with the
  * slowest dimension first, :206-221, raw payload, :457-502), LLaMA hyper-parameters with the
  * defaults and checks of ParseLLaMAHyperparameters (:505-642).  The file is mapped read-only;
- * pointers handed out stay valid until litenn_gguf_close.  Error texts are the reference's. */
+ * pointers handed out stay valid until litenn_gguf_close.  Error texts are the reference's.
+ *
+ * litenn_gguf_open also takes a LiteNN model archive (.ltnn, magic "LTNNMDL\0", versions 6..18,
+ * src/LiteNN/Serialization/ModelIO.h:25-26,1291-1341), the reference's own on-disk form of an
+ * imported model: its variable table (names, tensors, quantisation records with block format and
+ * expressed shape, :281-338,592-612) and metadata entries (:27-39,447-505) come before the graph
+ * and are exposed through the same handle and accessors; the graph itself is not read.  For such
+ * a file litenn_gguf_version returns the archive version and a tensor's ggml_type is the id of
+ * its block format's ggml type (negative for plain types ggml has no id for). */
 typedef struct litenn_gguf litenn_gguf;
 
 typedef struct litenn_gguf_tensor {
@@ -271,7 +279,7 @@ int litenn_gguf_metadata_array(const litenn_gguf* file, const char* key, unsigne
 /* Fills every field but kv_dtype; vocab_size comes from token_embd.weight
  * (tools/gguf/LLaMABuilder.cpp:685-703). */
 int litenn_gguf_llama_params(const litenn_gguf* file, litenn_hip_llama_params* out);
-/* Reads the file, uploads the tensors of the decoder (token_embd, output_norm, optional output,
+/* Reads the file (.gguf or .ltnn), uploads the tensors of the decoder (token_embd, output_norm, optional output,
  * and per block attn_norm, attn_q/k/v/output, ffn_norm, ffn_gate/up/down: the names of
  * tools/gguf/LLaMABuilder.cpp:171-178,466-500) and returns a resident model that owns them.
  * context_length > 0 overrides the file's; kv_dtype is F16 or F32. */

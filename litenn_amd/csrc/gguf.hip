@@ -29,6 +29,7 @@ namespace litenn_hip
 	namespace
 	{
 		const char* kReadAction = "GGUF import";
+		const char* kLtnnAction = "LiteNN model import";
 
 		// gguf metadata value types (published container layout)
 		enum GgufType : uint32_t
@@ -57,6 +58,9 @@ namespace litenn_hip
 			{ 24, "i8", 1, 1, -1, LITENN_I8 },      { 26, "i32", 1, 4, -1, LITENN_I32 },
 			{ 27, "i64", 1, 8, -1, LITENN_I64 },    { 28, "f64", 1, 8, -1, LITENN_F64 },
 			{ 30, "bf16", 1, 2, -1, LITENN_BF16 },
+			// plain DataTypes without a ggml id (a LiteNN archive can hold them): -(DataType + 1)
+			{ -(LITENN_BOOL + 1), "bool", 1, 1, -1, LITENN_BOOL },   { -(LITENN_F8E4M3 + 1), "f8e4m3", 1, 1, -1, LITENN_F8E4M3 },
+			{ -(LITENN_F8E5M2 + 1), "f8e5m2", 1, 1, -1, LITENN_F8E5M2 }, { -(LITENN_U8 + 1), "u8", 1, 1, -1, LITENN_U8 },
 		};
 		const TypeInfo* find_type(int ggml_type)
 		{
@@ -235,6 +239,42 @@ namespace
 		return fail(kReadAction, "GGUF metadata key '" + key + "' must be numeric");
 	}
 
+	// Byte size of every tensor from its type and shape, checked against the file
+	int finish_tensors(litenn_gguf* g, const char* what)
+	{
+		const std::string kind = what;
+		for (TensorEntry& t : g->tensors)
+		{
+			uint64_t elements = 1;
+			for (uint64_t n : t.ne)
+			{
+				if (n == 0 || n > (uint64_t{ 1 } << 40))
+				{
+					return fail(kReadAction, kind + " tensor '" + t.name + "' has non-positive dimension " + std::to_string(n));
+				}
+				elements *= n;
+			}
+			const TypeInfo* ti = find_type(t.ggml_type);
+			if (!ti)
+			{
+				return fail(kReadAction, "Unsupported ggml tensor type '" + std::to_string(t.ggml_type) + "' for tensor '" +
+				                             t.name + "'");
+			}
+			const uint64_t row = t.ne.empty() ? 1 : t.ne[0];
+			if (row % static_cast<uint64_t>(ti->block_elements) != 0)
+			{
+				return fail(kReadAction, kind + " tensor '" + t.name + "' has an invalid serialized byte size");
+			}
+			t.bytes = elements / ti->block_elements * ti->block_bytes;
+			if (g->data_offset + t.offset + t.bytes > g->size)
+			{
+				return fail(kReadAction, "Failed to read " + std::to_string(t.bytes) + " bytes for " + kind + " tensor '" +
+				                             t.name + "'");
+			}
+		}
+		return 0;
+	}
+
 	int parse(litenn_gguf* g)
 	{
 		Cursor c{ g };
@@ -331,32 +371,261 @@ namespace
 			}
 		}
 		g->data_offset = (c.pos + alignment - 1) / alignment * alignment;
-		for (TensorEntry& t : g->tensors)
+		return finish_tensors(g, "GGUF");
+	}
+
+	// ---- LiteNN model archive (.ltnn) ---------------------------------------------------------
+	// SaveModel writes, in this order (Serialization/ModelIO.h:1291-1341): magic "LTNNMDL\0", u32
+	// version, u64 forward subgraph, u8 + u64 optional backward subgraph, input and output names,
+	// u64 variable count, variable names, metadata entries, then per variable a tensor (u32 DataType,
+	// u64 rank, u64 dims, raw bytes; :592-612) and an optional QuantizationParams record (:281-338);
+	// activation slots, tape slots and the subgraphs follow.  Everything a weight loader needs comes
+	// before the graph, so the reader stops after the variables: an archive of an imported GGUF model
+	// (block-quantised variables keep their raw payload as UInt8 with the format and the expressed
+	// shape in the record, GGUFImporter.cpp:478-491; the GGUF key/values are the metadata entries)
+	// is exposed through the same handle and accessors as a .gguf file.
+	const char kLtnnMagic[8] = { 'L', 'T', 'N', 'N', 'M', 'D', 'L', '\0' };
+
+	size_t dtype_bytes(uint32_t dtype)
+	{
+		switch (dtype)
 		{
-			uint64_t elements = 1;
-			for (uint64_t n : t.ne)
+		case LITENN_F32: case LITENN_I32: return 4;
+		case LITENN_F64: case LITENN_I64: return 8;
+		case LITENN_F16: case LITENN_BF16: return 2;
+		case LITENN_BOOL: case LITENN_F8E4M3: case LITENN_F8E5M2: case LITENN_I8: case LITENN_U8: return 1;
+		default: return 0;
+		}
+	}
+
+	int dtype_to_type_id(uint32_t dtype)
+	{
+		switch (dtype)
+		{
+		case LITENN_F32: return 0;
+		case LITENN_F16: return 1;
+		case LITENN_I8: return 24;
+		case LITENN_I32: return 26;
+		case LITENN_I64: return 27;
+		case LITENN_F64: return 28;
+		case LITENN_BF16: return 30;
+		default: return -(static_cast<int>(dtype) + 1);
+		}
+	}
+
+	// QuantizedBlockFormat (Quantization.h:31-62) -> ggml type id, 0 when this reader has no size for it
+	int block_format_to_type_id(uint32_t fmt)
+	{
+		static const int ids[] = { 0, 2, 3, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15 }; // Scalar, Q4_0 .. Q8_K
+		return fmt < sizeof(ids) / sizeof(ids[0]) ? ids[fmt] : 0;
+	}
+
+	int parse_ltnn(litenn_gguf* g)
+	{
+		const auto bad = [&]() { return fail(kLtnnAction, "LiteNN model is truncated or unreadable"); };
+		Cursor c{ g };
+		c.skip(sizeof(kLtnnMagic));
+		g->version = c.read<uint32_t>();
+		if (!c.ok)
+		{
+			return bad();
+		}
+		// ModelIO.h:1361-1364; variable names and metadata exist from version 6 on (:1386-1390)
+		if (g->version == 0 || g->version > 18)
+		{
+			return fail(kLtnnAction, "Unsupported LiteNN model version");
+		}
+		if (g->version < 6)
+		{
+			return fail(kLtnnAction, "LiteNN model version " + std::to_string(g->version) +
+			                             " has no variable names; version 6 or later is needed");
+		}
+		c.read<uint64_t>(); // forward subgraph
+		if (c.read<uint8_t>() != 0)
+		{
+			c.read<uint64_t>(); // backward subgraph
+		}
+		for (int list = 0; list < 2 && c.ok; ++list) // input names, output names
+		{
+			const uint64_t n = c.read<uint64_t>();
+			for (uint64_t i = 0; i < n && c.ok; ++i)
 			{
-				if (n == 0 || n > (uint64_t{ 1 } << 40))
+				c.skip(c.read<uint64_t>());
+			}
+		}
+		const uint64_t n_vars = c.read<uint64_t>();
+		const uint64_t n_names = c.read<uint64_t>();
+		if (!c.ok || n_vars > g->size || n_names > g->size)
+		{
+			return bad();
+		}
+		std::vector<std::string> names;
+		for (uint64_t i = 0; i < n_names && c.ok; ++i)
+		{
+			names.push_back(c.read_string());
+		}
+		if (c.ok && n_names != n_vars)
+		{
+			return fail(kLtnnAction, "LiteNN model names " + std::to_string(n_names) + " variables but holds " +
+			                             std::to_string(n_vars));
+		}
+		// metadata entries (ModelIO.h:27-39,447-505)
+		const uint64_t n_meta = c.read<uint64_t>();
+		for (uint64_t i = 0; i < n_meta && c.ok; ++i)
+		{
+			std::string key = c.read_string();
+			const uint32_t kind = c.read<uint32_t>();
+			Value v;
+			switch (kind)
+			{
+			case 0: v.type = kI64; v.i = c.read<int64_t>(); break;
+			case 1: v.type = kU64; v.u = c.read<uint64_t>(); break;
+			case 2: v.type = kF64; v.f = c.read<double>(); break;
+			case 3:
+			{
+				const uint8_t b = c.read<uint8_t>();
+				if (c.ok && b > 1)
 				{
-					return fail(kReadAction, "GGUF tensor '" + t.name + "' has non-positive dimension " + std::to_string(n));
+					return fail(kLtnnAction, "Invalid boolean value in LiteNN model metadata");
 				}
-				elements *= n;
+				v.type = kBool;
+				v.b = b != 0;
+				break;
 			}
-			const TypeInfo* ti = find_type(t.ggml_type);
-			if (!ti)
+			case 4: v.type = kString; v.s = c.read_string(); break;
+			case 5: case 6: case 7: case 8:
 			{
-				return fail(kReadAction, "Unsupported ggml tensor type '" + std::to_string(t.ggml_type) + "' for tensor '" +
-				                             t.name + "'");
+				static const uint32_t elem[] = { kI64, kU64, kF64, kBool };
+				v.type = kArray;
+				v.elem_type = elem[kind - 5];
+				v.count = c.read<uint64_t>();
+				if (v.count > g->size)
+				{
+					c.ok = false;
+				}
+				c.skip(v.count * (kind == 8 ? 1 : 8));
+				break;
 			}
-			const uint64_t row = t.ne.empty() ? 1 : t.ne[0];
-			if (row % static_cast<uint64_t>(ti->block_elements) != 0)
-			{
-				return fail(kReadAction, "GGUF tensor '" + t.name + "' has an invalid serialized byte size");
+			case 9:
+				v.type = kArray;
+				v.elem_type = kString;
+				v.count = c.read<uint64_t>();
+				for (uint64_t e = 0; e < v.count && c.ok; ++e)
+				{
+					c.skip(c.read<uint64_t>());
+				}
+				break;
+			default:
+				if (c.ok)
+				{
+					return fail(kLtnnAction, "LiteNN model contains an unknown metadata value kind");
+				}
 			}
-			t.bytes = elements / ti->block_elements * ti->block_bytes;
-			if (g->data_offset + t.offset + t.bytes > g->size)
+			g->metadata_index.emplace(key, g->metadata.size());
+			g->metadata.emplace_back(std::move(key), std::move(v));
+		}
+		for (uint64_t i = 0; i < n_vars && c.ok; ++i)
+		{
+			TensorEntry t;
+			t.name = names[i];
+			const uint32_t dtype = c.read<uint32_t>();
+			const uint64_t rank = c.read<uint64_t>();
+			if (!c.ok || rank > 16)
 			{
-				return fail(kReadAction, "Failed to read " + std::to_string(t.bytes) + " bytes for GGUF tensor '" + t.name + "'");
+				return bad();
+			}
+			std::vector<uint64_t> dims;
+			uint64_t elements = 1;
+			for (uint64_t d = 0; d < rank; ++d)
+			{
+				dims.push_back(c.read<uint64_t>());
+				if (!c.ok || (dims.back() != 0 && elements > g->size / dims.back()))
+				{
+					return bad();
+				}
+				elements *= dims.back();
+			}
+			const size_t es = dtype_bytes(dtype);
+			if (es == 0)
+			{
+				return fail(kLtnnAction, "LiteNN model variable '" + t.name + "' has an unknown data type");
+			}
+			const uint64_t payload = elements * es;
+			t.offset = c.pos;
+			c.skip(payload);
+			const uint8_t has_q = c.read<uint8_t>();
+			if (c.ok && has_q > 1)
+			{
+				return fail(kLtnnAction, "Invalid quantization metadata presence flag");
+			}
+			std::vector<uint64_t> shape = dims;
+			t.ggml_type = dtype_to_type_id(dtype);
+			if (has_q == 1)
+			{
+				const uint32_t scheme = c.read<uint32_t>();
+				c.read<uint32_t>(); // granularity
+				const uint32_t block_format = c.read<uint32_t>();
+				c.read<uint32_t>(); // storage type
+				c.read<uint32_t>(); // expressed type
+				c.read<int64_t>();  // axis
+				c.read<uint64_t>(); // group size
+				const uint64_t n_scales = c.read<uint64_t>();
+				c.skip(n_scales > g->size ? g->size + 1 : n_scales * 4);
+				const uint64_t n_zero = c.read<uint64_t>();
+				c.skip(n_zero > g->size ? g->size + 1 : n_zero * 4);
+				const uint64_t n_expr = c.read<uint64_t>();
+				if (!c.ok || n_expr > 16)
+				{
+					return bad();
+				}
+				std::vector<uint64_t> expressed;
+				for (uint64_t d = 0; d < n_expr; ++d)
+				{
+					expressed.push_back(c.read<uint64_t>());
+				}
+				// QuantizationScheme::Block with a ggml format: the payload is raw blocks
+				if (scheme == 1 && block_format != 0)
+				{
+					const int id = block_format_to_type_id(block_format);
+					if (id == 0 || dtype != LITENN_U8)
+					{
+						return fail(kLtnnAction, "LiteNN model variable '" + t.name +
+						                             "' uses a block format this reader has no layout for");
+					}
+					t.ggml_type = id;
+					shape = expressed;
+				}
+			}
+			if (shape.size() > 4)
+			{
+				return fail(kLtnnAction, "LiteNN model variable '" + t.name + "' has more than four dimensions");
+			}
+			t.ne.assign(shape.rbegin(), shape.rend()); // stored slowest dimension first
+			t.bytes = payload;
+			g->tensor_index.emplace(t.name, g->tensors.size());
+			g->tensors.push_back(std::move(t));
+		}
+		if (!c.ok)
+		{
+			return bad();
+		}
+		g->data_offset = 0;
+		// sizes implied by type and shape must be the payload sizes read above
+		std::vector<uint64_t> payloads;
+		for (const TensorEntry& t : g->tensors)
+		{
+			payloads.push_back(t.bytes);
+		}
+		if (finish_tensors(g, "LiteNN model") != 0)
+		{
+			return 1;
+		}
+		for (size_t i = 0; i < g->tensors.size(); ++i)
+		{
+			if (g->tensors[i].bytes != payloads[i])
+			{
+				return fail(kLtnnAction, "LiteNN model variable '" + g->tensors[i].name +
+				                             "' has an invalid serialized byte size");
 			}
 		}
 		return 0;
@@ -409,7 +678,8 @@ extern "C" int litenn_gguf_open(const char* path, litenn_gguf** out)
 	g->path = path;
 	g->base = static_cast<const uint8_t*>(map);
 	g->size = static_cast<size_t>(st.st_size);
-	if (parse(g) != 0)
+	const bool ltnn = std::memcmp(g->base, kLtnnMagic, sizeof(kLtnnMagic)) == 0;
+	if ((ltnn ? parse_ltnn(g) : parse(g)) != 0)
 	{
 		litenn_gguf_close(g);
 		return 1;

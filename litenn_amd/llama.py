@@ -39,8 +39,9 @@ class LLaMA:
 
     @classmethod
     def from_gguf(cls, path: str, kv_dtype=DT_F16, context_length: int = 0, device: HIP = HIP()) -> "LLaMA":
-        """Read a GGUF file, upload its decoder tensors and return the resident model (the library
-        owns the uploaded buffers).  context_length > 0 overrides the file's."""
+        """Read a GGUF file (or a LiteNN .ltnn archive of an imported model), upload its decoder
+        tensors and return the resident model (the library owns the uploaded buffers).
+        context_length > 0 overrides the file's."""
         from .gguf import GGUFFile
         with GGUFFile(path) as f:
             p = f.llama_params()

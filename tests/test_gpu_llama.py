@@ -172,3 +172,24 @@ def test_model_loaded_from_a_gguf_file(hip, oracle, tmp_path):
         hip.LLaMA.from_gguf(str(gw.llama_gguf(tmp_path / "miss.gguf", cfg, 11, skip=("ffn_up",))))
     with pytest.raises(LiteNNHipError, match="Failed to open GGUF file"):
         hip.LLaMA.from_gguf(str(tmp_path / "absent.gguf"))
+
+
+def test_model_loaded_from_an_ltnn_archive(hip, oracle, tmp_path):
+    """LiteNN model archive (the variable table SaveModel writes for an imported GGUF model,
+    Serialization/ModelIO.h:1291-1341) -> resident decoder: the same logits, bit for bit, as the
+    same model loaded from a GGUF file, and the CPU checker's within the GEMV bar."""
+    import gguf_writer as gw
+    import ltnn_writer as lw
+    cfg = synth.tiny_llama(Q4_K, block_count=2, d_model=512, heads=4, kv_heads=2, ff=768, vocab=333, context_length=48,
+                           formats={"default": Q4_K, "attn_v": Q6_K, "ffn_down": Q6_K, "token_embd": Q8_0})
+    toks = synth.prompt_tokens(cfg, 9, 5)
+    from_archive = hip.LLaMA.from_gguf(str(lw.llama_ltnn(tmp_path / "m.ltnn", cfg, 13)))
+    from_gguf = hip.LLaMA.from_gguf(str(gw.llama_gguf(tmp_path / "m.gguf", cfg, 13)))
+    got = from_archive.eval(toks)
+    assert np.array_equal(got, from_gguf.eval(toks))
+    assert rel_l2(got, oracle_model(oracle, cfg, 13).eval(toks)) < 1e-4
+    from_archive.reset()
+    from_gguf.reset()
+    assert from_archive.generate(toks, 6)[0].tolist() == from_gguf.generate(toks, 6)[0].tolist()
+    from_archive.close()
+    from_gguf.close()
