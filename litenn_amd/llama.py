@@ -35,7 +35,8 @@ class LLaMA:
     def from_config(cls, cfg, kv_dtype=DT_F16, device: HIP = HIP()) -> "LLaMA":
         return cls(cfg.block_count, cfg.embedding_length, cfg.head_count, cfg.head_count_kv,
                    cfg.feed_forward_length, cfg.vocab, cfg.context_length, cfg.rms_eps, cfg.rope_freq_base,
-                   kv_dtype=kv_dtype, device=device)
+                   rope_freq_scale=getattr(cfg, "rope_freq_scale", 1.0),
+                   rope_dimension_count=getattr(cfg, "rope_dimension_count", 0), kv_dtype=kv_dtype, device=device)
 
     @classmethod
     def from_gguf(cls, path: str, kv_dtype=DT_F16, context_length: int = 0, device: HIP = HIP()) -> "LLaMA":

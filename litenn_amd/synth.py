@@ -68,7 +68,8 @@ class LLaMAConfig:
     """Shape of a LLaMA-family decoder (tools/gguf/GGUFImporter.cpp:505-642 field names)."""
 
     def __init__(self, name, block_count, embedding_length, head_count, head_count_kv, feed_forward_length,
-                 vocab, context_length, rms_eps=float(np.float32(1e-5)), rope_freq_base=1e4, formats=None):
+                 vocab, context_length, rms_eps=float(np.float32(1e-5)), rope_freq_base=1e4, formats=None,
+                 rope_freq_scale=1.0, rope_dimension_count=0):
         self.name = name
         self.block_count = block_count
         self.embedding_length = embedding_length
@@ -79,6 +80,8 @@ class LLaMAConfig:
         self.context_length = context_length
         self.rms_eps = rms_eps
         self.rope_freq_base = rope_freq_base
+        self.rope_freq_scale = rope_freq_scale            # 1 / factor of linear scaling
+        self.rope_dimension_count = rope_dimension_count  # 0: the whole head
         # tensor-kind -> block format
         self.formats = formats or {}
 

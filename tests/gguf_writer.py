@@ -82,6 +82,11 @@ def llama_gguf(path, cfg, seed, extra_metadata=(), skip=(), arch="llama", alignm
         ("tokenizer.ggml.tokens", ARRAY, (STRING, ["<s>", "</s>", "a"])),
         ("general.file_type", U32, 2),
     ] + list(extra_metadata)
+    if getattr(cfg, "rope_freq_scale", 1.0) != 1.0:
+        md += [(f"{arch}.rope.scaling.type", STRING, "linear"),
+               (f"{arch}.rope.scaling.factor", F32, 1.0 / cfg.rope_freq_scale)]
+    if getattr(cfg, "rope_dimension_count", 0):
+        md.append((f"{arch}.rope.dimension_count", U32, cfg.rope_dimension_count))
     tensors = []
     for kind, layer, fmt, payload, n, k in synth.llama_tensors(cfg, seed):
         if kind in skip:

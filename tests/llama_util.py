@@ -12,7 +12,8 @@ ORACLE_IDS = {"token_embd": 0, "output": 1, "attn_q": 2, "attn_k": 3, "attn_v": 
 def oracle_model(oracle, cfg, seed, kv_f16=True, materialize=False, tensors=None, skip=()):
     m = oracle.LLaMA(cfg.block_count, cfg.embedding_length, cfg.head_count, cfg.head_count_kv,
                      cfg.feed_forward_length, cfg.vocab, cfg.context_length, rms_eps=cfg.rms_eps,
-                     rope_base=cfg.rope_freq_base, kv_f16=kv_f16, materialize=materialize)
+                     rope_base=cfg.rope_freq_base, rope_freq_scale=cfg.rope_freq_scale,
+                     rope_dims=cfg.rope_dimension_count, kv_f16=kv_f16, materialize=materialize)
     for kind, layer, fmt, payload, n, k in (tensors if tensors is not None else synth.llama_tensors(cfg, seed)):
         if kind in skip:
             continue

@@ -193,3 +193,27 @@ def test_model_loaded_from_an_ltnn_archive(hip, oracle, tmp_path):
     assert from_archive.generate(toks, 6)[0].tolist() == from_gguf.generate(toks, 6)[0].tolist()
     from_archive.close()
     from_gguf.close()
+
+
+def test_linear_rope_scaling_and_partial_rotation(hip, oracle, tmp_path):
+    """rope.scaling.type = linear (freq_scale = 1 / factor) and rope.dimension_count below the head
+    dimension (tools/gguf/LLaMABuilder.cpp:311-348, GGUFImporter.cpp:571-601): prompt pass, single
+    steps (fused rotate + append + attention) and the file-loaded model against the CPU checker."""
+    import gguf_writer as gw
+    cfg = synth.tiny_llama(Q4_0, block_count=2, d_model=512, heads=4, kv_heads=2, ff=768, vocab=300, context_length=40)
+    cfg.rope_freq_scale = 0.25
+    cfg.rope_dimension_count = 64  # of a head dimension of 128
+    toks = synth.prompt_tokens(cfg, 6, 2)
+    ref = oracle_model(oracle, cfg, 21)
+    dev = hip_model(hip, cfg, 21)
+    plain = synth.tiny_llama(Q4_0, block_count=2, d_model=512, heads=4, kv_heads=2, ff=768, vocab=300, context_length=40)
+    want = ref.eval(toks)
+    assert rel_l2(dev.eval(toks), want) < 1e-4
+    assert rel_l2(oracle_model(oracle, plain, 21).eval(toks), want) > 1e-2  # the parameters matter
+    for t in (5, 17, 250):  # single-token steps on top of the prompt
+        assert rel_l2(dev.eval([t]), ref.eval([t])) < 1e-4
+    loaded = hip.LLaMA.from_gguf(str(gw.llama_gguf(tmp_path / "rope.gguf", cfg, 21)))
+    dev.reset()
+    assert np.array_equal(loaded.eval(toks), dev.eval(toks))
+    loaded.close()
+    dev.close()
