@@ -45,7 +45,7 @@ namespace LiteNN
 	// src/LiteNN/Quantization.h:31-62 (the members this backend executes)
 	enum class QuantizedBlockFormat
 	{
-		Q4_0 = 1, Q8_0 = 5, Q4_K = 9, Q6_K = 11, F16 = 25, F32 = 27,
+		Q4_0 = 1, Q4_1 = 2, Q5_0 = 3, Q5_1 = 4, Q8_0 = 5, Q2_K = 7, Q3_K = 8, Q4_K = 9, Q5_K = 10, Q6_K = 11, F16 = 25, F32 = 27,
 	};
 
 	// the view of a shape the traits take (src/LiteNN/Device.h uses ShapeView the same way)

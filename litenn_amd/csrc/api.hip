@@ -135,9 +135,15 @@ namespace litenn_hip
 		switch (fmt)
 		{
 		case LITENN_FMT_Q4_0:
+		case LITENN_FMT_Q4_1:
+		case LITENN_FMT_Q5_0:
+		case LITENN_FMT_Q5_1:
 		case LITENN_FMT_Q8_0:
 			return 32;
+		case LITENN_FMT_Q2_K:
+		case LITENN_FMT_Q3_K:
 		case LITENN_FMT_Q4_K:
+		case LITENN_FMT_Q5_K:
 		case LITENN_FMT_Q6_K:
 			return 256;
 		case LITENN_FMT_F16:
@@ -154,10 +160,22 @@ namespace litenn_hip
 		{
 		case LITENN_FMT_Q4_0:
 			return 18;
+		case LITENN_FMT_Q4_1:
+			return 20;
+		case LITENN_FMT_Q5_0:
+			return 22;
+		case LITENN_FMT_Q5_1:
+			return 24;
 		case LITENN_FMT_Q8_0:
 			return 34;
+		case LITENN_FMT_Q2_K:
+			return 84;
+		case LITENN_FMT_Q3_K:
+			return 110;
 		case LITENN_FMT_Q4_K:
 			return 144;
+		case LITENN_FMT_Q5_K:
+			return 176;
 		case LITENN_FMT_Q6_K:
 			return 210;
 		case LITENN_FMT_F16:

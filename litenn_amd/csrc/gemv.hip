@@ -1133,6 +1133,91 @@ namespace litenn_hip
 				const int q = j < 16 ? (b[2 + j] & 0xF) : (b[2 + j - 16] >> 4);
 				return static_cast<float>(q - 8) * d;
 			}
+			case LITENN_FMT_Q4_1: // { fp16 d; fp16 m; u8 qs[16]; }: q d + m
+			{
+				const uint8_t* b = row + static_cast<size_t>(k_idx >> 5) * 20;
+				const int j = k_idx & 31;
+				const float d = f16_bits_to_f32(b[0] | (b[1] << 8));
+				const float m = f16_bits_to_f32(b[2] | (b[3] << 8));
+				const int q = j < 16 ? (b[4 + j] & 0xF) : (b[4 + j - 16] >> 4);
+				return __fadd_rn(__fmul_rn(static_cast<float>(q), d), m);
+			}
+			case LITENN_FMT_Q5_0: // { fp16 d; u8 qh[4]; u8 qs[16]; }: bit j of qh is the fifth bit of element j
+			{
+				const uint8_t* b = row + static_cast<size_t>(k_idx >> 5) * 22;
+				const int j = k_idx & 31;
+				const float d = f16_bits_to_f32(b[0] | (b[1] << 8));
+				const int high = (b[2 + (j >> 3)] >> (j & 7)) & 1;
+				const int low = j < 16 ? (b[6 + j] & 0xF) : (b[6 + j - 16] >> 4);
+				return static_cast<float>((low | (high << 4)) - 16) * d;
+			}
+			case LITENN_FMT_Q5_1: // { fp16 d; fp16 m; u8 qh[4]; u8 qs[16]; }
+			{
+				const uint8_t* b = row + static_cast<size_t>(k_idx >> 5) * 24;
+				const int j = k_idx & 31;
+				const float d = f16_bits_to_f32(b[0] | (b[1] << 8));
+				const float m = f16_bits_to_f32(b[2] | (b[3] << 8));
+				const int high = (b[4 + (j >> 3)] >> (j & 7)) & 1;
+				const int low = j < 16 ? (b[8 + j] & 0xF) : (b[8 + j - 16] >> 4);
+				return __fadd_rn(__fmul_rn(static_cast<float>(low | (high << 4)), d), m);
+			}
+			case LITENN_FMT_Q2_K: // { u8 scales[16]; u8 qs[64]; fp16 d; fp16 dmin; }
+			{
+				const uint8_t* b = row + static_cast<size_t>(k_idx >> 8) * 84;
+				const int e = k_idx & 255;
+				const int half = e >> 7, plane = (e >> 5) & 3, l = e & 31;
+				const float d = f16_bits_to_f32(b[80] | (b[81] << 8));
+				const float dmin = f16_bits_to_f32(b[82] | (b[83] << 8));
+				const int sc = b[e >> 4];
+				const int q = (b[16 + 32 * half + l] >> (2 * plane)) & 3;
+				const float dl = __fmul_rn(d, static_cast<float>(sc & 0xF));
+				const float ml = __fmul_rn(dmin, static_cast<float>(sc >> 4));
+				return __fsub_rn(__fmul_rn(dl, static_cast<float>(q)), ml);
+			}
+			case LITENN_FMT_Q3_K: // { u8 hmask[32]; u8 qs[64]; u8 scales[12]; fp16 d; }
+			{
+				const uint8_t* b = row + static_cast<size_t>(k_idx >> 8) * 110;
+				const int e = k_idx & 255;
+				const int half = e >> 7, plane = (e >> 5) & 3, l = e & 31;
+				const float d = f16_bits_to_f32(b[108] | (b[109] << 8));
+				int q = (b[32 + 32 * half + l] >> (2 * plane)) & 3;
+				if (!((b[l] >> (e >> 5)) & 1))
+				{
+					q -= 4;
+				}
+				// six-bit scale s, biased by 32: low four bits from nibble s / 8 of byte s % 8, top two
+				// from bits 2 (s / 4) .. of byte 8 + s % 4
+				const int s = e >> 4;
+				const int low4 = (b[96 + (s & 7)] >> (4 * (s >> 3))) & 0xF;
+				const int top2 = (b[104 + (s & 3)] >> (2 * (s >> 2))) & 3;
+				const float dl = __fmul_rn(d, static_cast<float>((low4 | (top2 << 4)) - 32));
+				return __fmul_rn(dl, static_cast<float>(q));
+			}
+			case LITENN_FMT_Q5_K: // { fp16 d; fp16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]; }
+			{
+				const uint8_t* b = row + static_cast<size_t>(k_idx >> 8) * 176;
+				const int e = k_idx & 255;
+				const float d = f16_bits_to_f32(b[0] | (b[1] << 8));
+				const float dmin = f16_bits_to_f32(b[2] | (b[3] << 8));
+				const uint8_t* sc = b + 4;
+				const int j = e >> 5, l = e & 31; // sub-block, element
+				int s, m;
+				if (j < 4)
+				{
+					s = sc[j] & 63;
+					m = sc[j + 4] & 63;
+				}
+				else
+				{
+					s = (sc[j + 4] & 0xF) | ((sc[j - 4] >> 6) << 4);
+					m = (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4);
+				}
+				const uint8_t byte = b[48 + (j >> 1) * 32 + l];
+				const int q = ((j & 1) ? (byte >> 4) : (byte & 0xF)) + 16 * ((b[16 + l] >> j) & 1);
+				const float d1 = __fmul_rn(d, static_cast<float>(s));
+				const float m1 = __fmul_rn(dmin, static_cast<float>(m));
+				return __fsub_rn(__fmul_rn(d1, static_cast<float>(q)), m1);
+			}
 			case LITENN_FMT_Q8_0:
 			{
 				const uint8_t* b = row + static_cast<size_t>(k_idx >> 5) * 34;

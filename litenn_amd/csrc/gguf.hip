@@ -49,11 +49,11 @@ namespace litenn_hip
 		};
 		const TypeInfo kTypes[] = {
 			{ 0, "f32", 1, 4, -1, LITENN_F32 },    { 1, "f16", 1, 2, -1, LITENN_F16 },
-			{ 2, "q4_0", 32, 18, LITENN_FMT_Q4_0, -1 }, { 3, "q4_1", 32, 20, -1, -1 },
-			{ 6, "q5_0", 32, 22, -1, -1 },          { 7, "q5_1", 32, 24, -1, -1 },
+			{ 2, "q4_0", 32, 18, LITENN_FMT_Q4_0, -1 }, { 3, "q4_1", 32, 20, LITENN_FMT_Q4_1, -1 },
+			{ 6, "q5_0", 32, 22, LITENN_FMT_Q5_0, -1 }, { 7, "q5_1", 32, 24, LITENN_FMT_Q5_1, -1 },
 			{ 8, "q8_0", 32, 34, LITENN_FMT_Q8_0, -1 }, { 9, "q8_1", 32, 36, -1, -1 },
-			{ 10, "q2_K", 256, 84, -1, -1 },        { 11, "q3_K", 256, 110, -1, -1 },
-			{ 12, "q4_K", 256, 144, LITENN_FMT_Q4_K, -1 }, { 13, "q5_K", 256, 176, -1, -1 },
+			{ 10, "q2_K", 256, 84, LITENN_FMT_Q2_K, -1 }, { 11, "q3_K", 256, 110, LITENN_FMT_Q3_K, -1 },
+			{ 12, "q4_K", 256, 144, LITENN_FMT_Q4_K, -1 }, { 13, "q5_K", 256, 176, LITENN_FMT_Q5_K, -1 },
 			{ 14, "q6_K", 256, 210, LITENN_FMT_Q6_K, -1 }, { 15, "q8_K", 256, 292, -1, -1 },
 			{ 24, "i8", 1, 1, -1, LITENN_I8 },      { 26, "i32", 1, 4, -1, LITENN_I32 },
 			{ 27, "i64", 1, 8, -1, LITENN_I64 },    { 28, "f64", 1, 8, -1, LITENN_F64 },

@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import numpy as np
 
-from .formats import Q4_0, Q8_0, Q4_K, Q6_K, F32, block_layout, row_bytes
+from .formats import Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, F32, block_layout, row_bytes
 
 
 def _rng(seed, *stream) -> np.random.Generator:
@@ -55,6 +55,19 @@ def quant_weights(fmt: int, n: int, k: int, seed, *stream) -> np.ndarray:
     elif fmt == Q6_K:
         blocks[..., :208] = _uniform_bytes(rng, (n, nb, 208))
         _put_u16(blocks, 208, _scales_f16(rng, (n, nb)))
+    elif fmt in (Q4_1, Q5_0, Q5_1, Q5_K):
+        # fp16 d [, fp16 m / dmin] first, everything after them uniform bytes
+        heads = {Q4_1: 2, Q5_0: 1, Q5_1: 2, Q5_K: 2}[fmt]
+        for h in range(heads):
+            _put_u16(blocks, 2 * h, _scales_f16(rng, (n, nb)))
+        blocks[..., 2 * heads:] = _uniform_bytes(rng, (n, nb, nbytes - 2 * heads))
+    elif fmt == Q2_K:
+        blocks[..., :80] = _uniform_bytes(rng, (n, nb, 80))
+        _put_u16(blocks, 80, _scales_f16(rng, (n, nb)))
+        _put_u16(blocks, 82, _scales_f16(rng, (n, nb)))
+    elif fmt == Q3_K:
+        blocks[..., :108] = _uniform_bytes(rng, (n, nb, 108))
+        _put_u16(blocks, 108, _scales_f16(rng, (n, nb)))
     else:
         raise ValueError(f"unsupported format {fmt}")
     return blocks.reshape(n, nb * nbytes)

@@ -167,9 +167,15 @@ int oracle_block_elements(int fmt)
 	switch (fmt)
 	{
 	case ORACLE_FMT_Q4_0:
+	case ORACLE_FMT_Q4_1:
+	case ORACLE_FMT_Q5_0:
+	case ORACLE_FMT_Q5_1:
 	case ORACLE_FMT_Q8_0:
 		return 32;
+	case ORACLE_FMT_Q2_K:
+	case ORACLE_FMT_Q3_K:
 	case ORACLE_FMT_Q4_K:
+	case ORACLE_FMT_Q5_K:
 	case ORACLE_FMT_Q6_K:
 		return 256;
 	case ORACLE_FMT_F16:
@@ -186,10 +192,22 @@ int oracle_block_bytes(int fmt)
 	{
 	case ORACLE_FMT_Q4_0:
 		return 18;
+	case ORACLE_FMT_Q4_1:
+		return 20;
+	case ORACLE_FMT_Q5_0:
+		return 22;
+	case ORACLE_FMT_Q5_1:
+		return 24;
 	case ORACLE_FMT_Q8_0:
 		return 34;
+	case ORACLE_FMT_Q2_K:
+		return 84;
+	case ORACLE_FMT_Q3_K:
+		return 110;
 	case ORACLE_FMT_Q4_K:
 		return 144;
+	case ORACLE_FMT_Q5_K:
+		return 176;
 	case ORACLE_FMT_Q6_K:
 		return 210;
 	case ORACLE_FMT_F16:
@@ -235,6 +253,77 @@ static void dequant_q4_0(const uint8_t* src, float* y, size_t k)
 	}
 }
 
+/* ggml block_q4_1 { fp16 d; fp16 m; u8 qs[16]; }: dequantize_row_q4_1 */
+static void dequant_q4_1(const uint8_t* src, float* y, size_t k)
+{
+	const size_t nb = k / 32;
+	for (size_t i = 0; i < nb; ++i)
+	{
+		const uint8_t* b = src + i * 20;
+		const float d = oracle_f16_to_f32(load_u16(b));
+		const float m = oracle_f16_to_f32(load_u16(b + 2));
+		const uint8_t* qs = b + 4;
+		for (int j = 0; j < 16; ++j)
+		{
+			const int x0 = qs[j] & 0x0F;
+			const int x1 = qs[j] >> 4;
+			y[i * 32 + j] = (float)x0 * d + m;
+			y[i * 32 + j + 16] = (float)x1 * d + m;
+		}
+	}
+}
+
+/* the fifth bits of a 32-element block: bit j of the little-endian u32 qh belongs to element j */
+static inline uint32_t load_u32(const uint8_t* p)
+{
+	return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+}
+
+/* ggml block_q5_0 { fp16 d; u8 qh[4]; u8 qs[16]; }: dequantize_row_q5_0 */
+static void dequant_q5_0(const uint8_t* src, float* y, size_t k)
+{
+	const size_t nb = k / 32;
+	for (size_t i = 0; i < nb; ++i)
+	{
+		const uint8_t* b = src + i * 22;
+		const float d = oracle_f16_to_f32(load_u16(b));
+		const uint32_t qh = load_u32(b + 2);
+		const uint8_t* qs = b + 6;
+		for (int j = 0; j < 16; ++j)
+		{
+			const uint8_t xh_0 = (uint8_t)(((qh >> (j + 0)) << 4) & 0x10);
+			const uint8_t xh_1 = (uint8_t)((qh >> (j + 12)) & 0x10);
+			const int x0 = ((qs[j] & 0x0F) | xh_0) - 16;
+			const int x1 = ((qs[j] >> 4) | xh_1) - 16;
+			y[i * 32 + j] = (float)x0 * d;
+			y[i * 32 + j + 16] = (float)x1 * d;
+		}
+	}
+}
+
+/* ggml block_q5_1 { fp16 d; fp16 m; u8 qh[4]; u8 qs[16]; }: dequantize_row_q5_1 */
+static void dequant_q5_1(const uint8_t* src, float* y, size_t k)
+{
+	const size_t nb = k / 32;
+	for (size_t i = 0; i < nb; ++i)
+	{
+		const uint8_t* b = src + i * 24;
+		const float d = oracle_f16_to_f32(load_u16(b));
+		const float m = oracle_f16_to_f32(load_u16(b + 2));
+		const uint32_t qh = load_u32(b + 4);
+		const uint8_t* qs = b + 8;
+		for (int j = 0; j < 16; ++j)
+		{
+			const uint8_t xh_0 = (uint8_t)(((qh >> (j + 0)) << 4) & 0x10);
+			const uint8_t xh_1 = (uint8_t)((qh >> (j + 12)) & 0x10);
+			const int x0 = (qs[j] & 0x0F) | xh_0;
+			const int x1 = (qs[j] >> 4) | xh_1;
+			y[i * 32 + j] = (float)x0 * d + m;
+			y[i * 32 + j + 16] = (float)x1 * d + m;
+		}
+	}
+}
+
 /* ggml block_q8_0 { fp16 d; i8 qs[32]; }: dequantize_row_q8_0 */
 static void dequant_q8_0(const uint8_t* src, float* y, size_t k)
 {
@@ -263,6 +352,132 @@ static inline void scale_min_k4(int j, const uint8_t* q, uint8_t* sc, uint8_t* m
 	{
 		*sc = (uint8_t)((q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4));
 		*mn = (uint8_t)((q[j + 4] >> 4) | ((q[j - 0] >> 6) << 4));
+	}
+}
+
+/* ggml block_q2_K { u8 scales[16]; u8 qs[64]; fp16 d; fp16 dmin; }: dequantize_row_q2_K */
+static void dequant_q2_k(const uint8_t* src, float* y, size_t k)
+{
+	const size_t nb = k / 256;
+	for (size_t i = 0; i < nb; ++i)
+	{
+		const uint8_t* b = src + i * 84;
+		const uint8_t* scales = b;
+		const uint8_t* q = b + 16;
+		const float d = oracle_f16_to_f32(load_u16(b + 80));
+		const float dmin = oracle_f16_to_f32(load_u16(b + 82));
+		int is = 0;
+		for (int n = 0; n < 256; n += 128)
+		{
+			int shift = 0;
+			for (int j = 0; j < 4; ++j)
+			{
+				uint8_t sc = scales[is++];
+				float dl = d * (float)(sc & 0xF), ml = dmin * (float)(sc >> 4);
+				for (int l = 0; l < 16; ++l)
+				{
+					*y++ = dl * (float)((int8_t)((q[l] >> shift) & 3)) - ml;
+				}
+				sc = scales[is++];
+				dl = d * (float)(sc & 0xF);
+				ml = dmin * (float)(sc >> 4);
+				for (int l = 0; l < 16; ++l)
+				{
+					*y++ = dl * (float)((int8_t)((q[l + 16] >> shift) & 3)) - ml;
+				}
+				shift += 2;
+			}
+			q += 32;
+		}
+	}
+}
+
+/* ggml block_q3_K { u8 hmask[32]; u8 qs[64]; u8 scales[12]; fp16 d; }: dequantize_row_q3_K */
+static void dequant_q3_k(const uint8_t* src, float* y, size_t k)
+{
+	const uint32_t kmask1 = 0x03030303u, kmask2 = 0x0f0f0f0fu;
+	const size_t nb = k / 256;
+	for (size_t i = 0; i < nb; ++i)
+	{
+		const uint8_t* b = src + i * 110;
+		const uint8_t* hm = b;
+		const uint8_t* q = b + 32;
+		const float d_all = oracle_f16_to_f32(load_u16(b + 108));
+		uint32_t aux[4];
+		aux[0] = load_u32(b + 96);
+		aux[1] = load_u32(b + 100);
+		aux[2] = load_u32(b + 104);
+		const uint32_t tmp = aux[2];
+		aux[2] = ((aux[0] >> 4) & kmask2) | (((tmp >> 4) & kmask1) << 4);
+		aux[3] = ((aux[1] >> 4) & kmask2) | (((tmp >> 6) & kmask1) << 4);
+		aux[0] = (aux[0] & kmask2) | (((tmp >> 0) & kmask1) << 4);
+		aux[1] = (aux[1] & kmask2) | (((tmp >> 2) & kmask1) << 4);
+		int8_t scales[16];
+		for (int s = 0; s < 16; ++s)
+		{
+			scales[s] = (int8_t)((aux[s / 4] >> (8 * (s % 4))) & 0xff);
+		}
+		int is = 0;
+		uint8_t m = 1;
+		for (int n = 0; n < 256; n += 128)
+		{
+			int shift = 0;
+			for (int j = 0; j < 4; ++j)
+			{
+				float dl = d_all * (float)(scales[is++] - 32);
+				for (int l = 0; l < 16; ++l)
+				{
+					*y++ = dl * (float)((int8_t)((q[l + 0] >> shift) & 3) - ((hm[l + 0] & m) ? 0 : 4));
+				}
+				dl = d_all * (float)(scales[is++] - 32);
+				for (int l = 0; l < 16; ++l)
+				{
+					*y++ = dl * (float)((int8_t)((q[l + 16] >> shift) & 3) - ((hm[l + 16] & m) ? 0 : 4));
+				}
+				shift += 2;
+				m = (uint8_t)(m << 1);
+			}
+			q += 32;
+		}
+	}
+}
+
+/* ggml block_q5_K { fp16 d; fp16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]; }: dequantize_row_q5_K */
+static void dequant_q5_k(const uint8_t* src, float* y, size_t k)
+{
+	const size_t nb = k / 256;
+	for (size_t i = 0; i < nb; ++i)
+	{
+		const uint8_t* b = src + i * 176;
+		const float d = oracle_f16_to_f32(load_u16(b));
+		const float dmin = oracle_f16_to_f32(load_u16(b + 2));
+		const uint8_t* scales = b + 4;
+		const uint8_t* qh = b + 16;
+		const uint8_t* ql = b + 48;
+		int is = 0;
+		uint8_t u1 = 1, u2 = 2;
+		for (int j = 0; j < 256; j += 64)
+		{
+			uint8_t sc, mn;
+			scale_min_k4(is + 0, scales, &sc, &mn);
+			const float d1 = d * (float)sc;
+			const float m1 = dmin * (float)mn;
+			scale_min_k4(is + 1, scales, &sc, &mn);
+			const float d2 = d * (float)sc;
+			const float m2 = dmin * (float)mn;
+			for (int l = 0; l < 32; ++l)
+			{
+				*y++ = d1 * (float)((ql[l] & 0xF) + ((qh[l] & u1) ? 16 : 0)) - m1;
+			}
+			for (int l = 0; l < 32; ++l)
+			{
+				*y++ = d2 * (float)((ql[l] >> 4) + ((qh[l] & u2) ? 16 : 0)) - m2;
+			}
+			ql += 32;
+			is += 2;
+			u1 = (uint8_t)(u1 << 2);
+			u2 = (uint8_t)(u2 << 2);
+		}
 	}
 }
 
@@ -350,11 +565,29 @@ int oracle_dequantize_row(int fmt, const uint8_t* src, float* dst, size_t k)
 	case ORACLE_FMT_Q4_0:
 		dequant_q4_0(src, dst, k);
 		break;
+	case ORACLE_FMT_Q4_1:
+		dequant_q4_1(src, dst, k);
+		break;
+	case ORACLE_FMT_Q5_0:
+		dequant_q5_0(src, dst, k);
+		break;
+	case ORACLE_FMT_Q5_1:
+		dequant_q5_1(src, dst, k);
+		break;
 	case ORACLE_FMT_Q8_0:
 		dequant_q8_0(src, dst, k);
 		break;
+	case ORACLE_FMT_Q2_K:
+		dequant_q2_k(src, dst, k);
+		break;
+	case ORACLE_FMT_Q3_K:
+		dequant_q3_k(src, dst, k);
+		break;
 	case ORACLE_FMT_Q4_K:
 		dequant_q4_k(src, dst, k);
+		break;
+	case ORACLE_FMT_Q5_K:
+		dequant_q5_k(src, dst, k);
 		break;
 	case ORACLE_FMT_Q6_K:
 		dequant_q6_k(src, dst, k);

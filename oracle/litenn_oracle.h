@@ -18,13 +18,14 @@
  *     test vectors (tests/golden/reference_vectors.json) plus closed forms.
  *   - block sizes / raw payload layout: pinned (Quantization.h:190-211,
  *     tests/GGUFImporterTest.cpp:173-178).
- *   - dequantised VALUES of Q4_0 / Q8_0 / Q4_K / Q6_K: PARITY UNPINNED against
+ *   - dequantised VALUES of Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q8_0 / Q2_K / Q3_K / Q4_K / Q5_K / Q6_K:
+ *     PARITY UNPINNED against
  *     the reference.  The arithmetic lives in ggml (third_party/llama.cpp, an
  *     empty, un-pinned submodule; call site tools/gguf/LLaMABuilder.cpp:95,149)
  *     and no reference test holds a dequantised value.  The decoders here
- *     restate ggml's published block definitions (dequantize_row_q4_0,
- *     dequantize_row_q8_0, dequantize_row_q4_K + get_scale_min_k4,
- *     dequantize_row_q6_K) and are cross-checked against an independently
+ *     restate ggml's published block definitions (dequantize_row_q4_0, _q4_1,
+ *     _q5_0, _q5_1, _q8_0, _q2_K, _q3_K, _q4_K and _q5_K + get_scale_min_k4,
+ *     _q6_K) and are cross-checked against an independently
  *     written numpy decoder, hand-packed closed-form blocks and reduction
  *     invariants, which is everything short of a real ggml build.
  */
@@ -41,8 +42,14 @@ extern "C" {
 /* QuantizedBlockFormat positional values, src/LiteNN/Quantization.h:31-62 */
 enum {
 	ORACLE_FMT_Q4_0 = 1,
+	ORACLE_FMT_Q4_1 = 2,
+	ORACLE_FMT_Q5_0 = 3,
+	ORACLE_FMT_Q5_1 = 4,
 	ORACLE_FMT_Q8_0 = 5,
+	ORACLE_FMT_Q2_K = 7,
+	ORACLE_FMT_Q3_K = 8,
 	ORACLE_FMT_Q4_K = 9,
+	ORACLE_FMT_Q5_K = 10,
 	ORACLE_FMT_Q6_K = 11,
 	ORACLE_FMT_F16 = 25,
 	ORACLE_FMT_F32 = 27,

@@ -51,7 +51,7 @@ int main()
 	// argument validation is reported as an exception carrying the library's message, device or not
 	try
 	{
-		Traits::DoQuantizedMatMul(dev, static_cast<QuantizedBlockFormat>(2), nullptr, 4, 32, nullptr, 1, nullptr);
+		Traits::DoQuantizedMatMul(dev, static_cast<QuantizedBlockFormat>(6), nullptr, 4, 32, nullptr, 1, nullptr); // Q8_1: no dequantizer
 		Check(false, "unsupported block format throws");
 	}
 	catch (const std::runtime_error& e)

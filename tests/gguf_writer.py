@@ -9,7 +9,8 @@ import struct
 import numpy as np
 
 U8, I8, U16, I16, U32, I32, F32, BOOL, STRING, ARRAY, U64, I64, F64 = range(13)
-GGML_TYPE = {"f32": 0, "f16": 1, "q4_0": 2, "q4_1": 3, "q8_0": 8, "q4_k": 12, "q5_k": 13, "q6_k": 14, "i32": 26}
+GGML_TYPE = {"f32": 0, "f16": 1, "q4_0": 2, "q4_1": 3, "q5_0": 6, "q5_1": 7, "q8_0": 8, "q2_k": 10, "q3_k": 11,
+             "q4_k": 12, "q5_k": 13, "q6_k": 14, "i32": 26}
 _SCALAR = {U8: "<B", I8: "<b", U16: "<H", I16: "<h", U32: "<I", I32: "<i", F32: "<f", BOOL: "<B", U64: "<Q",
            I64: "<q", F64: "<d"}
 
@@ -62,7 +63,8 @@ def write_gguf(path, metadata, tensors, alignment: int = 32, version: int = 3, d
     return path
 
 
-FORMAT_NAMES = {1: "q4_0", 5: "q8_0", 9: "q4_k", 11: "q6_k", 27: "f32", 25: "f16"}
+FORMAT_NAMES = {1: "q4_0", 2: "q4_1", 3: "q5_0", 4: "q5_1", 5: "q8_0", 7: "q2_k", 8: "q3_k", 9: "q4_k", 10: "q5_k",
+                11: "q6_k", 27: "f32", 25: "f16"}
 
 
 def llama_gguf(path, cfg, seed, extra_metadata=(), skip=(), arch="llama", alignment=32):

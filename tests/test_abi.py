@@ -40,5 +40,5 @@ def test_device_count_never_fails_and_errors_are_reported_without_a_device():
     # argument validation happens before any device work
     assert lib.litenn_hip_mul_mat_q(0, 9, None, 4, 100, None, 0, 1, None, None, 0, None) != 0
     assert b"block size" in lib.litenn_hip_last_error()
-    assert lib.litenn_hip_mul_mat_q(0, 2, None, 4, 32, None, 0, 1, None, None, 0, None) != 0
+    assert lib.litenn_hip_mul_mat_q(0, 6, None, 4, 32, None, 0, 1, None, None, 0, None) != 0  # Q8_1: no dequantizer
     assert b"unsupported block format" in lib.litenn_hip_last_error()

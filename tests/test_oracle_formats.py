@@ -4,17 +4,18 @@ import pytest
 
 import np_decoders
 from litenn_amd import synth
-from litenn_amd.formats import Q4_0, Q4_K, Q6_K, Q8_0
+from litenn_amd.formats import Q2_K, Q3_K, Q4_0, Q4_1, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0, FORMAT_NAMES
 
-FORMATS = [Q4_0, Q8_0, Q4_K, Q6_K]
+FORMATS = [Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K]
 
 
 def test_block_layouts_match_reference_table(oracle, golden):
     table = golden["block_layouts"]
-    for name, fmt in (("Q4_0", Q4_0), ("Q8_0", Q8_0), ("Q4_K", Q4_K), ("Q6_K", Q6_K)):
+    for fmt in FORMATS:
+        name = FORMAT_NAMES[fmt]
         assert list(oracle.block_layout(fmt)) == table[name]
         assert oracle.row_bytes(fmt, 4096) == 4096 // table[name][0] * table[name][1]
-    assert oracle.block_layout(2) == (0, 0)  # Q4_1 is not executed
+    assert oracle.block_layout(6) == (0, 0) and oracle.block_layout(12) == (0, 0)  # Q8_1, Q8_K: no dequantizer
     assert oracle.row_bytes(Q4_K, 4096 + 32) == 0  # not a whole number of super-blocks
 
 
@@ -208,4 +209,112 @@ def test_dequantize_rejects_ragged_rows(oracle):
     with pytest.raises(oracle.OracleError):
         oracle.dequantize(Q4_K, np.zeros(144, np.uint8), 1, 128)
     with pytest.raises(oracle.OracleError):
-        oracle.dequantize(3, np.zeros(22, np.uint8), 1, 32)
+        oracle.dequantize(6, np.zeros(40, np.uint8), 1, 32)
+
+
+# ---- the 32-element formats with a fifth bit and / or a minimum, and the remaining K-quants ----------
+# Expected values are written element by element straight from the published block definitions, with
+# the bit positions spelled out (not through the vectorised decoder above).
+
+def test_q4_1_closed_form(oracle):
+    """{fp16 d, fp16 m, 16 bytes}: element j is the low nibble of byte j, element j + 16 its high
+    nibble; y = q d + m."""
+    blk = np.zeros(20, np.uint8)
+    blk[0:2], blk[2:4] = _f16_bytes(0.5), _f16_bytes(-3.0)
+    qs = np.random.default_rng(3).integers(0, 256, 16, dtype=np.uint8)
+    blk[4:] = qs
+    y = oracle.dequantize(Q4_1, blk, 1, 32)[0]
+    want = np.array([(int(qs[j % 16]) >> (4 if j >= 16 else 0)) & 15 for j in range(32)], np.float32) * 0.5 - 3.0
+    assert np.array_equal(y, want)
+
+
+@pytest.mark.parametrize("fmt", [Q5_0, Q5_1])
+def test_q5_fifth_bit_one_hot(oracle, fmt):
+    """Bit j of the 32-bit little-endian qh word is the fifth bit of element j (for the low-nibble
+    half and the high-nibble half alike); Q5_0 subtracts 16, Q5_1 adds the minimum."""
+    head = 2 if fmt == Q5_0 else 4
+    for j in range(32):
+        blk = np.zeros(head + 4 + 16, np.uint8)
+        blk[0:2] = _f16_bytes(0.25)
+        if fmt == Q5_1:
+            blk[2:4] = _f16_bytes(1.5)
+        blk[head + j // 8] = 1 << (j % 8)
+        blk[head + 4:] = 0x21  # low nibbles 1, high nibbles 2
+        y = oracle.dequantize(fmt, blk, 1, 32)[0]
+        q = np.array([1] * 16 + [2] * 16, np.float32)
+        q[j] += 16
+        want = (q - 16) * 0.25 if fmt == Q5_0 else q * 0.25 + 1.5
+        assert np.array_equal(y, want.astype(np.float32)), j
+
+
+def test_q2_k_brute_force(oracle):
+    """{16 scale bytes, 64 quant bytes, fp16 d, fp16 dmin}: output e sits in half n = e / 128, bit
+    plane p = (e % 128) / 32 of byte 32 n + e % 32; scale byte e / 16: low nibble multiplies d, high
+    nibble multiplies dmin."""
+    rng = np.random.default_rng(4)
+    blk = rng.integers(0, 256, 84, dtype=np.uint8)
+    blk[80:82], blk[82:84] = _f16_bytes(0.5), _f16_bytes(0.125)
+    y = oracle.dequantize(Q2_K, blk, 1, 256)[0]
+    want = np.zeros(256, np.float32)
+    for e in range(256):
+        n, p, l = e // 128, (e % 128) // 32, e % 32
+        q = (int(blk[16 + 32 * n + l]) >> (2 * p)) & 3
+        sc = int(blk[e // 16])
+        want[e] = np.float32(np.float32(0.5 * (sc & 15)) * q) - np.float32(0.125 * (sc >> 4))
+    assert np.array_equal(y, want)
+
+
+def test_q3_k_brute_force_and_scale_packing(oracle):
+    """{32 mask bytes, 64 quant bytes, 12 scale bytes, fp16 d}: low two bits as in Q2_K; bit
+    e / 32 of mask byte e % 32 set means no -4; scale s = e / 16 is six bits, biased by 32: low
+    four from nibble (s / 8) of byte s % 8, top two from bits 2 (s / 4), .. of byte 8 + s % 4."""
+    rng = np.random.default_rng(5)
+    blk = rng.integers(0, 256, 110, dtype=np.uint8)
+    blk[108:110] = _f16_bytes(0.25)
+    y = oracle.dequantize(Q3_K, blk, 1, 256)[0]
+    want = np.zeros(256, np.float32)
+    for e in range(256):
+        n, p, l = e // 128, (e % 128) // 32, e % 32
+        q = (int(blk[32 + 32 * n + l]) >> (2 * p)) & 3
+        if not (int(blk[l]) >> (e // 32)) & 1:
+            q -= 4
+        s = e // 16
+        low4 = (int(blk[96 + s % 8]) >> (4 * (s // 8))) & 15
+        top2 = (int(blk[96 + 8 + s % 4]) >> (2 * (s // 4))) & 3
+        want[e] = np.float32(0.25 * ((low4 | (top2 << 4)) - 32)) * q
+    assert np.array_equal(y, want)
+    # one scale alone, with a value that needs its top bits
+    for s in range(16):
+        blk = np.zeros(110, np.uint8)
+        blk[0:32] = 0xFF                      # every mask bit set: no -4
+        blk[32:96] = 0x55                     # every 2-bit value 1
+        blk[108:110] = _f16_bytes(1.0)
+        value = 59                            # 6-bit field; 59 - 32 = 27
+        blk[96 + s % 8] |= (value & 15) << (4 * (s // 8))
+        blk[96 + 8 + s % 4] |= (value >> 4) << (2 * (s // 4))
+        y = oracle.dequantize(Q3_K, blk, 1, 256)[0].reshape(16, 16)
+        for t in range(16):
+            assert np.all(y[t] == (27.0 if t == s else -32.0)), (s, t)
+
+
+def test_q5_k_brute_force(oracle):
+    """{fp16 d, fp16 dmin, 12 scale bytes (packed as in Q4_K), 32 high-bit bytes, 128 nibble bytes}:
+    sub-block s = e / 32 takes the low (s even) or high (s odd) nibbles of bytes 32 (s / 2) + l and
+    bit s of high-bit byte l."""
+    rng = np.random.default_rng(6)
+    blk = rng.integers(0, 256, 176, dtype=np.uint8)
+    blk[0:2], blk[2:4] = _f16_bytes(0.5), _f16_bytes(0.25)
+    y = oracle.dequantize(Q5_K, blk, 1, 256)[0]
+    sc = blk[4:16].astype(np.int32)
+    want = np.zeros(256, np.float32)
+    for e in range(256):
+        s, l = e // 32, e % 32
+        byte = int(blk[48 + 32 * (s // 2) + l])
+        q = ((byte >> 4) if s & 1 else (byte & 15)) + 16 * ((int(blk[16 + l]) >> s) & 1)
+        if s < 4:
+            scale, mn = sc[s] & 63, sc[s + 4] & 63
+        else:
+            scale = (sc[s + 4] & 15) | ((sc[s - 4] >> 6) << 4)
+            mn = (sc[s + 4] >> 4) | ((sc[s] >> 6) << 4)
+        want[e] = np.float32(np.float32(0.5 * scale) * q) - np.float32(0.25 * mn)
+    assert np.array_equal(y, want)
