@@ -270,6 +270,59 @@ namespace litenn_hip
 			}
 		};
 
+		struct Q5_KFrag
+		{
+			static constexpr int kChunkBytes = 176;
+			static constexpr int kFragValu = 27;
+			static constexpr bool kAligned16 = true;
+			static constexpr bool kWideTile = false;
+			// header (d, dmin, 12 scale bytes), the 32 fifth-bit bytes, the 32 nibble bytes of group g
+			struct Raw { u32x4 h; uint32_t qh[8]; uint32_t q[8]; };
+			struct Scale { float s0, m0, s1, m1; int shift; }; // as Q4_K; shift = 2g, the group's bit pair in qh
+			static __device__ __forceinline__ Raw load(lds_bytes_t chunk, int g)
+			{
+				Raw r;
+				r.h = *(lds_u32x4_t)(chunk);
+				const u32x4 ha = *(lds_u32x4_t)(chunk + 16);
+				const u32x4 hb = *(lds_u32x4_t)(chunk + 32);
+				const u32x4 a = *(lds_u32x4_t)(chunk + 48 + 32 * g);
+				const u32x4 b = *(lds_u32x4_t)(chunk + 64 + 32 * g);
+				r.qh[0] = ha.x, r.qh[1] = ha.y, r.qh[2] = ha.z, r.qh[3] = ha.w;
+				r.qh[4] = hb.x, r.qh[5] = hb.y, r.qh[6] = hb.z, r.qh[7] = hb.w;
+				r.q[0] = a.x, r.q[1] = a.y, r.q[2] = a.z, r.q[3] = a.w;
+				r.q[4] = b.x, r.q[5] = b.y, r.q[6] = b.z, r.q[7] = b.w;
+				return r;
+			}
+			static __device__ __forceinline__ Scale prep(const Raw& r, int g)
+			{
+				Q4_KFrag::Raw head;
+				head.h = r.h;
+				const Q4_KFrag::Scale s = Q4_KFrag::prep(head, g);
+				return { s.s0, s.m0, s.s1, s.m1, 2 * g };
+			}
+			// low nibbles | bit 2g of qh: sub-block 2g, elements 4s ..; high nibbles | bit 2g+1: sub-block 2g+1.
+			// The fifth bit joins its nibble inside the 16-bit lane (16 units of the nibble's own scale).
+			static __device__ __forceinline__ void frag(const Raw& r, const Scale& sc, int s, uint32_t (&out)[4])
+			{
+				const uint32_t v = r.q[s], t = v >> 8;
+				const uint32_t lo_bits = r.qh[s] >> sc.shift, hi_bits = lo_bits >> 1;
+				float f0, f1, f2, f3;
+				scale_pair((v & 0x000f000fu) | ((lo_bits & 0x00010001u) << 4), sc.s0, sc.m0, f0, f2);        // bytes 0, 2
+				scale_pair((t & 0x000f000fu) | (((lo_bits >> 8) & 0x00010001u) << 4), sc.s0, sc.m0, f1, f3); // bytes 1, 3
+				out[0] = pack_f16(f0, f1);
+				out[1] = pack_f16(f2, f3);
+				scale_pair((v & 0x00f000f0u) | ((hi_bits & 0x00010001u) << 8), sc.s1, sc.m1, f0, f2);
+				scale_pair((t & 0x00f000f0u) | (((hi_bits >> 8) & 0x00010001u) << 8), sc.s1, sc.m1, f1, f3);
+				out[2] = pack_f16(f0, f1);
+				out[3] = pack_f16(f2, f3);
+			}
+			static __device__ __forceinline__ void koff(int g, int s, int& k0, int& k1)
+			{
+				k0 = 64 * g + 4 * s;
+				k1 = k0 + 32;
+			}
+		};
+
 		struct Q6_KFrag
 		{
 			static constexpr int kChunkBytes = 210;
@@ -1004,7 +1057,8 @@ namespace litenn_hip
 	                       const float* up, void* scratch_halves, hipStream_t stream)
 	{
 		const size_t rb = row_bytes(fmt, k);
-		if (fmt != LITENN_FMT_Q4_0 && fmt != LITENN_FMT_Q8_0 && fmt != LITENN_FMT_Q4_K && fmt != LITENN_FMT_Q6_K)
+		if (fmt != LITENN_FMT_Q4_0 && fmt != LITENN_FMT_Q8_0 && fmt != LITENN_FMT_Q4_K && fmt != LITENN_FMT_Q5_K &&
+		    fmt != LITENN_FMT_Q6_K)
 		{
 			return false;
 		}
@@ -1064,6 +1118,7 @@ namespace litenn_hip
 		case LITENN_FMT_Q4_0: launch_prepass_and_gemm<Q4_0Frag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
 		case LITENN_FMT_Q8_0: launch_prepass_and_gemm<Q8_0Frag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
 		case LITENN_FMT_Q4_K: launch_prepass_and_gemm<Q4_KFrag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
+		case LITENN_FMT_Q5_K: launch_prepass_and_gemm<Q5_KFrag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
 		default: launch_prepass_and_gemm<Q6_KFrag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
 		}
 		return true;

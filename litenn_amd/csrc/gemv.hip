@@ -129,6 +129,10 @@ namespace litenn_hip
 		{
 			asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c) : : "memory");
 		}
+		__device__ __forceinline__ void lds_wait(u32x4& a, u32x4& b, u32x4& c, u32x4& d, u32x4& e)
+		{
+			asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e) : : "memory");
+		}
 		__device__ __forceinline__ void lds_wait(u32x4& a, u32x4& b, u32x4& c, u32x4& d, uint32_t& e)
 		{
 			asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e) : : "memory");
@@ -420,6 +424,92 @@ namespace litenn_hip
 			}
 		};
 
+		// Q5_K: Q4_K's nibbles plus a fifth bit per element.  Super-block = {fp16 d, fp16 dmin,
+		// scales[12] (packed as in Q4_K), qh[32], qs[128]}: sub-block s takes the low (s even) or
+		// high (s odd) nibbles of bytes 32 (s / 2) + l and bit s of qh[l]; value =
+		// d sc (nibble + 16 bit) - dmin m.  A unit is the 64 elements of sub-blocks 2g, 2g+1.
+		struct Q5_KUnit
+		{
+			struct Raw { u32x4 h, a, b, ha, hb; };
+			struct Prep { float s0, s1; };
+
+			static __device__ __forceinline__ int x_offset(int unit, int i) { return unit * 64 + i; }
+			static __device__ __forceinline__ int unit_of(int k) { return k >> 6; }
+			static __device__ __forceinline__ int index_of(int k) { return k & 63; }
+			static __device__ __forceinline__ Prep prep(const float* xr)
+			{
+				return { sum_run(xr, 32), sum_run(xr + 32, 32) };
+			}
+			static __device__ __forceinline__ Raw load(const uint8_t* row, int unit)
+			{
+				const uint8_t* sb = row + static_cast<uint32_t>(unit >> 2) * 176u;
+				const uint8_t* q = sb + 48u + static_cast<uint32_t>(unit & 3) * 32u;
+				Raw r;
+				r.h = ld4(sb);
+				r.ha = ld4(sb + 16);
+				r.hb = ld4(sb + 32);
+				r.a = ld4(q);
+				r.b = ld4(q + 16);
+				return r;
+			}
+			static constexpr int kSliceBytes = 16 * 176;
+			// the super-block at the returned offset; the nibbles of the lane's group 48 + 32 g further
+			static __device__ __forceinline__ uint32_t lds_lane_offset(int u)
+			{
+				return static_cast<uint32_t>(u >> 2) * 176u;
+			}
+			static __device__ __forceinline__ Raw lds_load(uint32_t sb, int u)
+			{
+				const uint32_t q = sb + static_cast<uint32_t>(u & 3) * 32u;
+				Raw r;
+				r.h = lds_rd128<0>(sb);
+				r.ha = lds_rd128<16>(sb);
+				r.hb = lds_rd128<32>(sb);
+				r.a = lds_rd128<48>(q);
+				r.b = lds_rd128<64>(q);
+				lds_wait(r.h, r.ha, r.hb, r.a, r.b);
+				return r;
+			}
+			static __device__ __forceinline__ float dot(const Raw& r, const float* xr, const Prep& pz, int unit)
+			{
+				const int g = unit & 3;
+				const float d = f16_bits_to_f32(r.h.x);
+				const float dmin = f16_bits_to_f32(r.h.x >> 16);
+				const int sh = (g & 1) * 16;
+				const uint32_t s_lo = (r.h.y >> sh) & 0xffffu;
+				const uint32_t s_mid = (r.h.z >> sh) & 0xffffu;
+				const uint32_t s_hi = (r.h.w >> sh) & 0xffffu;
+				uint32_t sc, mn;
+				if (g < 2)
+				{
+					sc = s_lo & 0x3f3fu;
+					mn = s_mid & 0x3f3fu;
+				}
+				else
+				{
+					sc = (s_hi & 0x0f0fu) | ((s_lo >> 2) & 0x3030u);
+					mn = ((s_hi >> 4) & 0x0f0fu) | ((s_mid >> 2) & 0x3030u);
+				}
+				const uint32_t q[8] = { r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w };
+				const uint32_t qh[8] = { r.ha.x, r.ha.y, r.ha.z, r.ha.w, r.hb.x, r.hb.y, r.hb.z, r.hb.w };
+				float lo = 0.0f, hi = 0.0f;   // nibble sums at 2^-24 / 2^-20
+				float lo5 = 0.0f, hi5 = 0.0f; // fifth-bit sums at 2^-24
+#pragma unroll
+				for (int i = 0; i < 8; ++i)
+				{
+					dot8_nibbles(q[i], xr + 4 * i, xr + 32 + 4 * i, lo, hi);
+					const uint32_t bits = qh[i] >> (2 * g);
+					lo5 = dot4_bytes(bits & 0x01010101u, xr + 4 * i, lo5);
+					hi5 = dot4_bytes((bits >> 1) & 0x01010101u, xr + 32 + 4 * i, hi5);
+				}
+				const float q0 = lo * kLoNibbleScale + lo5 * (16.0f * kHalfSubnormalScale);
+				const float q1 = hi * kHiNibbleScale + hi5 * (16.0f * kHalfSubnormalScale);
+				const float sum = ub0(sc) * q0 + ub1(sc) * q1;
+				const float off = ub0(mn) * pz.s0 + ub1(mn) * pz.s1;
+				return d * sum - dmin * off;
+			}
+		};
+
 		struct Q6_KUnit
 		{
 			struct Raw { u32x4 la, lb, h; u32x2 sc; uint32_t d; };
@@ -517,6 +607,8 @@ namespace litenn_hip
 		struct HasUnitArg { static constexpr bool value = false; };
 		template <>
 		struct HasUnitArg<Q4_KUnit> { static constexpr bool value = true; };
+		template <>
+		struct HasUnitArg<Q5_KUnit> { static constexpr bool value = true; };
 		template <>
 		struct HasUnitArg<Q6_KUnit> { static constexpr bool value = true; };
 
@@ -1454,7 +1546,8 @@ namespace litenn_hip
 
 		bool is_block_format(int fmt)
 		{
-			return fmt == LITENN_FMT_Q4_0 || fmt == LITENN_FMT_Q8_0 || fmt == LITENN_FMT_Q4_K || fmt == LITENN_FMT_Q6_K;
+			return fmt == LITENN_FMT_Q4_0 || fmt == LITENN_FMT_Q8_0 || fmt == LITENN_FMT_Q4_K || fmt == LITENN_FMT_Q5_K ||
+			       fmt == LITENN_FMT_Q6_K;
 		}
 
 		bool stream_dispatch(int fmt, const GemvArgs& a, hipStream_t stream)
@@ -1470,6 +1563,7 @@ namespace litenn_hip
 			case LITENN_FMT_Q4_0: return launch_stream<Q4_0Unit>(a, stream);
 			case LITENN_FMT_Q8_0: return launch_stream<Q8_0Unit>(a, stream);
 			case LITENN_FMT_Q4_K: return launch_stream<Q4_KUnit>(a, stream);
+			case LITENN_FMT_Q5_K: return launch_stream<Q5_KUnit>(a, stream);
 			default: return launch_stream<Q6_KUnit>(a, stream);
 			}
 		}
@@ -1554,6 +1648,9 @@ namespace litenn_hip
 					break;
 				case LITENN_FMT_Q4_K:
 					launch_register<Q4_KUnit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
+					break;
+				case LITENN_FMT_Q5_K:
+					launch_register<Q5_KUnit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
 					break;
 				default:
 					launch_register<Q6_KUnit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);

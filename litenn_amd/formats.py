@@ -12,7 +12,7 @@ FORMAT_NAMES = {Q4_0: "Q4_0", Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", Q8_0: "Q
                 Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", F16: "F16", F32: "F32"}
 # formats the streaming GEMV and the matrix-core GEMM decode in-kernel; the others go through the
 # generic per-element kernels
-FAST_FORMATS = (Q4_0, Q8_0, Q4_K, Q6_K)
+FAST_FORMATS = (Q4_0, Q8_0, Q4_K, Q5_K, Q6_K)
 
 # DataType
 DT_F32, DT_F64, DT_I32, DT_I64, DT_BOOL, DT_F16, DT_BF16, DT_F8E4M3, DT_F8E5M2, DT_I8, DT_U8 = range(11)

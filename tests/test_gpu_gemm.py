@@ -10,13 +10,13 @@ import pytest
 
 from conftest import rel_l2
 from litenn_amd import synth
-from litenn_amd.formats import Q4_0, Q4_K, Q6_K, Q8_0, row_bytes
+from litenn_amd.formats import Q4_0, Q4_K, Q5_K, Q6_K, Q8_0, row_bytes
 from litenn_amd.llama import MATMUL_PRECISE
 from llama_util import hip_model, oracle_model
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
-FORMATS = [Q4_0, Q8_0, Q4_K, Q6_K]
+FORMATS = [Q4_0, Q8_0, Q4_K, Q5_K, Q6_K]
 
 
 def run_case(hip, oracle, fmt, m, n, k, seed=0, residual=False, rows=None, flags=0):
@@ -95,7 +95,7 @@ def test_gemm_is_linear_in_x_at_full_size(hip):
     assert rel_l2(y(2.0 * x1 + x2), 2.0 * y(x1) + y(x2)) <= TOL
 
 
-@pytest.mark.parametrize("fmt", [Q4_0, Q4_K])
+@pytest.mark.parametrize("fmt", [Q4_0, Q4_K, Q5_K])
 def test_prefill_through_the_matrix_cores(hip, oracle, fmt):
     """The runtime's multi-row pass with fp16 matmul operands: logits stay within the matmul bar
     of the checker's f32 pass per layer (looser after three blocks), the cache matches, and decoding

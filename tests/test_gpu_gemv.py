@@ -8,11 +8,11 @@ import pytest
 
 from conftest import rel_l2
 from litenn_amd import synth
-from litenn_amd.formats import F16, F32, Q4_0, Q4_K, Q6_K, Q8_0, row_bytes
+from litenn_amd.formats import F16, F32, Q4_0, Q4_K, Q5_K, Q6_K, Q8_0, row_bytes
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
-FORMATS = [Q4_0, Q8_0, Q4_K, Q6_K]
+FORMATS = [Q4_0, Q8_0, Q4_K, Q5_K, Q6_K]
 
 
 def run_case(hip, oracle, fmt, n, k, m=1, seed=0, residual=False, flags=0):
@@ -117,7 +117,7 @@ def test_errors_and_empty_inputs(hip):
     with pytest.raises(hip.LiteNNHipError, match="payload size"):
         hip.mul_mat_q(Q4_K, wq, 2, 256, x)
     with pytest.raises(hip.LiteNNHipError, match="unsupported block format"):
-        hip.mul_mat_q(2, wq, 1, 256, x)
+        hip.mul_mat_q(6, wq, 1, 256, x)  # Q8_1: no dequantizer
     with pytest.raises(hip.LiteNNHipError, match="block size"):
         hip.mul_mat_q(Q4_K, wq, 1, 128, x)
     empty = hip.mul_mat_q(Q4_K, hip.Tensor.from_numpy(np.zeros(0, np.uint8)), 0, 256, x)
