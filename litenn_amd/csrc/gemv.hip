@@ -125,6 +125,14 @@ namespace litenn_hip
 		{
 			asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c) : : "memory");
 		}
+		__device__ __forceinline__ void lds_wait(u32x4& a, u32x4& b, u32x2& c)
+		{
+			asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c) : : "memory");
+		}
+		__device__ __forceinline__ void lds_wait(u32x4& a, u32x4& b, u32x2& c, uint32_t& d)
+		{
+			asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : : "memory");
+		}
 		__device__ __forceinline__ void lds_wait(u32x4& a, u32x4& b, uint32_t& c)
 		{
 			asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c) : : "memory");
@@ -136,6 +144,14 @@ namespace litenn_hip
 		__device__ __forceinline__ void lds_wait(u32x4& a, u32x4& b, u32x4& c, u32x4& d, uint32_t& e)
 		{
 			asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e) : : "memory");
+		}
+		__device__ __forceinline__ void lds_wait(u32x4& a, u32x4& b, uint32_t& c, uint32_t& d)
+		{
+			asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : : "memory");
+		}
+		__device__ __forceinline__ void lds_wait(u32x4& a, u32x4& b, u32x4& c, u32x4& d, u32x2& e, uint32_t& f, uint32_t& g)
+		{
+			asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(f), "+v"(g) : : "memory");
 		}
 		__device__ __forceinline__ void lds_wait(u32x4& a, u32x4& b, u32x4& c, u32x2& d, uint32_t& e)
 		{
@@ -287,6 +303,304 @@ namespace litenn_hip
 				                       __builtin_amdgcn_alignbit(r.b.x, r.a.w, 16), xr);
 				const float a1 = block(r.b.y, r.b.z, r.b.w, r.c, xr + 32);
 				return d0 * (a0 - 8.0f * pz.s0) + d1 * (a1 - 8.0f * pz.s1);
+			}
+		};
+
+		// ---- the 32-element formats with a minimum and / or a fifth bit (units of two blocks) --------
+		// one block's nibbles (as Q4_0: low nibbles are elements 0..15, high nibbles 16..31) and,
+		// when qh is given, its fifth bits (bit j of the word belongs to element j):
+		// returns sum((nibble + 16 bit) * x)
+		template <bool FIFTH>
+		__device__ __forceinline__ float block32(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t q3, uint32_t qh,
+		                                         const float* x)
+		{
+			const uint32_t q[4] = { q0, q1, q2, q3 };
+			float lo = 0.0f, hi = 0.0f, fifth = 0.0f;
+#pragma unroll
+			for (int i = 0; i < 4; ++i)
+			{
+				dot8_nibbles(q[i], x + 4 * i, x + 16 + 4 * i, lo, hi);
+			}
+			if (FIFTH)
+			{
+#pragma unroll
+				for (int i = 0; i < 8; ++i)
+				{
+					// four bits -> four 0/1 bytes: the multiplier copies the nibble to bit offsets 0, 7, 14, 21
+					const uint32_t bits = (((qh >> (4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u;
+					fifth = dot4_bytes(bits, x + 4 * i, fifth);
+				}
+			}
+			return lo * kLoNibbleScale + hi * kHiNibbleScale + fifth * (16.0f * kHalfSubnormalScale);
+		}
+
+		struct Q4_1Unit // block { fp16 d; fp16 m; u8 qs[16]; }: q d + m
+		{
+			struct Raw { u32x4 a, b; u32x2 c; };
+			struct Prep { float s0, s1; };
+			static __device__ __forceinline__ int x_offset(int unit, int i) { return unit * 64 + i; }
+			static __device__ __forceinline__ int unit_of(int k) { return k >> 6; }
+			static __device__ __forceinline__ int index_of(int k) { return k & 63; }
+			static __device__ __forceinline__ Prep prep(const float* xr) { return { sum_run(xr, 32), sum_run(xr + 32, 32) }; }
+			static __device__ __forceinline__ Raw load(const uint8_t* row, int unit)
+			{
+				const uint8_t* p = row + static_cast<uint32_t>(unit) * 40u;
+				Raw r;
+				r.a = ld4(p);
+				r.b = ld4(p + 16);
+				r.c = ld2(p + 32);
+				return r;
+			}
+			static constexpr int kSliceBytes = 128 * 20;
+			static __device__ __forceinline__ uint32_t lds_lane_offset(int u) { return static_cast<uint32_t>(u) * 40u; }
+			static __device__ __forceinline__ Raw lds_load(uint32_t p)
+			{
+				Raw r;
+				r.a = lds_rd128<0>(p);
+				r.b = lds_rd128<16>(p);
+				r.c = lds_rd64<32>(p);
+				lds_wait(r.a, r.b, r.c);
+				return r;
+			}
+			static __device__ __forceinline__ float dot(const Raw& r, const float* xr, const Prep& pz)
+			{
+				// dwords: {d0 m0} q q q q {d1 m1} q q q q
+				const float d0 = f16_bits_to_f32(r.a.x), m0 = f16_bits_to_f32(r.a.x >> 16);
+				const float d1 = f16_bits_to_f32(r.b.y), m1 = f16_bits_to_f32(r.b.y >> 16);
+				const float a0 = block32<false>(r.a.y, r.a.z, r.a.w, r.b.x, 0u, xr);
+				const float a1 = block32<false>(r.b.z, r.b.w, r.c.x, r.c.y, 0u, xr + 32);
+				return d0 * a0 + m0 * pz.s0 + d1 * a1 + m1 * pz.s1;
+			}
+		};
+
+		struct Q5_0Unit // block { fp16 d; u8 qh[4]; u8 qs[16]; }: ((nibble | bit << 4) - 16) d
+		{
+			struct Raw { u32x4 a, b; u32x2 c; uint32_t e; };
+			struct Prep { float s0, s1; };
+			static __device__ __forceinline__ int x_offset(int unit, int i) { return unit * 64 + i; }
+			static __device__ __forceinline__ int unit_of(int k) { return k >> 6; }
+			static __device__ __forceinline__ int index_of(int k) { return k & 63; }
+			static __device__ __forceinline__ Prep prep(const float* xr) { return { sum_run(xr, 32), sum_run(xr + 32, 32) }; }
+			static __device__ __forceinline__ Raw load(const uint8_t* row, int unit)
+			{
+				const uint8_t* p = row + static_cast<uint32_t>(unit) * 44u;
+				Raw r;
+				r.a = ld4(p);
+				r.b = ld4(p + 16);
+				r.c = ld2(p + 32);
+				r.e = ld1(p + 40);
+				return r;
+			}
+			static constexpr int kSliceBytes = 128 * 22;
+			static __device__ __forceinline__ uint32_t lds_lane_offset(int u) { return static_cast<uint32_t>(u) * 44u; }
+			static __device__ __forceinline__ Raw lds_load(uint32_t p)
+			{
+				Raw r;
+				r.a = lds_rd128<0>(p);
+				r.b = lds_rd128<16>(p);
+				r.c = lds_rd64<32>(p);
+				r.e = lds_rd32<40>(p);
+				lds_wait(r.a, r.b, r.c, r.e);
+				return r;
+			}
+			static __device__ __forceinline__ float dot(const Raw& r, const float* xr, const Prep& pz)
+			{
+				// block 0 is bytes 0..21 (d, qh at 2, qs at 6), block 1 bytes 22..43 (d at 22, qh at 24, qs at 28)
+				const uint32_t w[11] = { r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, r.c.x, r.c.y, r.e };
+				const float d0 = f16_bits_to_f32(w[0]);
+				const float d1 = f16_bits_to_f32(w[5] >> 16);
+				const float a0 = block32<true>(__builtin_amdgcn_alignbit(w[2], w[1], 16), __builtin_amdgcn_alignbit(w[3], w[2], 16),
+				                               __builtin_amdgcn_alignbit(w[4], w[3], 16), __builtin_amdgcn_alignbit(w[5], w[4], 16),
+				                               __builtin_amdgcn_alignbit(w[1], w[0], 16), xr);
+				const float a1 = block32<true>(w[7], w[8], w[9], w[10], w[6], xr + 32);
+				return d0 * (a0 - 16.0f * pz.s0) + d1 * (a1 - 16.0f * pz.s1);
+			}
+		};
+
+		struct Q5_1Unit // block { fp16 d; fp16 m; u8 qh[4]; u8 qs[16]; }: (nibble | bit << 4) d + m
+		{
+			struct Raw { u32x4 a, b, c; };
+			struct Prep { float s0, s1; };
+			static __device__ __forceinline__ int x_offset(int unit, int i) { return unit * 64 + i; }
+			static __device__ __forceinline__ int unit_of(int k) { return k >> 6; }
+			static __device__ __forceinline__ int index_of(int k) { return k & 63; }
+			static __device__ __forceinline__ Prep prep(const float* xr) { return { sum_run(xr, 32), sum_run(xr + 32, 32) }; }
+			static __device__ __forceinline__ Raw load(const uint8_t* row, int unit)
+			{
+				const uint8_t* p = row + static_cast<uint32_t>(unit) * 48u;
+				Raw r;
+				r.a = ld4(p);
+				r.b = ld4(p + 16);
+				r.c = ld4(p + 32);
+				return r;
+			}
+			static constexpr int kSliceBytes = 128 * 24;
+			static __device__ __forceinline__ uint32_t lds_lane_offset(int u) { return static_cast<uint32_t>(u) * 48u; }
+			static __device__ __forceinline__ Raw lds_load(uint32_t p)
+			{
+				Raw r;
+				r.a = lds_rd128<0>(p);
+				r.b = lds_rd128<16>(p);
+				r.c = lds_rd128<32>(p);
+				lds_wait(r.a, r.b, r.c);
+				return r;
+			}
+			static __device__ __forceinline__ float dot(const Raw& r, const float* xr, const Prep& pz)
+			{
+				// dwords: {d0 m0} qh q q q q {d1 m1} qh q q q q
+				const float d0 = f16_bits_to_f32(r.a.x), m0 = f16_bits_to_f32(r.a.x >> 16);
+				const float d1 = f16_bits_to_f32(r.b.z), m1 = f16_bits_to_f32(r.b.z >> 16);
+				const float a0 = block32<true>(r.a.z, r.a.w, r.b.x, r.b.y, r.a.y, xr);
+				const float a1 = block32<true>(r.c.x, r.c.y, r.c.z, r.c.w, r.b.w, xr + 32);
+				return d0 * a0 + m0 * pz.s0 + d1 * a1 + m1 * pz.s1;
+			}
+		};
+
+		// ---- Q2_K and Q3_K: 2-bit planes ---------------------------------------------------------------
+		// Both store the low two bits of element e in plane (e % 128) / 32 of byte 32 (e / 128) + e % 32
+		// of a 64-byte field, and a scale per 16 elements.  A unit is 64 consecutive elements: two
+		// planes of one 32-byte half; its four 16-element groups have scale indices 4 u .. 4 u + 3.
+		struct Q2_KUnit // { u8 scales[16]; u8 qs[64]; fp16 d; fp16 dmin; }: d (sc & 15) q - dmin (sc >> 4)
+		{
+			struct Raw { u32x4 qa, qb; uint32_t sc, dd; };
+			struct Prep { float s[4]; };
+			static __device__ __forceinline__ int x_offset(int unit, int i) { return unit * 64 + i; }
+			static __device__ __forceinline__ int unit_of(int k) { return k >> 6; }
+			static __device__ __forceinline__ int index_of(int k) { return k & 63; }
+			static __device__ __forceinline__ Prep prep(const float* xr)
+			{
+				Prep p;
+#pragma unroll
+				for (int g = 0; g < 4; ++g)
+				{
+					p.s[g] = sum_run(xr + 16 * g, 16);
+				}
+				return p;
+			}
+			static __device__ __forceinline__ Raw load(const uint8_t* row, int unit)
+			{
+				const uint8_t* sb = row + static_cast<uint32_t>(unit >> 2) * 84u;
+				const uint8_t* q = sb + 16u + static_cast<uint32_t>((unit >> 1) & 1) * 32u;
+				Raw r;
+				r.qa = ld4(q);
+				r.qb = ld4(q + 16);
+				r.sc = ld1(sb + 4u * static_cast<uint32_t>(unit & 3));
+				r.dd = ld1(sb + 80);
+				return r;
+			}
+			static constexpr int kSliceBytes = 16 * 84;
+			static __device__ __forceinline__ uint32_t lds_lane_offset(int u) { return static_cast<uint32_t>(u >> 2) * 84u; }
+			static __device__ __forceinline__ Raw lds_load(uint32_t sb, int u)
+			{
+				const uint32_t q = sb + static_cast<uint32_t>((u >> 1) & 1) * 32u;
+				Raw r;
+				r.qa = lds_rd128<16>(q);
+				r.qb = lds_rd128<32>(q);
+				r.sc = lds_rd32<0>(sb + 4u * static_cast<uint32_t>(u & 3));
+				r.dd = lds_rd32<80>(sb);
+				lds_wait(r.qa, r.qb, r.sc, r.dd);
+				return r;
+			}
+			static __device__ __forceinline__ float dot(const Raw& r, const float* xr, const Prep& pz, int unit)
+			{
+				const uint32_t q[8] = { r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w };
+				const int plane0 = (unit & 1) * 4; // bit offset of the unit's first plane
+				const float d = f16_bits_to_f32(r.dd), dmin = f16_bits_to_f32(r.dd >> 16);
+				float sum = 0.0f, off = 0.0f;
+#pragma unroll
+				for (int g = 0; g < 4; ++g) // group g: plane g / 2, bytes 16 (g % 2) .. + 15
+				{
+					float a = 0.0f;
+#pragma unroll
+					for (int i = 0; i < 4; ++i)
+					{
+						a = dot4_bytes((q[4 * (g & 1) + i] >> (plane0 + 2 * (g >> 1))) & 0x03030303u, xr + 16 * g + 4 * i, a);
+					}
+					const uint32_t sc = (r.sc >> (8 * g)) & 0xffu;
+					sum += static_cast<float>(sc & 0xFu) * a;
+					off += static_cast<float>(sc >> 4) * pz.s[g];
+				}
+				return d * (sum * kHalfSubnormalScale) - dmin * off;
+			}
+		};
+
+		struct Q3_KUnit // { u8 hmask[32]; u8 qs[64]; u8 scales[12]; fp16 d; }: d (sc - 32) (q - (bit ? 0 : 4))
+		{
+			struct Raw { u32x4 ha, hb, qa, qb; u32x2 s01; uint32_t s2, d; };
+			struct Prep { float s[4]; };
+			static __device__ __forceinline__ int x_offset(int unit, int i) { return unit * 64 + i; }
+			static __device__ __forceinline__ int unit_of(int k) { return k >> 6; }
+			static __device__ __forceinline__ int index_of(int k) { return k & 63; }
+			static __device__ __forceinline__ Prep prep(const float* xr)
+			{
+				Prep p;
+#pragma unroll
+				for (int g = 0; g < 4; ++g)
+				{
+					p.s[g] = sum_run(xr + 16 * g, 16);
+				}
+				return p;
+			}
+			static __device__ __forceinline__ Raw load(const uint8_t* row, int unit)
+			{
+				const uint8_t* sb = row + static_cast<uint32_t>(unit >> 2) * 110u;
+				const uint8_t* q = sb + 32u + static_cast<uint32_t>((unit >> 1) & 1) * 32u;
+				Raw r;
+				r.ha = ld4(sb);
+				r.hb = ld4(sb + 16);
+				r.qa = ld4(q);
+				r.qb = ld4(q + 16);
+				r.s01 = ld2(sb + 96);
+				r.s2 = ld1(sb + 104);
+				r.d = ldh(sb + 108);
+				return r;
+			}
+			static constexpr int kSliceBytes = 16 * 110;
+			static __device__ __forceinline__ uint32_t lds_lane_offset(int u) { return static_cast<uint32_t>(u >> 2) * 110u; }
+			static __device__ __forceinline__ Raw lds_load(uint32_t sb, int u)
+			{
+				const uint32_t q = sb + static_cast<uint32_t>((u >> 1) & 1) * 32u;
+				Raw r;
+				r.ha = lds_rd128<0>(sb);
+				r.hb = lds_rd128<16>(sb);
+				r.qa = lds_rd128<32>(q);
+				r.qb = lds_rd128<48>(q);
+				r.s01 = lds_rd64<96>(sb);
+				r.s2 = lds_rd32<104>(sb);
+				r.d = lds_rd16<108>(sb);
+				lds_wait(r.ha, r.hb, r.qa, r.qb, r.s01, r.s2, r.d);
+				return r;
+			}
+			static __device__ __forceinline__ float dot(const Raw& r, const float* xr, const Prep& pz, int unit)
+			{
+				const uint32_t q[8] = { r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w };
+				const uint32_t hm[8] = { r.ha.x, r.ha.y, r.ha.z, r.ha.w, r.hb.x, r.hb.y, r.hb.z, r.hb.w };
+				const int u = unit & 3;
+				const int plane0 = (u & 1) * 4; // bit offset of the unit's first plane in the quant bytes
+				const int hbit0 = 2 * u;        // ... and of its first high-bit plane in the mask bytes
+				// the unit's four six-bit scales 4 u .. 4 u + 3: low four bits are the low (u < 2) or high
+				// nibbles of scale bytes 4 (u & 1) .. + 3, the top two bits 2 u, 2 u + 1 of bytes 8 .. 11
+				const uint32_t low_word = (u & 1) ? r.s01.y : r.s01.x;
+				const uint32_t low4 = (low_word >> (4 * (u >> 1))) & 0x0f0f0f0fu;
+				const uint32_t top2 = ((r.s2 >> (2 * u)) & 0x03030303u) << 4;
+				const uint32_t scales = low4 | top2;
+				float sum = 0.0f;
+#pragma unroll
+				for (int g = 0; g < 4; ++g) // group g: plane g / 2, bytes 16 (g % 2) .. + 15
+				{
+					float a = 0.0f;
+#pragma unroll
+					for (int i = 0; i < 4; ++i)
+					{
+						const int w = 4 * (g & 1) + i;
+						const uint32_t two = (q[w] >> (plane0 + 2 * (g >> 1))) & 0x03030303u;
+						const uint32_t high = (hm[w] >> (hbit0 + (g >> 1))) & 0x01010101u;
+						a = dot4_bytes(two | (high << 2), xr + 16 * g + 4 * i, a); // q + 4 bit
+					}
+					const float sc = static_cast<float>(static_cast<int>((scales >> (8 * g)) & 0xffu) - 32);
+					sum += sc * (a * kHalfSubnormalScale - 4.0f * pz.s[g]);
+				}
+				return f16_bits_to_f32(r.d) * sum;
 			}
 		};
 
@@ -609,6 +923,10 @@ namespace litenn_hip
 		struct HasUnitArg<Q4_KUnit> { static constexpr bool value = true; };
 		template <>
 		struct HasUnitArg<Q5_KUnit> { static constexpr bool value = true; };
+		template <>
+		struct HasUnitArg<Q2_KUnit> { static constexpr bool value = true; };
+		template <>
+		struct HasUnitArg<Q3_KUnit> { static constexpr bool value = true; };
 		template <>
 		struct HasUnitArg<Q6_KUnit> { static constexpr bool value = true; };
 
@@ -1546,8 +1864,9 @@ namespace litenn_hip
 
 		bool is_block_format(int fmt)
 		{
-			return fmt == LITENN_FMT_Q4_0 || fmt == LITENN_FMT_Q8_0 || fmt == LITENN_FMT_Q4_K || fmt == LITENN_FMT_Q5_K ||
-			       fmt == LITENN_FMT_Q6_K;
+			return fmt == LITENN_FMT_Q4_0 || fmt == LITENN_FMT_Q4_1 || fmt == LITENN_FMT_Q5_0 || fmt == LITENN_FMT_Q5_1 ||
+			       fmt == LITENN_FMT_Q8_0 || fmt == LITENN_FMT_Q2_K || fmt == LITENN_FMT_Q3_K || fmt == LITENN_FMT_Q4_K ||
+			       fmt == LITENN_FMT_Q5_K || fmt == LITENN_FMT_Q6_K;
 		}
 
 		bool stream_dispatch(int fmt, const GemvArgs& a, hipStream_t stream)
@@ -1561,7 +1880,12 @@ namespace litenn_hip
 			switch (fmt)
 			{
 			case LITENN_FMT_Q4_0: return launch_stream<Q4_0Unit>(a, stream);
+			case LITENN_FMT_Q4_1: return launch_stream<Q4_1Unit>(a, stream);
+			case LITENN_FMT_Q5_0: return launch_stream<Q5_0Unit>(a, stream);
+			case LITENN_FMT_Q5_1: return launch_stream<Q5_1Unit>(a, stream);
 			case LITENN_FMT_Q8_0: return launch_stream<Q8_0Unit>(a, stream);
+			case LITENN_FMT_Q2_K: return launch_stream<Q2_KUnit>(a, stream);
+			case LITENN_FMT_Q3_K: return launch_stream<Q3_KUnit>(a, stream);
 			case LITENN_FMT_Q4_K: return launch_stream<Q4_KUnit>(a, stream);
 			case LITENN_FMT_Q5_K: return launch_stream<Q5_KUnit>(a, stream);
 			default: return launch_stream<Q6_KUnit>(a, stream);
@@ -1643,8 +1967,23 @@ namespace litenn_hip
 				case LITENN_FMT_Q4_0:
 					launch_register<Q4_0Unit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
 					break;
+				case LITENN_FMT_Q4_1:
+					launch_register<Q4_1Unit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
+					break;
+				case LITENN_FMT_Q5_0:
+					launch_register<Q5_0Unit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
+					break;
+				case LITENN_FMT_Q5_1:
+					launch_register<Q5_1Unit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
+					break;
 				case LITENN_FMT_Q8_0:
 					launch_register<Q8_0Unit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
+					break;
+				case LITENN_FMT_Q2_K:
+					launch_register<Q2_KUnit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
+					break;
+				case LITENN_FMT_Q3_K:
+					launch_register<Q3_KUnit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);
 					break;
 				case LITENN_FMT_Q4_K:
 					launch_register<Q4_KUnit>(w, xi, yi, ri, static_cast<int>(n), static_cast<int>(k), rb, stream);

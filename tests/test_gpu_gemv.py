@@ -8,11 +8,11 @@ import pytest
 
 from conftest import rel_l2
 from litenn_amd import synth
-from litenn_amd.formats import F16, F32, Q4_0, Q4_K, Q5_K, Q6_K, Q8_0, row_bytes
+from litenn_amd.formats import F16, F32, Q2_K, Q3_K, Q4_0, Q4_1, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0, row_bytes
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
-FORMATS = [Q4_0, Q8_0, Q4_K, Q5_K, Q6_K]
+FORMATS = [Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K]
 
 
 def run_case(hip, oracle, fmt, n, k, m=1, seed=0, residual=False, flags=0):
@@ -54,7 +54,7 @@ def test_north_star_shape_q4_k_4096x14336(hip, oracle):
 @pytest.mark.parametrize("fmt", FORMATS)
 def test_ragged_shapes_take_the_generic_kernel(hip, oracle, fmt):
     """K not a multiple of 256 (single blocks, odd block counts) and tiny N."""
-    for n, k in [(1, 32), (3, 96), (7, 32 * 37)] if fmt in (Q4_0, Q8_0) else [(1, 256), (3, 768)]:
+    for n, k in [(1, 32), (3, 96), (7, 32 * 37)] if fmt in (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0) else [(1, 256), (3, 768)]:
         assert run_case(hip, oracle, fmt, n, k, seed=k) <= TOL
 
 
