@@ -47,8 +47,7 @@ enum litenn_dtype {
 /* QuantizedBlockFormat, src/LiteNN/Quantization.h:31-62 (only the members this backend executes:
  * the ggml formats that have a dequantizer and a layout in the reference's table, :186-217; Q8_1 and
  * Q8_K have none in ggml and are refused, as tools/gguf/LLaMABuilder.cpp:95-101 refuses them).
- * All of them are decoded inside the streaming GEMV; Q4_0, Q8_0, Q4_K, Q5_K and Q6_K also inside the
- * matrix-core GEMM (multi-row inputs in the other formats run the GEMV row by row). */
+ * All of them are decoded inside the streaming GEMV and the matrix-core GEMM. */
 enum litenn_block_format {
 	LITENN_FMT_Q4_0 = 1, LITENN_FMT_Q4_1 = 2, LITENN_FMT_Q5_0 = 3, LITENN_FMT_Q5_1 = 4, LITENN_FMT_Q8_0 = 5,
 	LITENN_FMT_Q2_K = 7, LITENN_FMT_Q3_K = 8, LITENN_FMT_Q4_K = 9, LITENN_FMT_Q5_K = 10, LITENN_FMT_Q6_K = 11,

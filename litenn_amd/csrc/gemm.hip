@@ -163,6 +163,248 @@ namespace litenn_hip
 			}
 		};
 
+		// One dword of packed nibbles plus their fifth bits -> 8 values: `lo4` / `hi4` hold the fifth
+		// bits of the four low-nibble / high-nibble elements (bit j for byte j).  The bit joins its
+		// nibble inside the 16-bit lane (16 units of the nibble's own scale); the multipliers copy
+		// bits 0 and 2 (bytes 0, 2) or 1 and 3 (bytes 1, 3) to the lanes' positions.
+		__device__ __forceinline__ void nibbles8_fifth(uint32_t v, uint32_t lo4, uint32_t hi4, float s_lo, float b_lo,
+		                                                float s_hi, float b_hi, uint32_t (&out)[4])
+		{
+			const uint32_t t = v >> 8;
+			float f0, f1, f2, f3;
+			scale_pair((v & 0x000f000fu) | ((lo4 * 0x00040010u) & 0x00100010u), s_lo, b_lo, f0, f2); // bytes 0, 2
+			scale_pair((t & 0x000f000fu) | ((lo4 * 0x00020008u) & 0x00100010u), s_lo, b_lo, f1, f3); // bytes 1, 3
+			out[0] = pack_f16(f0, f1);
+			out[1] = pack_f16(f2, f3);
+			scale_pair((v & 0x00f000f0u) | ((hi4 * 0x00400100u) & 0x01000100u), s_hi, b_hi, f0, f2);
+			scale_pair((t & 0x00f000f0u) | ((hi4 * 0x00200080u) & 0x01000100u), s_hi, b_hi, f1, f3);
+			out[2] = pack_f16(f0, f1);
+			out[3] = pack_f16(f2, f3);
+		}
+
+		struct Q4_1Frag // block { fp16 d; fp16 m; u8 qs[16]; }: q d + m
+		{
+			static constexpr int kChunkBytes = 8 * 20;
+			static constexpr int kFragValu = 19;
+			static constexpr bool kAligned16 = true;
+			static constexpr bool kWideTile = false;
+			struct Raw { uint32_t w[10]; }; // blocks 2g and 2g+1: {d m} q q q q {d m} q q q q
+			struct Scale { float d0, m0, d1, m1; };
+			static __device__ __forceinline__ Raw load(lds_bytes_t chunk, int g)
+			{
+				Raw r;
+				lds_bytes_t p = chunk + 40 * g;
+#pragma unroll
+				for (int i = 0; i < 10; ++i)
+				{
+					r.w[i] = ld_u32_aligned(p + 4 * i);
+				}
+				return r;
+			}
+			static __device__ __forceinline__ Scale prep(const Raw& r, int)
+			{
+				return { f16_bits_to_f32(r.w[0]), f16_bits_to_f32(r.w[0] >> 16), f16_bits_to_f32(r.w[5]),
+					     f16_bits_to_f32(r.w[5] >> 16) };
+			}
+			static __device__ __forceinline__ void frag(const Raw& r, const Scale& sc, int s, uint32_t (&out)[4])
+			{
+				const int b = s >> 2, t = s & 3;
+				const float d = b == 0 ? sc.d0 : sc.d1, m = b == 0 ? sc.m0 : sc.m1;
+				nibbles8(r.w[5 * b + 1 + t], d * kTwo24, m, d * kTwo20, m, out);
+			}
+			static __device__ __forceinline__ void koff(int g, int s, int& k0, int& k1) { Q4_0Frag::koff(g, s, k0, k1); }
+		};
+
+		struct Q5_0Frag // block { fp16 d; u8 qh[4]; u8 qs[16]; }: ((nibble | bit << 4) - 16) d
+		{
+			static constexpr int kChunkBytes = 8 * 22;
+			static constexpr int kFragValu = 33;
+			static constexpr bool kAligned16 = true;
+			static constexpr bool kWideTile = false;
+			struct Raw { uint32_t w[11]; }; // blocks 2g and 2g+1: bytes 0..21 and 22..43
+			struct Scale { float d0, d1; };
+			static __device__ __forceinline__ Raw load(lds_bytes_t chunk, int g)
+			{
+				Raw r;
+				lds_bytes_t p = chunk + 44 * g;
+#pragma unroll
+				for (int i = 0; i < 11; ++i)
+				{
+					r.w[i] = ld_u32_aligned(p + 4 * i);
+				}
+				return r;
+			}
+			static __device__ __forceinline__ Scale prep(const Raw& r, int)
+			{
+				return { f16_bits_to_f32(r.w[0]), f16_bits_to_f32(r.w[5] >> 16) };
+			}
+			static __device__ __forceinline__ void frag(const Raw& r, const Scale& sc, int s, uint32_t (&out)[4])
+			{
+				const int b = s >> 2, t = s & 3;
+				// block 0: qh at byte 2, qs at byte 6; block 1: qh at byte 24, qs at byte 28
+				const uint32_t qh = b == 0 ? ((r.w[0] >> 16) | (r.w[1] << 16)) : r.w[6];
+				const uint32_t qs = b == 0 ? ((r.w[1 + t] >> 16) | (r.w[2 + t] << 16)) : r.w[7 + t];
+				const float d = b == 0 ? sc.d0 : sc.d1;
+				nibbles8_fifth(qs, (qh >> (4 * t)) & 0xFu, (qh >> (16 + 4 * t)) & 0xFu, d * kTwo24, -16.0f * d, d * kTwo20,
+				               -16.0f * d, out);
+			}
+			static __device__ __forceinline__ void koff(int g, int s, int& k0, int& k1) { Q4_0Frag::koff(g, s, k0, k1); }
+		};
+
+		struct Q5_1Frag // block { fp16 d; fp16 m; u8 qh[4]; u8 qs[16]; }: (nibble | bit << 4) d + m
+		{
+			static constexpr int kChunkBytes = 8 * 24;
+			static constexpr int kFragValu = 33;
+			static constexpr bool kAligned16 = true;
+			static constexpr bool kWideTile = false;
+			struct Raw { uint32_t w[12]; }; // {d m} qh q q q q, twice
+			struct Scale { float d0, m0, d1, m1; };
+			static __device__ __forceinline__ Raw load(lds_bytes_t chunk, int g)
+			{
+				Raw r;
+				lds_bytes_t p = chunk + 48 * g;
+#pragma unroll
+				for (int i = 0; i < 12; ++i)
+				{
+					r.w[i] = ld_u32_aligned(p + 4 * i);
+				}
+				return r;
+			}
+			static __device__ __forceinline__ Scale prep(const Raw& r, int)
+			{
+				return { f16_bits_to_f32(r.w[0]), f16_bits_to_f32(r.w[0] >> 16), f16_bits_to_f32(r.w[6]),
+					     f16_bits_to_f32(r.w[6] >> 16) };
+			}
+			static __device__ __forceinline__ void frag(const Raw& r, const Scale& sc, int s, uint32_t (&out)[4])
+			{
+				const int b = s >> 2, t = s & 3;
+				const uint32_t qh = r.w[6 * b + 1];
+				const float d = b == 0 ? sc.d0 : sc.d1, m = b == 0 ? sc.m0 : sc.m1;
+				nibbles8_fifth(r.w[6 * b + 2 + t], (qh >> (4 * t)) & 0xFu, (qh >> (16 + 4 * t)) & 0xFu, d * kTwo24, m,
+				               d * kTwo20, m, out);
+			}
+			static __device__ __forceinline__ void koff(int g, int s, int& k0, int& k1) { Q4_0Frag::koff(g, s, k0, k1); }
+		};
+
+		// Q2_K and Q3_K: lane g owns the 64 consecutive elements 64 g .. of the super-block: planes
+		// 2 (g % 2) and 2 (g % 2) + 1 of the 32 quant bytes of half g / 2.  Step s covers elements
+		// 16 (s / 2) + 8 (s % 2) .. + 7 of the lane's 64: group s / 2 (one scale), plane (s / 2) / 2,
+		// bytes 16 ((s / 2) % 2) + 8 (s % 2) .. + 7.
+		struct Q2_KFrag // { u8 scales[16]; u8 qs[64]; fp16 d; fp16 dmin; }: d (sc & 15) q - dmin (sc >> 4)
+		{
+			static constexpr int kChunkBytes = 84;
+			static constexpr int kFragValu = 24;
+			static constexpr bool kAligned16 = false; // 84-byte blocks: 4-byte aligned
+			static constexpr bool kWideTile = false;
+			struct Raw { uint32_t q[8]; uint32_t sc, dd; };
+			struct Scale { float s[4], b[4]; int shift; };
+			static __device__ __forceinline__ Raw load(lds_bytes_t chunk, int g)
+			{
+				Raw r;
+				lds_bytes_t q = chunk + 16 + 32 * (g >> 1);
+#pragma unroll
+				for (int i = 0; i < 8; ++i)
+				{
+					r.q[i] = ld_u32_aligned(q + 4 * i);
+				}
+				r.sc = ld_u32_aligned(chunk + 4 * g);
+				r.dd = ld_u32_aligned(chunk + 80);
+				return r;
+			}
+			static __device__ __forceinline__ Scale prep(const Raw& r, int g)
+			{
+				const float d = f16_bits_to_f32(r.dd), dmin = f16_bits_to_f32(r.dd >> 16);
+				Scale s;
+#pragma unroll
+				for (int i = 0; i < 4; ++i)
+				{
+					const uint32_t sc = (r.sc >> (8 * i)) & 0xffu;
+					s.s[i] = d * static_cast<float>(sc & 0xFu) * kTwo24;
+					s.b[i] = -(dmin * static_cast<float>(sc >> 4));
+				}
+				s.shift = 4 * (g & 1);
+				return s;
+			}
+			static __device__ __forceinline__ void frag(const Raw& r, const Scale& sc, int s, uint32_t (&out)[4])
+			{
+				const int grp = s >> 1, w0 = 4 * (grp & 1) + 2 * (s & 1);
+				const int shift = sc.shift + 2 * (grp >> 1);
+				bytes4((r.q[w0] >> shift) & 0x03030303u, sc.s[grp], sc.b[grp], out[0], out[1]);
+				bytes4((r.q[w0 + 1] >> shift) & 0x03030303u, sc.s[grp], sc.b[grp], out[2], out[3]);
+			}
+			static __device__ __forceinline__ void koff(int g, int s, int& k0, int& k1)
+			{
+				k0 = 64 * g + 8 * s;
+				k1 = k0 + 4;
+			}
+		};
+
+		struct Q3_KFrag // { u8 hmask[32]; u8 qs[64]; u8 scales[12]; fp16 d; }: d (sc - 32) (q - (bit ? 0 : 4))
+		{
+			static constexpr int kChunkBytes = 110;
+			static constexpr int kFragValu = 34;
+			static constexpr bool kAligned16 = false; // 110-byte blocks: 2-byte aligned
+			static constexpr bool kWideTile = false;
+			struct Raw { uint32_t hm[8], q[8], s[3], d; };
+			struct Scale { float s[4], b[4]; int shift, hshift; };
+			static __device__ __forceinline__ Raw load(lds_bytes_t chunk, int g)
+			{
+				Raw r;
+				lds_bytes_t q = chunk + 32 + 32 * (g >> 1);
+#pragma unroll
+				for (int i = 0; i < 8; ++i)
+				{
+					r.hm[i] = ld_u32(chunk + 4 * i);
+					r.q[i] = ld_u32(q + 4 * i);
+				}
+#pragma unroll
+				for (int i = 0; i < 3; ++i)
+				{
+					r.s[i] = ld_u32(chunk + 96 + 4 * i);
+				}
+				r.d = ld_u16(chunk + 108);
+				return r;
+			}
+			// the lane's four six-bit scales 4 g .. 4 g + 3, biased by 32: low four bits are the low
+			// (g < 2) or high nibbles of scale bytes 4 (g % 2) .. + 3, the top two are bits 2 g, 2 g + 1
+			// of bytes 8 .. 11
+			static __device__ __forceinline__ Scale prep(const Raw& r, int g)
+			{
+				const float d = f16_bits_to_f32(r.d);
+				const uint32_t low4 = (((g & 1) ? r.s[1] : r.s[0]) >> (4 * (g >> 1))) & 0x0f0f0f0fu;
+				const uint32_t top2 = ((r.s[2] >> (2 * g)) & 0x03030303u) << 4;
+				const uint32_t six = low4 | top2;
+				Scale s;
+#pragma unroll
+				for (int i = 0; i < 4; ++i)
+				{
+					const float ds = d * static_cast<float>(static_cast<int>((six >> (8 * i)) & 0xffu) - 32);
+					s.s[i] = ds * kTwo24;
+					s.b[i] = -4.0f * ds;
+				}
+				s.shift = 4 * (g & 1);
+				s.hshift = 2 * g;
+				return s;
+			}
+			static __device__ __forceinline__ void frag(const Raw& r, const Scale& sc, int s, uint32_t (&out)[4])
+			{
+				const int grp = s >> 1, w0 = 4 * (grp & 1) + 2 * (s & 1);
+				const int shift = sc.shift + 2 * (grp >> 1), hshift = sc.hshift + (grp >> 1);
+#pragma unroll
+				for (int w = 0; w < 2; ++w)
+				{
+					const uint32_t two = (r.q[w0 + w] >> shift) & 0x03030303u;
+					const uint32_t high = ((r.hm[w0 + w] >> hshift) & 0x01010101u) << 2;
+					bytes4(two | high, sc.s[grp], sc.b[grp], out[2 * w], out[2 * w + 1]); // (q + 4 bit - 4) d (sc - 32)
+				}
+			}
+			static __device__ __forceinline__ void koff(int g, int s, int& k0, int& k1)
+			{
+				k0 = 64 * g + 8 * s;
+				k1 = k0 + 4;
+			}
+		};
+
 		struct Q8_0Frag
 		{
 			static constexpr int kChunkBytes = 8 * 34;
@@ -1057,9 +1299,12 @@ namespace litenn_hip
 	                       const float* up, void* scratch_halves, hipStream_t stream)
 	{
 		const size_t rb = row_bytes(fmt, k);
-		if (fmt != LITENN_FMT_Q4_0 && fmt != LITENN_FMT_Q8_0 && fmt != LITENN_FMT_Q4_K && fmt != LITENN_FMT_Q5_K &&
-		    fmt != LITENN_FMT_Q6_K)
+		switch (fmt)
 		{
+		case LITENN_FMT_Q4_0: case LITENN_FMT_Q4_1: case LITENN_FMT_Q5_0: case LITENN_FMT_Q5_1: case LITENN_FMT_Q8_0:
+		case LITENN_FMT_Q2_K: case LITENN_FMT_Q3_K: case LITENN_FMT_Q4_K: case LITENN_FMT_Q5_K: case LITENN_FMT_Q6_K:
+			break;
+		default:
 			return false;
 		}
 		if (count < 1 || count > 3 || (count > 1 && residual) || (norm_w && up))
@@ -1068,7 +1313,7 @@ namespace litenn_hip
 		}
 		// Q6_K blocks (210 bytes) are fetched from the 16-byte boundary below them; the other formats'
 		// chunks must start on one
-		const uintptr_t w_align = fmt == LITENN_FMT_Q6_K ? 2 : 16;
+		const uintptr_t w_align = fmt == LITENN_FMT_Q6_K || fmt == LITENN_FMT_Q3_K ? 2 : (fmt == LITENN_FMT_Q2_K ? 4 : 16);
 		for (int i = 0; i < count; ++i)
 		{
 			if (reinterpret_cast<uintptr_t>(wq[i]) % w_align != 0 || n[i] == 0 || n[i] > 0x7fffffffu)
@@ -1116,6 +1361,11 @@ namespace litenn_hip
 		switch (fmt)
 		{
 		case LITENN_FMT_Q4_0: launch_prepass_and_gemm<Q4_0Frag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
+		case LITENN_FMT_Q4_1: launch_prepass_and_gemm<Q4_1Frag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
+		case LITENN_FMT_Q5_0: launch_prepass_and_gemm<Q5_0Frag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
+		case LITENN_FMT_Q5_1: launch_prepass_and_gemm<Q5_1Frag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
+		case LITENN_FMT_Q2_K: launch_prepass_and_gemm<Q2_KFrag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
+		case LITENN_FMT_Q3_K: launch_prepass_and_gemm<Q3_KFrag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
 		case LITENN_FMT_Q8_0: launch_prepass_and_gemm<Q8_0Frag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
 		case LITENN_FMT_Q4_K: launch_prepass_and_gemm<Q4_KFrag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
 		case LITENN_FMT_Q5_K: launch_prepass_and_gemm<Q5_KFrag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;

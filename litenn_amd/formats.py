@@ -10,10 +10,9 @@ from __future__ import annotations
 Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, F16, F32 = 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 25, 27
 FORMAT_NAMES = {Q4_0: "Q4_0", Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", Q8_0: "Q8_0", Q2_K: "Q2_K", Q3_K: "Q3_K",
                 Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", F16: "F16", F32: "F32"}
-# every block format is decoded inside the streaming GEMV; five of them also inside the matrix-core
-# GEMM (the others take the GEMV row by row for multi-row inputs)
+# every block format is decoded inside the streaming GEMV and the matrix-core GEMM
 FAST_FORMATS = (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K)  # streaming GEMV
-GEMM_FORMATS = (Q4_0, Q8_0, Q4_K, Q5_K, Q6_K)  # also decoded inside the matrix-core GEMM
+GEMM_FORMATS = FAST_FORMATS  # and inside the matrix-core GEMM
 
 # DataType
 DT_F32, DT_F64, DT_I32, DT_I64, DT_BOOL, DT_F16, DT_BF16, DT_F8E4M3, DT_F8E5M2, DT_I8, DT_U8 = range(11)

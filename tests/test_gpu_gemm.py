@@ -10,13 +10,13 @@ import pytest
 
 from conftest import rel_l2
 from litenn_amd import synth
-from litenn_amd.formats import Q4_0, Q4_K, Q5_K, Q6_K, Q8_0, row_bytes
+from litenn_amd.formats import Q2_K, Q3_K, Q4_0, Q4_1, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0, row_bytes
 from litenn_amd.llama import MATMUL_PRECISE
 from llama_util import hip_model, oracle_model
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
-FORMATS = [Q4_0, Q8_0, Q4_K, Q5_K, Q6_K]
+FORMATS = [Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K]
 
 
 def run_case(hip, oracle, fmt, m, n, k, seed=0, residual=False, rows=None, flags=0):
