@@ -209,11 +209,15 @@ namespace
 		return 0;
 	}
 
+	// From this many rows on (and unless f32 operands are asked for) a matmul goes to the matrix cores:
+	// one padded 16-row tile costs about as much as three single-row GEMVs.
+	constexpr size_t kGemmMinRows = 4;
+
 	void matmul(litenn_hip_llama* m, const Weight& w, const float* x, size_t rows, float* y, const float* residual,
 	            unsigned flags, hipStream_t s)
 	{
 		const bool quant = w.fmt != LITENN_FMT_F16 && w.fmt != LITENN_FMT_F32;
-		if (rows >= 16 && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && w.k % 256 == 0 &&
+		if (rows >= kGemmMinRows && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && w.k % 256 == 0 &&
 		    launch_gemm(w.fmt, w.data, w.n, w.k, x, rows, y, residual, m->xh, s))
 		{
 			return;
@@ -236,7 +240,7 @@ namespace
 			same = same && ws[i]->fmt == w0.fmt && ws[i]->k == w0.k;
 		}
 		const bool quant = w0.fmt != LITENN_FMT_F16 && w0.fmt != LITENN_FMT_F32;
-		if (same && rows >= 16 && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && w0.k % 256 == 0)
+		if (same && rows >= kGemmMinRows && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && w0.k % 256 == 0)
 		{
 			const void* w[3] = { nullptr, nullptr, nullptr };
 			size_t n[3] = { 0, 0, 0 };

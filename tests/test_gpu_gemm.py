@@ -101,7 +101,7 @@ def test_prefill_through_the_matrix_cores(hip, oracle, fmt):
     of the checker's f32 pass per layer (looser after three blocks), the cache matches, and decoding
     continues from it."""
     cfg = synth.tiny_llama(fmt, block_count=3, d_model=512, heads=4, kv_heads=2, ff=1024, vocab=777)
-    toks = synth.prompt_tokens(cfg, 40, 2)
+    toks = synth.prompt_tokens(cfg, 49, 2)
     ref = oracle_model(oracle, cfg, 2, kv_f16=True)
     dev = hip_model(hip, cfg, 2)
     want = ref.eval(toks[:32])
@@ -110,5 +110,9 @@ def test_prefill_through_the_matrix_cores(hip, oracle, fmt):
     kd, vd = dev.get_kv(2)
     kr, vr = ref.get_kv(2)
     assert rel_l2(kd, kr) < 5e-3 and rel_l2(vd, vr) < 5e-3
-    for t in toks[32:]:
+    for t in toks[32:36]:
         assert rel_l2(dev.eval([t])[0], ref.eval([t])[0]) < 5e-3
+    # short multi-row passes: four rows and more take the matrix cores as well (padded tile), fewer
+    # go row by row through the GEMV
+    for lo, hi in ((36, 40), (40, 47), (47, 49)):
+        assert rel_l2(dev.eval(toks[lo:hi], precise=False), ref.eval(toks[lo:hi])) < 5e-3
