@@ -184,6 +184,15 @@ int litenn_hip_kv_append(int dev, void* cache, int cache_dtype, size_t past, con
 int litenn_hip_attn_decode(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
                            size_t past, size_t n_head, size_t n_kv_head, size_t head_dim, void* out,
                            const litenn_hip_exec* opts);
+/* The same attention for a prompt's rows: with m >= 16, an F16 cache, 128-wide heads and
+ * 16-byte aligned buffers both contractions run on the matrix cores (fp16 operands: q / sqrt(d)
+ * and the softmax weights are rounded once, f32 accumulation and softmax; relative L2 error
+ * about 3e-4), tiled so that the keys are read once per 64 rows instead of once per row.
+ * flags: LITENN_HIP_MATMUL_PRECISE keeps the f32 row kernel of litenn_hip_attn_decode, which
+ * every other shape uses as well. */
+int litenn_hip_attn_rows(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
+                         size_t past, size_t n_head, size_t n_kv_head, size_t head_dim, void* out, unsigned flags,
+                         const litenn_hip_exec* opts);
 /* y = silu(gate) * up (src/LiteNN/Layer/SwiGLU.h:59-69, Activation.h:22-63) */
 int litenn_hip_silu_mul(int dev, const void* gate, const void* up, void* y, size_t n, const litenn_hip_exec* opts);
 /* out_index[row] (I32) = first maximal index of x[row, :] (f32); ties pick the lowest index

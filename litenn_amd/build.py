@@ -11,7 +11,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "liblitenn_hip.so")
 
-SOURCES = ["api.hip", "gemv.hip", "gemm.hip", "glue.hip", "primitives.hip", "llama.hip", "gguf.hip"]
+SOURCES = ["api.hip", "gemv.hip", "gemm.hip", "glue.hip", "attn_tile.hip", "primitives.hip", "llama.hip", "gguf.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",

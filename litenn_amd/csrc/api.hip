@@ -31,6 +31,9 @@ namespace litenn_hip
 	                      hipStream_t s);
 	size_t attn_splits(size_t m, size_t max_len, size_t n_head);
 	size_t attn_partial_floats(size_t m, size_t n_head, size_t head_dim, size_t splits);
+	bool launch_attn_tile(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
+	                      const int* past_dev, size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim,
+	                      float* out, hipStream_t s);
 	void launch_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
 	                        const int* past_dev, size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim,
 	                        float* out, size_t splits, float* partial, int* counters, hipStream_t s);
@@ -802,9 +805,9 @@ extern "C" int litenn_hip_kv_append(int dev, void* cache, int cache_dtype, size_
 	return finish(action, opts);
 }
 
-extern "C" int litenn_hip_attn_decode(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype,
-                                      size_t m, size_t past, size_t n_head, size_t n_kv_head, size_t head_dim,
-                                      void* out, const litenn_hip_exec* opts)
+static int attn_rows_impl(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
+                          size_t past, size_t n_head, size_t n_kv_head, size_t head_dim, void* out, bool matrix_cores,
+                          const litenn_hip_exec* opts)
 {
 	const char* action = "HIP attention";
 	if (cache_dtype != LITENN_F16 && cache_dtype != LITENN_F32)
@@ -832,6 +835,12 @@ extern "C" int litenn_hip_attn_decode(int dev, const void* q, const void* kcache
 		return fail(action, "too many query rows or heads");
 	}
 	GUARD(action, dev);
+	if (matrix_cores && m >= 16 &&
+	    launch_attn_tile(static_cast<const float*>(q), kcache, vcache, cache_dtype, m, nullptr, past, n_head, n_kv_head,
+	                     head_dim, static_cast<float*>(out), stream_of(opts)))
+	{
+		return finish(action, opts);
+	}
 	// a single row against a long cache is cut into chunks that meet in scratch memory, which
 	// this call owns: it is freed after the stream has drained, whatever opts->synchronize says
 	const size_t splits = attn_splits(m, past + m, n_head);
@@ -863,6 +872,21 @@ extern "C" int litenn_hip_attn_decode(int dev, const void* q, const void* kcache
 		return 0;
 	}
 	return finish(action, opts);
+}
+
+extern "C" int litenn_hip_attn_decode(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype,
+                                      size_t m, size_t past, size_t n_head, size_t n_kv_head, size_t head_dim,
+                                      void* out, const litenn_hip_exec* opts)
+{
+	return attn_rows_impl(dev, q, kcache, vcache, cache_dtype, m, past, n_head, n_kv_head, head_dim, out, false, opts);
+}
+
+extern "C" int litenn_hip_attn_rows(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype,
+                                    size_t m, size_t past, size_t n_head, size_t n_kv_head, size_t head_dim, void* out,
+                                    unsigned flags, const litenn_hip_exec* opts)
+{
+	return attn_rows_impl(dev, q, kcache, vcache, cache_dtype, m, past, n_head, n_kv_head, head_dim, out,
+	                      !(flags & LITENN_HIP_MATMUL_PRECISE), opts);
 }
 
 extern "C" int litenn_hip_silu_mul(int dev, const void* gate, const void* up, void* y, size_t n,

@@ -42,6 +42,9 @@ namespace litenn_hip
 	                      int* counters, hipStream_t s);
 	size_t attn_splits(size_t m, size_t max_len, size_t n_head);
 	size_t attn_partial_floats(size_t m, size_t n_head, size_t head_dim, size_t splits);
+	bool launch_attn_tile(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
+	                      const int* past_dev, size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim,
+	                      float* out, hipStream_t s);
 	void launch_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
 	                        const int* past_dev, size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim,
 	                        float* out, size_t splits, float* partial, int* counters, hipStream_t s);
@@ -212,6 +215,8 @@ namespace
 	// From this many rows on (and unless f32 operands are asked for) a matmul goes to the matrix cores:
 	// one padded 16-row tile costs about as much as three single-row GEMVs.
 	constexpr size_t kGemmMinRows = 4;
+	// From this many rows on the prompt's attention runs tiled on the matrix cores.
+	constexpr size_t kAttnTileMinRows = 16;
 
 	void matmul(litenn_hip_llama* m, const Weight& w, const float* x, size_t rows, float* y, const float* residual,
 	            unsigned flags, hipStream_t s)
@@ -376,8 +381,13 @@ namespace
 			matmul_group(m, 3, qkv, qkv_out, m->x, rows, nullptr, L.attn_norm, nullptr, m->xn, flags, s);
 			launch_rope_qkv_append(m->q, m->k, m->v, L.kcache, L.vcache, m->p.kv_dtype, past_dev, rows, H, KH, hd,
 			                       m->p.rope_dimension_count, m->cos_t, m->sin_t, s);
-			launch_attn_decode(m->q, L.kcache, L.vcache, m->p.kv_dtype, rows, past_dev, 0, H, KH, hd, m->attn,
-			                   rows == 1 ? m->attn_splits : 1, m->attn_partial, m->attn_counters, s);
+			// a prompt's rows go through the matrix cores (fp16 operands) unless f32 operands are asked for
+			if (rows < kAttnTileMinRows || (flags & LITENN_HIP_MATMUL_PRECISE) ||
+			    !launch_attn_tile(m->q, L.kcache, L.vcache, m->p.kv_dtype, rows, past_dev, 0, H, KH, hd, m->attn, s))
+			{
+				launch_attn_decode(m->q, L.kcache, L.vcache, m->p.kv_dtype, rows, past_dev, 0, H, KH, hd, m->attn,
+				                   rows == 1 ? m->attn_splits : 1, m->attn_partial, m->attn_counters, s);
+			}
 			matmul(m, L.wo, m->attn, rows, m->x, m->x, flags, s); // x = x + attn . Wo
 			const Weight* gu[2] = { &L.gate, &L.up };
 			float* gu_out[2] = { m->gate, m->up };

@@ -263,6 +263,16 @@ def attn_decode(q: Tensor, kcache: Tensor, vcache: Tensor, m: int, past: int, n_
     return out
 
 
+def attn_rows(q: Tensor, kcache: Tensor, vcache: Tensor, m: int, past: int, n_head: int, n_kv_head: int,
+              head_dim: int, precise: bool = False) -> Tensor:
+    """attn_decode for a prompt's rows: on the matrix cores when the shape allows and precise is False."""
+    out = Tensor((m, n_head * head_dim), DT_F32, q.device)
+    check(_lib.load().litenn_hip_attn_rows(q.device.deviceIndex, q.ptr, kcache.ptr, vcache.ptr, kcache.dtype, m, past,
+                                           n_head, n_kv_head, head_dim, out.ptr, MATMUL_PRECISE if precise else 0,
+                                           None))
+    return out
+
+
 def silu_mul(gate: Tensor, up: Tensor) -> Tensor:
     y = Tensor(gate.shape, DT_F32, gate.device)
     check(_lib.load().litenn_hip_silu_mul(gate.device.deviceIndex, gate.ptr, up.ptr, y.ptr, gate.size, None))

@@ -96,6 +96,50 @@ def test_attention_decode(hip, oracle, cache_dtype):
         assert rel_l2(got, want) < 1e-5, (m, past, H, KH, hd)
 
 
+def _attention_want(oracle, q, k, v, past, H, KH, hd):
+    want = np.empty_like(q)
+    for h in range(H):
+        kvh = h // (H // KH)
+        want[:, h * hd:(h + 1) * hd] = oracle.attention_head(
+            q[:, h * hd:(h + 1) * hd].copy(), k[:, kvh * hd:(kvh + 1) * hd].copy(),
+            v[:, kvh * hd:(kvh + 1) * hd].copy(), 1.0 / math.sqrt(hd), True, 0, past)
+    return want
+
+
+def test_attention_of_a_prompt_on_the_matrix_cores(hip, oracle):
+    """litenn_hip_attn_rows: fp16 operands, f32 softmax and accumulation; tolerance 1e-3 relative L2
+    (fp16 rounding of q / sqrt(d) and of the softmax weights).  Ragged row and key counts, a filled
+    cache before the rows (past > 0), grouped KV heads, outliers in q."""
+    rng = np.random.default_rng(14)
+    for m, past, H, KH in [(16, 0, 4, 4), (64, 0, 8, 2), (65, 0, 4, 1), (100, 37, 4, 2), (128, 0, 32, 32),
+                           (512, 0, 32, 8), (200, 1000, 8, 8), (17, 63, 2, 2), (48, 64, 2, 1)]:
+        hd = 128
+        L = past + m
+        q = rng.standard_normal((m, H * hd)).astype(np.float32)
+        q[rng.integers(0, m, 4), rng.integers(0, H * hd, 4)] *= 30.0
+        k = oracle.f16_to_f32(oracle.f32_to_f16_bits(rng.standard_normal((L, KH * hd)).astype(np.float32)))
+        v = oracle.f16_to_f32(oracle.f32_to_f16_bits(rng.standard_normal((L, KH * hd)).astype(np.float32)))
+        kc, vc = T(hip, k, np.float16), T(hip, v, np.float16)
+        want = _attention_want(oracle, q, k, v, past, H, KH, hd)
+        got = hip.attn_rows(T(hip, q), kc, vc, m, past, H, KH, hd).numpy()
+        assert rel_l2(got, want) < 1e-3, (m, past, H, KH, rel_l2(got, want))
+        # every row on its own as well: no row may hide behind the others
+        row_err = np.linalg.norm(got - want, axis=1) / np.linalg.norm(want, axis=1)
+        assert row_err.max() < 3e-3, (m, past, H, KH, int(row_err.argmax()), float(row_err.max()))
+        # the precise flag and every other shape keep the f32 row kernel
+        exact = hip.attn_rows(T(hip, q), kc, vc, m, past, H, KH, hd, precise=True).numpy()
+        assert rel_l2(exact, want) < 1e-5
+    # shapes the tiled kernel does not take: f32 cache, other head widths, fewer than 16 rows
+    for m, past, H, KH, hd, f16 in [(40, 3, 4, 2, 128, False), (32, 0, 4, 4, 64, True), (8, 20, 4, 4, 128, True)]:
+        L = past + m
+        q = rng.standard_normal((m, H * hd)).astype(np.float32)
+        k = oracle.f16_to_f32(oracle.f32_to_f16_bits(rng.standard_normal((L, KH * hd)).astype(np.float32)))
+        v = oracle.f16_to_f32(oracle.f32_to_f16_bits(rng.standard_normal((L, KH * hd)).astype(np.float32)))
+        kc, vc = (T(hip, k, np.float16), T(hip, v, np.float16)) if f16 else (T(hip, k), T(hip, v))
+        got = hip.attn_rows(T(hip, q), kc, vc, m, past, H, KH, hd).numpy()
+        assert rel_l2(got, _attention_want(oracle, q, k, v, past, H, KH, hd)) < 1e-5
+
+
 def test_attention_reference_vectors(hip, golden):
     c0, c1 = golden["attention"]
     # causal 3x3, head_dim 2 (scale 1/sqrt(2) is the kernel's own 1/sqrt(head_dim))
