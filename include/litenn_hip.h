@@ -184,8 +184,10 @@ int litenn_hip_kv_append(int dev, void* cache, int cache_dtype, size_t past, con
 int litenn_hip_attn_decode(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
                            size_t past, size_t n_head, size_t n_kv_head, size_t head_dim, void* out,
                            const litenn_hip_exec* opts);
-/* The same attention for a prompt's rows: with m >= 16, an F16 cache, 128-wide heads and
- * 16-byte aligned buffers both contractions run on the matrix cores (fp16 operands: q / sqrt(d)
+/* The same attention for a prompt's rows (the multi-row lowering of
+ * tools/gguf/LLaMABuilder.cpp:350-404,502-557; mask of src/LiteNN/Layer/CausalMask.h:16-56):
+ * with m >= 16, an F16 cache, 128-wide heads and 16-byte aligned buffers both contractions
+ * run on the matrix cores (fp16 operands: q / sqrt(d)
  * and the softmax weights are rounded once, f32 accumulation and softmax; relative L2 error
  * about 3e-4), tiled so that the keys are read once per 64 rows instead of once per row.
  * flags: LITENN_HIP_MATMUL_PRECISE keeps the f32 row kernel of litenn_hip_attn_decode, which
