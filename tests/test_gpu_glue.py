@@ -140,6 +140,36 @@ def test_attention_of_a_prompt_on_the_matrix_cores(hip, oracle):
         assert rel_l2(got, _attention_want(oracle, q, k, v, past, H, KH, hd)) < 1e-5
 
 
+def test_prompt_attention_closed_forms_at_full_size(hip):
+    """Properties that need no checker, at the prompt sizes of the 7B and 8B configurations:
+    a zero query weighs all visible keys equally, so row r returns the mean of the first
+    past + r + 1 value rows; one key that dominates the scores returns that key's value row."""
+    rng = np.random.default_rng(15)
+    hd = 128
+    for m, past, H, KH in [(128, 0, 32, 32), (512, 0, 32, 8), (512, 512, 32, 8)]:
+        L = past + m
+        k = rng.standard_normal((L, KH * hd)).astype(np.float16)
+        v = rng.standard_normal((L, KH * hd)).astype(np.float16)
+        kc, vc = T(hip, k, np.float16), T(hip, v, np.float16)
+        got = hip.attn_rows(T(hip, np.zeros((m, H * hd), np.float32)), kc, vc, m, past, H, KH, hd).numpy()
+        prefix_mean = np.cumsum(v.astype(np.float64), axis=0)[past:] / np.arange(past + 1, L + 1)[:, None]
+        want = np.concatenate([prefix_mean[:, (h // (H // KH)) * hd:(h // (H // KH) + 1) * hd] for h in range(H)],
+                              axis=1)
+        # the weights 1/n are rounded to fp16 before the second product: 2^-11 relative at most
+        assert np.max(np.abs(got - want)) < 2e-3 * np.max(np.abs(want)) + 1e-4, (m, past)
+        # key 5 carries a huge component along dimension 0 and every query points at it
+        k2 = k.copy()
+        k2[5, :] = 0
+        k2[5, 0::hd] = 300.0
+        q = np.zeros((m, H * hd), np.float32)
+        q[:, 0::hd] = 10.0
+        got = hip.attn_rows(T(hip, q), T(hip, k2, np.float16), vc, m, past, H, KH, hd).numpy()
+        first = 0 if past >= 5 else 5 - past  # rows that can see key 5
+        want = np.concatenate([np.broadcast_to(v[5, (h // (H // KH)) * hd:(h // (H // KH) + 1) * hd], (m, hd))
+                               for h in range(H)], axis=1).astype(np.float32)
+        assert np.max(np.abs(got[first:] - want[first:])) < 1e-3
+
+
 def test_attention_reference_vectors(hip, golden):
     c0, c1 = golden["attention"]
     # causal 3x3, head_dim 2 (scale 1/sqrt(2) is the kernel's own 1/sqrt(head_dim))
