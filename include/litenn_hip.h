@@ -132,7 +132,10 @@ int litenn_hip_permute(int dev, void* dst, int dtype, const size_t* src_shape, s
  * 4e-4.  LITENN_HIP_MATMUL_PRECISE in `flags` keeps f32 operands (GEMV path) for any m.
  * The matrix-core path needs a device workspace of litenn_hip_mul_mat_q_workspace_bytes(m, k):
  * litenn_hip_mul_mat_q allocates and frees it itself (and therefore always synchronises for
- * m >= 16); litenn_hip_mul_mat_q_ws takes the caller's (16-byte aligned; NULL = as above). */
+ * m >= 16); litenn_hip_mul_mat_q_ws takes the caller's (16-byte aligned; NULL = as above).
+ * A workspace at least 4*m*n bytes larger than that (rounded up to 16) also lets a product with
+ * k >= 8192 whose 128 x 128 tiles would fill only half the card walk K in two halves at once;
+ * the halves are added in a fixed order, so results do not depend on scheduling. */
 #define LITENN_HIP_MATMUL_PRECISE 1u
 int litenn_hip_mul_mat_q(int dev, int fmt, const void* wq, size_t n, size_t k, const void* x, int x_dtype, size_t m,
                          void* y, const void* residual, unsigned flags, const litenn_hip_exec* opts);

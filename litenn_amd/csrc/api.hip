@@ -15,7 +15,7 @@ namespace litenn_hip
 	                const float* residual, hipStream_t stream);
 	size_t gemm_scratch_halves(size_t m, size_t k);
 	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
-	                 const float* residual, void* scratch_halves, hipStream_t stream);
+	                 const float* residual, void* scratch_halves, float* partial, hipStream_t stream);
 	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
 	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
 	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream);
@@ -553,13 +553,18 @@ extern "C" int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t 
 	{
 		// the matrix-core path rounds the activations to fp16 into a workspace
 		const size_t need = 2 * gemm_scratch_halves(m, k);
+		// room for a second m x n product behind it lets a long K be cut in two
+		const size_t need16 = (need + 15) & ~size_t{ 15 };
+		const size_t with_partial = need16 + sizeof(float) * m * n;
 		if (workspace)
 		{
 			if (workspace_bytes < need)
 			{
 				return fail(action, "workspace is smaller than litenn_hip_mul_mat_q_workspace_bytes(m, k)");
 			}
-			if (!launch_gemm(fmt, wq, n, k, xf, m, yf, rf, workspace, s))
+			float* partial =
+			    workspace_bytes >= with_partial ? reinterpret_cast<float*>(static_cast<char*>(workspace) + need16) : nullptr;
+			if (!launch_gemm(fmt, wq, n, k, xf, m, yf, rf, workspace, partial, s))
 			{
 				launch_gemv(fmt, wq, n, k, xf, m, yf, rf, s);
 			}
@@ -568,8 +573,10 @@ extern "C" int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t 
 		// none given: this call owns one, and frees it after the stream has drained, whatever
 		// opts->synchronize says
 		void* scratch = nullptr;
-		LITENN_HIP_TRY(action, hipMalloc(&scratch, need));
-		if (!launch_gemm(fmt, wq, n, k, xf, m, yf, rf, scratch, s))
+		const bool long_k = k >= 8192 && m >= 128;
+		LITENN_HIP_TRY(action, hipMalloc(&scratch, long_k ? with_partial : need));
+		float* partial = long_k ? reinterpret_cast<float*>(static_cast<char*>(scratch) + need16) : nullptr;
+		if (!launch_gemm(fmt, wq, n, k, xf, m, yf, rf, scratch, partial, s))
 		{
 			launch_gemv(fmt, wq, n, k, xf, m, yf, rf, s);
 		}

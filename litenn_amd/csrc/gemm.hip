@@ -660,6 +660,7 @@ namespace litenn_hip
 			__shared__ float red[4];
 			__shared__ double red64[4];
 			const int row = blockIdx.x;
+
 			const int chunks = k / kChunk;
 			const int mt = row >> 4, r = row & 15;
 			uint8_t* tile_row = xf + static_cast<size_t>(mt) * chunks * kChunkTileBytes + r * 16;
@@ -853,6 +854,7 @@ namespace litenn_hip
 			float* y[3];
 			int n[3];
 			int first_block[3]; // grid x index of each matrix's first row block (INT_MAX when unused)
+			float* partial;     // [M, n[0]]: product of the second K range when grid z = 2 (single matrix)
 		};
 
 		template <typename F, int MT, int NG, int WAVES>
@@ -881,6 +883,9 @@ namespace litenn_hip
 			const int n_base = (block_x * WAVES + wave) * 16 * NG;
 			const int mt_base = blockIdx.y * MT;
 			const int chunks = k / kChunk;
+			// grid z splits the K walk: this workgroup multiplies chunks [c_begin, c_end)
+			const int c_begin = static_cast<int>(blockIdx.z) * chunks / static_cast<int>(gridDim.z);
+			const int c_end = (static_cast<int>(blockIdx.z) + 1) * chunks / static_cast<int>(gridDim.z);
 			const uint32_t lds_base =
 			    static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const uint8_t*)(lds)));
 			const uint32_t slot_lds = lds_base + 3 * kHalfBytes + wave * kSlotBytes;
@@ -1104,12 +1109,12 @@ namespace litenn_hip
 				}
 			};
 
-			issue_w(0);
-			issue_x(0, 0);
-			issue_x(1, kHalfBytes);
+			issue_w(c_begin);
+			issue_x(2 * c_begin, 0);
+			issue_x(2 * c_begin + 1, kHalfBytes);
 			vm_wait<0>();
 			__syncthreads();
-			load_raw(0);
+			load_raw(c_begin);
 #pragma unroll
 			for (int t = 0; t < MT; ++t)
 			{
@@ -1118,8 +1123,8 @@ namespace litenn_hip
 			decode(a_cur, 0);
 			using std::false_type;
 			using std::true_type;
-			int c = 0;
-			for (; c + 1 < chunks; ++c)
+			int c = c_begin;
+			for (; c + 1 < c_end; ++c)
 			{
 				chunk(true_type{}, c);
 			}
@@ -1138,8 +1143,10 @@ namespace litenn_hip
 					const int mm = (mt_base + t) * 16 + r;
 					if (mm < m)
 					{
-						float* dst = y + static_cast<size_t>(mm) * n + n0;
-						const float* res = residual ? residual + static_cast<size_t>(mm) * n + n0 : nullptr;
+						// the second K range of a split walk leaves its product beside y (no residual)
+						float* dst = (blockIdx.z == 0 ? y : mats.partial) + static_cast<size_t>(mm) * n + n0;
+						const float* res =
+						    residual && blockIdx.z == 0 ? residual + static_cast<size_t>(mm) * n + n0 : nullptr;
 						const float us = unscale[mm];
 						const float vals[4] = { acc[q][t].x * us, acc[q][t].y * us, acc[q][t].z * us, acc[q][t].w * us };
 						if (vec_ok && n0 + 3 < n)
@@ -1181,6 +1188,9 @@ namespace litenn_hip
 			const float* residual;
 			int k, m, m_tiles;
 			size_t row_bytes;
+			int tile;       // MT * 100 + NG * 10 + WAVES
+			int k_splits;   // 1, or 2: two workgroups share a tile's K walk, the second writes `partial`
+			float* partial; // [M, n[0]] floats, or null: K is never split
 			hipStream_t stream;
 		};
 
@@ -1195,6 +1205,7 @@ namespace litenn_hip
 			(void)attr;
 			constexpr int bn = 16 * WAVES * NG;
 			GemmMats mats;
+			mats.partial = c.partial;
 			int blocks = 0;
 			for (int i = 0; i < 3; ++i)
 			{
@@ -1204,7 +1215,7 @@ namespace litenn_hip
 				mats.first_block[i] = i < c.count ? blocks : 0x7fffffff;
 				blocks += i < c.count ? (c.n[i] + bn - 1) / bn : 0;
 			}
-			const dim3 grid(blocks, (c.m_tiles + MT - 1) / MT);
+			const dim3 grid(blocks, (c.m_tiles + MT - 1) / MT, c.k_splits);
 			gemm_q_kernel<F, MT, NG, WAVES><<<grid, dim3(64 * WAVES), lds, c.stream>>>(mats, c.xf, c.unscale, c.residual,
 			                                                                          c.k, c.m, c.m_tiles, c.row_bytes);
 		}
@@ -1212,8 +1223,33 @@ namespace litenn_hip
 		// Tile choice: MT activation tiles per workgroup so that a weight is decoded as few times as
 		// possible; two weight groups per wavefront (each activation fragment read from LDS feeds two
 		// MFMAs) when that still nearly fills the card.
+		// y += partial, element by element: the fixed order (first K range, then second) keeps the
+		// result independent of scheduling
+		__global__ __launch_bounds__(256) void add_partial_kernel(float* __restrict__ y, const float* __restrict__ partial,
+		                                                           size_t total)
+		{
+			const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+			if (i + 3 < total && (reinterpret_cast<uintptr_t>(y) & 15) == 0 && (reinterpret_cast<uintptr_t>(partial) & 15) == 0)
+			{
+				float4 a = *reinterpret_cast<float4*>(y + i);
+				const float4 b = *reinterpret_cast<const float4*>(partial + i);
+				a.x += b.x, a.y += b.y, a.z += b.z, a.w += b.w;
+				*reinterpret_cast<float4*>(y + i) = a;
+			}
+			else
+			{
+				for (size_t e = i; e < total && e < i + 4; ++e)
+				{
+					y[e] += partial[e];
+				}
+			}
+		}
+
+		// K from which splitting pays: the extra pass over y costs about 7 us
+		constexpr int kSplitMinK = 8192;
+
 		template <typename F>
-		void launch_format(const GemmCall& c, int cus)
+		void choose_tile(GemmCall& c, int cus)
 		{
 			const auto blocks = [&](int mt, int bn) {
 				long nb = 0;
@@ -1224,21 +1260,17 @@ namespace litenn_hip
 				return nb * ((c.m_tiles + mt - 1) / mt);
 			};
 			static const int forced = env_int("LITENN_HIP_GEMM_TILE", 0); // MT * 100 + NG * 10 + WAVES
-#define LITENN_GEMM_CASE(MT_, NG_, WV_)                                                                              \
-	if constexpr (gemm_lds_bytes<F, MT_, NG_, WV_>() <= kLdsLimit && (NG_ == 1 || F::kWideTile))                   \
-	{                                                                                                              \
-		if (pick == MT_ * 100 + NG_ * 10 + WV_)                                                                    \
-		{                                                                                                          \
-			launch_variant<F, MT_, NG_, WV_>(c);                                                                   \
-			return;                                                                                                \
-		}                                                                                                          \
-	}
+			static const int split_ok = env_int("LITENN_HIP_GEMM_SPLITK", 1);
 			int pick = forced;
+			c.k_splits = 1;
 			if (pick == 0)
 			{
 				// measured on the MI355X (K = 4096, N = 4096 and 14336, M = 16 .. 512): the widest tile
 				// wins once it nearly fills the card, otherwise the tallest single-group tile that
-				// still gives (nearly) every CU a workgroup
+				// still gives (nearly) every CU a workgroup.  A single matrix with a long K whose
+				// 128 x 128 tiles fill only half the card (N = 4096 at M = 512) keeps that tile and
+				// cuts K in two when the caller lends a buffer for the second product: each weight is
+				// then decoded four times instead of eight, and one pass adds the two products.
 				const int m_tiles = c.m_tiles;
 				if (m_tiles >= 8 && F::kWideTile && 5 * blocks(8, 256) >= 4 * cus)
 				{
@@ -1247,6 +1279,12 @@ namespace litenn_hip
 				else if (m_tiles >= 8 && 5 * blocks(8, 128) >= 4 * cus)
 				{
 					pick = 818;
+				}
+				else if (split_ok && c.partial && m_tiles >= 8 && c.count == 1 && c.k >= kSplitMinK &&
+				         10 * blocks(8, 128) >= 4 * cus)
+				{
+					pick = 818;
+					c.k_splits = 2;
 				}
 				else if (m_tiles >= 4 && 5 * blocks(4, 64) >= 4 * cus)
 				{
@@ -1261,6 +1299,22 @@ namespace litenn_hip
 					pick = 114;
 				}
 			}
+			c.tile = pick;
+		}
+
+		template <typename F>
+		void launch_format(const GemmCall& c)
+		{
+#define LITENN_GEMM_CASE(MT_, NG_, WV_)                                                                              \
+	if constexpr (gemm_lds_bytes<F, MT_, NG_, WV_>() <= kLdsLimit && (NG_ == 1 || F::kWideTile))                   \
+	{                                                                                                              \
+		if (pick == MT_ * 100 + NG_ * 10 + WV_)                                                                    \
+		{                                                                                                          \
+			launch_variant<F, MT_, NG_, WV_>(c);                                                                   \
+			return;                                                                                                \
+		}                                                                                                          \
+	}
+			const int pick = c.tile;
 			LITENN_GEMM_CASE(8, 2, 8)
 			LITENN_GEMM_CASE(8, 1, 8)
 			LITENN_GEMM_CASE(4, 1, 4)
@@ -1271,12 +1325,19 @@ namespace litenn_hip
 		}
 
 		template <typename F>
-		void launch_prepass_and_gemm(const GemmCall& c, const float* x, const float* norm_w, double eps, const float* up,
+		void launch_prepass_and_gemm(GemmCall& c, const float* x, const float* norm_w, double eps, const float* up,
 		                             uint8_t* xf, float* unscale, int m_pad, int cus)
 		{
+			choose_tile<F>(c, cus);
 			to_half_kernel<F><<<dim3(static_cast<unsigned>(m_pad)), dim3(256), 0, c.stream>>>(x, xf, unscale, c.m, c.k,
 			                                                                                 norm_w, eps, up);
-			launch_format<F>(c, cus);
+			launch_format<F>(c);
+			if (c.k_splits > 1)
+			{
+				const size_t total = static_cast<size_t>(c.m) * c.n[0];
+				add_partial_kernel<<<dim3(static_cast<unsigned>((total / 4 + 255) / 256 + 1)), dim3(256), 0, c.stream>>>(
+				    c.y[0], c.partial, total);
+			}
 		}
 	} // namespace
 
@@ -1294,9 +1355,10 @@ namespace litenn_hip
 	// not one this kernel takes (the caller then composes the operators and uses the GEMV): K must be
 	// a whole number of 256-element chunks and at most 16384 (a thread of the pre-pass holds its share
 	// of a row in registers), and the rows 16-byte aligned (2-byte for Q6_K).
+	// partial: null, or M x n[0] floats the launch may use to cut a long K in two (single matrix).
 	bool launch_gemm_group(int fmt, int count, const void* const* wq, const size_t* n, size_t k, const float* x,
 	                       size_t m, float* const* y, const float* residual, const float* norm_w, double eps,
-	                       const float* up, void* scratch_halves, hipStream_t stream)
+	                       const float* up, void* scratch_halves, float* partial, hipStream_t stream)
 	{
 		const size_t rb = row_bytes(fmt, k);
 		switch (fmt)
@@ -1356,6 +1418,7 @@ namespace litenn_hip
 		c.m = static_cast<int>(m);
 		c.m_tiles = static_cast<int>(m_pad / 16);
 		c.row_bytes = rb;
+		c.partial = partial;
 		c.stream = stream;
 		const int mp = static_cast<int>(m_pad);
 		switch (fmt)
@@ -1375,10 +1438,11 @@ namespace litenn_hip
 	}
 
 	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
-	                 const float* residual, void* scratch_halves, hipStream_t stream)
+	                 const float* residual, void* scratch_halves, float* partial, hipStream_t stream)
 	{
 		const void* w[1] = { wq };
 		float* ys[1] = { y };
-		return launch_gemm_group(fmt, 1, w, &n, k, x, m, ys, residual, nullptr, 0.0, nullptr, scratch_halves, stream);
+		return launch_gemm_group(fmt, 1, w, &n, k, x, m, ys, residual, nullptr, 0.0, nullptr, scratch_halves, partial,
+		                         stream);
 	}
 } // namespace litenn_hip

@@ -22,9 +22,9 @@ namespace litenn_hip
 	size_t gemm_scratch_halves(size_t m, size_t k);
 	bool launch_gemm_group(int fmt, int count, const void* const* wq, const size_t* n, size_t k, const float* x,
 	                       size_t m, float* const* y, const float* residual, const float* norm_w, double eps,
-	                       const float* up, void* scratch_halves, hipStream_t stream);
+	                       const float* up, void* scratch_halves, float* partial, hipStream_t stream);
 	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
-	                 const float* residual, void* scratch_halves, hipStream_t stream);
+	                 const float* residual, void* scratch_halves, float* partial, hipStream_t stream);
 	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
 	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
 	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream);
@@ -223,7 +223,7 @@ namespace
 	{
 		const bool quant = w.fmt != LITENN_FMT_F16 && w.fmt != LITENN_FMT_F32;
 		if (rows >= kGemmMinRows && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && w.k % 256 == 0 &&
-		    launch_gemm(w.fmt, w.data, w.n, w.k, x, rows, y, residual, m->xh, s))
+		    launch_gemm(w.fmt, w.data, w.n, w.k, x, rows, y, residual, m->xh, nullptr, s))
 		{
 			return;
 		}
@@ -236,7 +236,7 @@ namespace
 	// the producer's result).
 	void matmul_group(litenn_hip_llama* m, int count, const Weight* const* ws, float* const* ys, const float* x,
 	                  size_t rows, const float* residual, const float* norm_w, const float* up, float* tmp,
-	                  unsigned flags, hipStream_t s)
+	                  float* partial, unsigned flags, hipStream_t s)
 	{
 		const Weight& w0 = *ws[0];
 		bool same = true;
@@ -255,7 +255,7 @@ namespace
 				n[i] = ws[i]->n;
 			}
 			if (launch_gemm_group(w0.fmt, count, w, n, w0.k, x, rows, ys, residual, norm_w, m->p.rms_norm_epsilon, up,
-			                      m->xh, s))
+			                      m->xh, partial, s))
 			{
 				return;
 			}
@@ -378,7 +378,7 @@ namespace
 		{
 			const Weight* qkv[3] = { &L.wq, &L.wk, &L.wv };
 			float* qkv_out[3] = { m->q, m->k, m->v };
-			matmul_group(m, 3, qkv, qkv_out, m->x, rows, nullptr, L.attn_norm, nullptr, m->xn, flags, s);
+			matmul_group(m, 3, qkv, qkv_out, m->x, rows, nullptr, L.attn_norm, nullptr, m->xn, nullptr, flags, s);
 			launch_rope_qkv_append(m->q, m->k, m->v, L.kcache, L.vcache, m->p.kv_dtype, past_dev, rows, H, KH, hd,
 			                       m->p.rope_dimension_count, m->cos_t, m->sin_t, s);
 			// a prompt's rows go through the matrix cores (fp16 operands) unless f32 operands are asked for
@@ -391,10 +391,11 @@ namespace
 			matmul(m, L.wo, m->attn, rows, m->x, m->x, flags, s); // x = x + attn . Wo
 			const Weight* gu[2] = { &L.gate, &L.up };
 			float* gu_out[2] = { m->gate, m->up };
-			matmul_group(m, 2, gu, gu_out, m->x, rows, nullptr, L.ffn_norm, nullptr, m->xn, flags, s);
+			matmul_group(m, 2, gu, gu_out, m->x, rows, nullptr, L.ffn_norm, nullptr, m->xn, nullptr, flags, s);
 			const Weight* wd[1] = { &L.down };
 			float* xo[1] = { m->x };
-			matmul_group(m, 1, wd, xo, m->gate, rows, m->x, nullptr, m->up, m->gate2, flags, s); // x = x + mlp
+			// xn is idle here: the GEMM may leave the product of K's second half there
+			matmul_group(m, 1, wd, xo, m->gate, rows, m->x, nullptr, m->up, m->gate2, m->xn, flags, s); // x = x + mlp
 		}
 		const size_t first = rows - logit_rows;
 		launch_rmsnorm(m->x + first * d, m->output_norm, m->p.rms_norm_epsilon, logit_rows, d, m->xn, s);

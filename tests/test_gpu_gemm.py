@@ -85,6 +85,46 @@ def test_gemm_every_tile_shape(hip, oracle, fmt, m, n, k):
     assert run_case(hip, oracle, fmt, m, n, k, seed=n % 97, rows=rows, residual=(k == 512)) <= TOL
 
 
+@pytest.mark.parametrize("fmt,k", [(Q4_0, 11008), (Q6_K, 14336), (Q4_K, 8192)])
+@pytest.mark.parametrize("m", [512, 400])
+def test_long_k_is_walked_in_two_halves(hip, oracle, fmt, k, m):
+    """The down projections of the benchmark shapes (N = 4096, K = 11008 / 14336) at prompt sizes:
+    with room for a second product in the workspace two workgroups per tile share the K walk.
+    Checked against the CPU checker on a sample of weight rows (with a residual), and against the
+    same product computed without the split (same operands, other summation order)."""
+    import ctypes as C
+    from litenn_amd._lib import Exec, check, load
+    n = 4096
+    wq = synth.quant_weights(fmt, n, k, k % 89, 1)
+    x = synth.activations(m, k, 5, 2)
+    res = synth.activations(m, n, 6, 3)
+    lib = load()
+    w_t, x_t, r_t = hip.Tensor.from_numpy(wq), hip.Tensor.from_numpy(x), hip.Tensor.from_numpy(res)
+    base = lib.litenn_hip_mul_mat_q_workspace_bytes(m, k)
+    roomy = (base + 15) // 16 * 16 + 4 * m * n
+    ws = hip.Tensor(((roomy + 3) // 4,))
+    opts = Exec(None, 1)
+    outs = []
+    for ws_bytes in (base, roomy):
+        y = hip.Tensor((m, n))
+        check(lib.litenn_hip_mul_mat_q_ws(0, fmt, w_t.ptr, n, k, x_t.ptr, 0, m, y.ptr, r_t.ptr, 0, ws.ptr, ws_bytes,
+                                          C.byref(opts)))
+        outs.append(y.numpy())
+    plain, split = outs
+    assert rel_l2(split - res, plain - res) < 1e-5
+    assert not np.array_equal(split, plain)  # the split path ran
+    # in place (residual aliases y), the way the decoder calls it
+    y = hip.Tensor.from_numpy(res)
+    check(lib.litenn_hip_mul_mat_q_ws(0, fmt, w_t.ptr, n, k, x_t.ptr, 0, m, y.ptr, y.ptr, 0, ws.ptr, roomy,
+                                      C.byref(opts)))
+    assert np.array_equal(y.numpy(), split)
+    rows = np.sort(np.random.default_rng(k).choice(n, 256, replace=False))
+    rows[0], rows[-1] = 0, n - 1
+    sub = np.ascontiguousarray(wq.reshape(n, row_bytes(fmt, k))[rows]).reshape(-1)
+    ref = oracle.mul_mat_q(fmt, sub, len(rows), k, x)
+    assert rel_l2(split[:, rows] - res[:, rows], ref) <= TOL
+
+
 def test_gemm_is_linear_in_x_at_full_size(hip):
     """Size-independent property at the full north-star shape: Y(a x1 + x2) = a Y(x1) + Y(x2) up to
     the fp16 rounding of the activations."""
