@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes one launch of the headline GEMV moves, from the profiler's FETCH_SIZE / WRITE_SIZE
 # counters scaled by a known-size copy (profiles/gemv_q4_k_14336x4096_hbm_traffic.txt); it is a
 # property of the kernel and the shape, not re-measured by this script.
-GEMV_Q4_K_14336x4096_TRAFFIC_BYTES = 33321300
+GEMV_Q4_K_14336x4096_TRAFFIC_BYTES = 33321350
 
 
 def log(*a):
