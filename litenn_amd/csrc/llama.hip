@@ -378,7 +378,18 @@ namespace
 		{
 			const Weight* qkv[3] = { &L.wq, &L.wk, &L.wv };
 			float* qkv_out[3] = { m->q, m->k, m->v };
-			matmul_group(m, 3, qkv, qkv_out, m->x, rows, nullptr, L.attn_norm, nullptr, m->xn, nullptr, flags, s);
+			// consecutive projections of one format share a launch (and its fused norm)
+			for (int i = 0; i < 3;)
+			{
+				int j = i + 1;
+				while (j < 3 && qkv[j]->fmt == qkv[i]->fmt && qkv[j]->k == qkv[i]->k)
+				{
+					++j;
+				}
+				matmul_group(m, j - i, qkv + i, qkv_out + i, m->x, rows, nullptr, L.attn_norm, nullptr, m->xn, nullptr,
+				             flags, s);
+				i = j;
+			}
 			launch_rope_qkv_append(m->q, m->k, m->v, L.kcache, L.vcache, m->p.kv_dtype, past_dev, rows, H, KH, hd,
 			                       m->p.rope_dimension_count, m->cos_t, m->sin_t, s);
 			// a prompt's rows go through the matrix cores (fp16 operands) unless f32 operands are asked for
