@@ -120,7 +120,9 @@ def bench_gemm(ln, hiprt, fmt, n, k, m, iters=40, n_buffers=8, seed=7):
     weights = [ln.Tensor.from_numpy(np.roll(wq_host, b, axis=0).reshape(-1)) for b in range(n_buffers)]
     x = ln.Tensor.from_numpy(synth.activations(m, k, seed + 1))
     y = ln.Tensor((m, n))
-    ws_bytes = lib.litenn_hip_mul_mat_q_workspace_bytes(m, k)
+    # the fp16 copy of the activations, plus room for three more products: lets the library walk K
+    # in parts at once where a single walk would leave the card short of work
+    ws_bytes = (lib.litenn_hip_mul_mat_q_workspace_bytes(m, k) + 15) // 16 * 16 + 3 * 4 * m * n
     ws = ln.Tensor((ws_bytes // 4,))
     stream = hiprt.Stream()
     opts = Exec(stream.handle, 0)

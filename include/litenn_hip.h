@@ -133,9 +133,11 @@ int litenn_hip_permute(int dev, void* dst, int dtype, const size_t* src_shape, s
  * The matrix-core path needs a device workspace of litenn_hip_mul_mat_q_workspace_bytes(m, k):
  * litenn_hip_mul_mat_q allocates and frees it itself (and therefore always synchronises for
  * m >= 16); litenn_hip_mul_mat_q_ws takes the caller's (16-byte aligned; NULL = as above).
- * A workspace at least 4*m*n bytes larger than that (rounded up to 16) also lets a product with
- * k >= 8192 whose 128 x 128 tiles would fill only half the card walk K in two halves at once;
- * the halves are added in a fixed order, so results do not depend on scheduling. */
+ * A workspace larger than that (rounded up to 16) by 4*m*n bytes, or by three times as much,
+ * also lets a launch that would leave the card short of work walk K in two, or four, parts at
+ * once (k >= 8192 with 128 x 128 tiles on half the card; m <= 32 or so, where the launch is a
+ * stream of the weights); the parts are added in K order, so results do not depend on
+ * scheduling. */
 #define LITENN_HIP_MATMUL_PRECISE 1u
 int litenn_hip_mul_mat_q(int dev, int fmt, const void* wq, size_t n, size_t k, const void* x, int x_dtype, size_t m,
                          void* y, const void* residual, unsigned flags, const litenn_hip_exec* opts);

@@ -15,7 +15,8 @@ namespace litenn_hip
 	                const float* residual, hipStream_t stream);
 	size_t gemm_scratch_halves(size_t m, size_t k);
 	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
-	                 const float* residual, void* scratch_halves, float* partial, hipStream_t stream);
+	                 const float* residual, void* scratch_halves, float* partial, size_t partial_floats,
+	                 hipStream_t stream);
 	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
 	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
 	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream);
@@ -553,18 +554,19 @@ extern "C" int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t 
 	{
 		// the matrix-core path rounds the activations to fp16 into a workspace
 		const size_t need = 2 * gemm_scratch_halves(m, k);
-		// room for a second m x n product behind it lets a long K be cut in two
+		// room for more m x n products behind it lets K be walked in parts
 		const size_t need16 = (need + 15) & ~size_t{ 15 };
-		const size_t with_partial = need16 + sizeof(float) * m * n;
+		const size_t with_partial = need16 + sizeof(float) * m * n * (m <= 64 ? 3 : 1);
 		if (workspace)
 		{
 			if (workspace_bytes < need)
 			{
 				return fail(action, "workspace is smaller than litenn_hip_mul_mat_q_workspace_bytes(m, k)");
 			}
-			float* partial =
-			    workspace_bytes >= with_partial ? reinterpret_cast<float*>(static_cast<char*>(workspace) + need16) : nullptr;
-			if (!launch_gemm(fmt, wq, n, k, xf, m, yf, rf, workspace, partial, s))
+			const bool roomy = workspace_bytes >= need16 + sizeof(float) * m * n;
+			float* partial = roomy ? reinterpret_cast<float*>(static_cast<char*>(workspace) + need16) : nullptr;
+			const size_t partial_floats = roomy ? (workspace_bytes - need16) / sizeof(float) : 0;
+			if (!launch_gemm(fmt, wq, n, k, xf, m, yf, rf, workspace, partial, partial_floats, s))
 			{
 				launch_gemv(fmt, wq, n, k, xf, m, yf, rf, s);
 			}
@@ -573,10 +575,11 @@ extern "C" int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t 
 		// none given: this call owns one, and frees it after the stream has drained, whatever
 		// opts->synchronize says
 		void* scratch = nullptr;
-		const bool long_k = k >= 8192 && m >= 128;
-		LITENN_HIP_TRY(action, hipMalloc(&scratch, long_k ? with_partial : need));
-		float* partial = long_k ? reinterpret_cast<float*>(static_cast<char*>(scratch) + need16) : nullptr;
-		if (!launch_gemm(fmt, wq, n, k, xf, m, yf, rf, scratch, partial, s))
+		const bool splits = (k >= 8192 && m >= 128) || m <= 64;
+		LITENN_HIP_TRY(action, hipMalloc(&scratch, splits ? with_partial : need));
+		float* partial = splits ? reinterpret_cast<float*>(static_cast<char*>(scratch) + need16) : nullptr;
+		if (!launch_gemm(fmt, wq, n, k, xf, m, yf, rf, scratch, partial, splits ? (with_partial - need16) / sizeof(float) : 0,
+		                 s))
 		{
 			launch_gemv(fmt, wq, n, k, xf, m, yf, rf, s);
 		}

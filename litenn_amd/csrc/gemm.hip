@@ -854,7 +854,7 @@ namespace litenn_hip
 			float* y[3];
 			int n[3];
 			int first_block[3]; // grid x index of each matrix's first row block (INT_MAX when unused)
-			float* partial;     // [M, n[0]]: product of the second K range when grid z = 2 (single matrix)
+			float* partial;     // [grid z - 1][M, n[0]]: products of the later K ranges of a split walk (single matrix)
 		};
 
 		template <typename F, int MT, int NG, int WAVES>
@@ -1060,6 +1060,10 @@ namespace litenn_hip
 				if (has_next)
 				{
 					issue_x(2 * c + 2, far);
+					// The weight slot is about to be overwritten: the reads that moved chunk c out of it
+					// (issued one step ago, waited for only as the decode needs them) must have returned.
+					// Under LDS contention a late read can otherwise meet a request served from L2.
+					asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 					issue_w(c + 1);
 				}
 				plain_step(cur, 0);
@@ -1144,7 +1148,8 @@ namespace litenn_hip
 					if (mm < m)
 					{
 						// the second K range of a split walk leaves its product beside y (no residual)
-						float* dst = (blockIdx.z == 0 ? y : mats.partial) + static_cast<size_t>(mm) * n + n0;
+						float* dst = (blockIdx.z == 0 ? y : mats.partial + (blockIdx.z - 1) * (static_cast<size_t>(m) * n)) +
+						             static_cast<size_t>(mm) * n + n0;
 						const float* res =
 						    residual && blockIdx.z == 0 ? residual + static_cast<size_t>(mm) * n + n0 : nullptr;
 						const float us = unscale[mm];
@@ -1189,8 +1194,9 @@ namespace litenn_hip
 			int k, m, m_tiles;
 			size_t row_bytes;
 			int tile;       // MT * 100 + NG * 10 + WAVES
-			int k_splits;   // 1, or 2: two workgroups share a tile's K walk, the second writes `partial`
-			float* partial; // [M, n[0]] floats, or null: K is never split
+			int k_splits;   // 1, 2 or 4 workgroups share a tile's K walk; all but the first write `partial`
+			float* partial; // room for the later K ranges' products, or null: K is never split
+			size_t partial_floats;
 			hipStream_t stream;
 		};
 
@@ -1223,24 +1229,33 @@ namespace litenn_hip
 		// Tile choice: MT activation tiles per workgroup so that a weight is decoded as few times as
 		// possible; two weight groups per wavefront (each activation fragment read from LDS feeds two
 		// MFMAs) when that still nearly fills the card.
-		// y += partial, element by element: the fixed order (first K range, then second) keeps the
+		// y += partial[0] + partial[1] + ..., element by element in K order: the fixed order keeps the
 		// result independent of scheduling
 		__global__ __launch_bounds__(256) void add_partial_kernel(float* __restrict__ y, const float* __restrict__ partial,
-		                                                           size_t total)
+		                                                           size_t total, int parts)
 		{
 			const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
-			if (i + 3 < total && (reinterpret_cast<uintptr_t>(y) & 15) == 0 && (reinterpret_cast<uintptr_t>(partial) & 15) == 0)
+			if (i + 3 < total && (total & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 &&
+			    (reinterpret_cast<uintptr_t>(partial) & 15) == 0)
 			{
 				float4 a = *reinterpret_cast<float4*>(y + i);
-				const float4 b = *reinterpret_cast<const float4*>(partial + i);
-				a.x += b.x, a.y += b.y, a.z += b.z, a.w += b.w;
+				for (int p = 0; p < parts; ++p)
+				{
+					const float4 b = *reinterpret_cast<const float4*>(partial + p * total + i);
+					a.x += b.x, a.y += b.y, a.z += b.z, a.w += b.w;
+				}
 				*reinterpret_cast<float4*>(y + i) = a;
 			}
 			else
 			{
 				for (size_t e = i; e < total && e < i + 4; ++e)
 				{
-					y[e] += partial[e];
+					float a = y[e];
+					for (int p = 0; p < parts; ++p)
+					{
+						a += partial[p * total + e];
+					}
+					y[e] = a;
 				}
 			}
 		}
@@ -1280,8 +1295,8 @@ namespace litenn_hip
 				{
 					pick = 818;
 				}
-				else if (split_ok && c.partial && m_tiles >= 8 && c.count == 1 && c.k >= kSplitMinK &&
-				         10 * blocks(8, 128) >= 4 * cus)
+				else if (split_ok && c.partial && c.partial_floats >= static_cast<size_t>(c.m) * c.n[0] && m_tiles >= 8 &&
+				         c.count == 1 && c.k >= kSplitMinK && 10 * blocks(8, 128) >= 4 * cus)
 				{
 					pick = 818;
 					c.k_splits = 2;
@@ -1300,6 +1315,22 @@ namespace litenn_hip
 				}
 			}
 			c.tile = pick;
+			// Few rows of activations: the launch is a stream of the weights, and the four-wavefront
+			// tiles keep too few bytes in flight to fill the memory system (one chunk per wavefront).
+			// More workgroups over the same tiles, each walking a part of K, put them there.
+			if (forced == 0 && split_ok && c.k_splits == 1 && c.partial && c.count == 1 && (pick == 114 || pick == 214))
+			{
+				const long waves = blocks(pick / 100, 64) * 4;
+				const size_t one = static_cast<size_t>(c.m) * c.n[0];
+				const int chunks = c.k / kChunk;
+				int splits = 1;
+				while (splits < 4 && waves * splits < 8L * cus && chunks / (2 * splits) >= 2 &&
+				       c.partial_floats >= (2 * splits - 1) * one)
+				{
+					splits *= 2;
+				}
+				c.k_splits = splits;
+			}
 		}
 
 		template <typename F>
@@ -1336,7 +1367,7 @@ namespace litenn_hip
 			{
 				const size_t total = static_cast<size_t>(c.m) * c.n[0];
 				add_partial_kernel<<<dim3(static_cast<unsigned>((total / 4 + 255) / 256 + 1)), dim3(256), 0, c.stream>>>(
-				    c.y[0], c.partial, total);
+				    c.y[0], c.partial, total, c.k_splits - 1);
 			}
 		}
 	} // namespace
@@ -1355,10 +1386,12 @@ namespace litenn_hip
 	// not one this kernel takes (the caller then composes the operators and uses the GEMV): K must be
 	// a whole number of 256-element chunks and at most 16384 (a thread of the pre-pass holds its share
 	// of a row in registers), and the rows 16-byte aligned (2-byte for Q6_K).
-	// partial: null, or M x n[0] floats the launch may use to cut a long K in two (single matrix).
+	// partial: null, or partial_floats floats the launch may use to walk K in 2 or 4 parts at once
+	// (single matrix): M x n[0] per part after the first.
 	bool launch_gemm_group(int fmt, int count, const void* const* wq, const size_t* n, size_t k, const float* x,
 	                       size_t m, float* const* y, const float* residual, const float* norm_w, double eps,
-	                       const float* up, void* scratch_halves, float* partial, hipStream_t stream)
+	                       const float* up, void* scratch_halves, float* partial, size_t partial_floats,
+	                       hipStream_t stream)
 	{
 		const size_t rb = row_bytes(fmt, k);
 		switch (fmt)
@@ -1419,6 +1452,7 @@ namespace litenn_hip
 		c.m_tiles = static_cast<int>(m_pad / 16);
 		c.row_bytes = rb;
 		c.partial = partial;
+		c.partial_floats = partial ? partial_floats : 0;
 		c.stream = stream;
 		const int mp = static_cast<int>(m_pad);
 		switch (fmt)
@@ -1438,11 +1472,12 @@ namespace litenn_hip
 	}
 
 	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
-	                 const float* residual, void* scratch_halves, float* partial, hipStream_t stream)
+	                 const float* residual, void* scratch_halves, float* partial, size_t partial_floats,
+	                 hipStream_t stream)
 	{
 		const void* w[1] = { wq };
 		float* ys[1] = { y };
 		return launch_gemm_group(fmt, 1, w, &n, k, x, m, ys, residual, nullptr, 0.0, nullptr, scratch_halves, partial,
-		                         stream);
+		                         partial_floats, stream);
 	}
 } // namespace litenn_hip

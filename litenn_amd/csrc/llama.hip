@@ -22,9 +22,11 @@ namespace litenn_hip
 	size_t gemm_scratch_halves(size_t m, size_t k);
 	bool launch_gemm_group(int fmt, int count, const void* const* wq, const size_t* n, size_t k, const float* x,
 	                       size_t m, float* const* y, const float* residual, const float* norm_w, double eps,
-	                       const float* up, void* scratch_halves, float* partial, hipStream_t stream);
+	                       const float* up, void* scratch_halves, float* partial, size_t partial_floats,
+	                       hipStream_t stream);
 	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
-	                 const float* residual, void* scratch_halves, float* partial, hipStream_t stream);
+	                 const float* residual, void* scratch_halves, float* partial, size_t partial_floats,
+	                 hipStream_t stream);
 	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
 	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
 	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream);
@@ -223,7 +225,7 @@ namespace
 	{
 		const bool quant = w.fmt != LITENN_FMT_F16 && w.fmt != LITENN_FMT_F32;
 		if (rows >= kGemmMinRows && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && w.k % 256 == 0 &&
-		    launch_gemm(w.fmt, w.data, w.n, w.k, x, rows, y, residual, m->xh, nullptr, s))
+		    launch_gemm(w.fmt, w.data, w.n, w.k, x, rows, y, residual, m->xh, nullptr, 0, s))
 		{
 			return;
 		}
@@ -255,7 +257,7 @@ namespace
 				n[i] = ws[i]->n;
 			}
 			if (launch_gemm_group(w0.fmt, count, w, n, w0.k, x, rows, ys, residual, norm_w, m->p.rms_norm_epsilon, up,
-			                      m->xh, partial, s))
+			                      m->xh, partial, partial ? rows * static_cast<size_t>(m->p.embedding_length) : 0, s))
 			{
 				return;
 			}

@@ -125,6 +125,23 @@ def test_long_k_is_walked_in_two_halves(hip, oracle, fmt, k, m):
     assert rel_l2(split[:, rows] - res[:, rows], ref) <= TOL
 
 
+@pytest.mark.parametrize("fmt", FORMATS)
+def test_many_small_workgroups_share_a_cu(hip, fmt):
+    """Few activation rows against a wide matrix: small tiles, several workgroups resident on every
+    CU (with room for more products the K walk is also split), so LDS traffic is at its densest.
+    A wavefront's weight slot must not be refilled while reads of it are still queued: no output
+    may be an outlier against the f32-operand path, launch after launch."""
+    for m, n, k in [(64, 4096, 4096), (32, 8192, 2048), (64, 16384, 1024)]:
+        wq = hip.Tensor.from_numpy(synth.quant_weights(fmt, n, k, 3, 1))
+        x = hip.Tensor.from_numpy(synth.activations(m, k, 4, 2))
+        exact = hip.mul_mat_q(fmt, wq, n, k, x, flags=MATMUL_PRECISE).numpy()
+        bound = 0.02 * float(np.abs(exact).max())
+        for _ in range(3):
+            got = hip.mul_mat_q(fmt, wq, n, k, x).numpy()
+            assert rel_l2(got, exact) <= TOL
+            assert float(np.abs(got - exact).max()) < bound
+
+
 def test_gemm_is_linear_in_x_at_full_size(hip):
     """Size-independent property at the full north-star shape: Y(a x1 + x2) = a Y(x1) + Y(x2) up to
     the fp16 rounding of the activations."""
