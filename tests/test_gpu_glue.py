@@ -146,7 +146,8 @@ def test_prompt_attention_closed_forms_at_full_size(hip):
     past + r + 1 value rows; one key that dominates the scores returns that key's value row."""
     rng = np.random.default_rng(15)
     hd = 128
-    for m, past, H, KH in [(128, 0, 32, 32), (512, 0, 32, 8), (512, 512, 32, 8)]:
+    # the last case puts two workgroups on every CU
+    for m, past, H, KH in [(128, 0, 32, 32), (512, 0, 32, 8), (512, 512, 32, 8), (1536, 100, 32, 8)]:
         L = past + m
         k = rng.standard_normal((L, KH * hd)).astype(np.float16)
         v = rng.standard_normal((L, KH * hd)).astype(np.float16)
