@@ -303,10 +303,7 @@ namespace litenn_hip
 			return false;
 		}
 		const float scale = static_cast<float>(1.0 / sqrt(static_cast<double>(head_dim)));
-		static const hipError_t attr =
-		    hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_tile_kernel),
-		                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kAttnTileLds));
-		(void)attr;
+		allow_dynamic_lds(reinterpret_cast<const void*>(&attn_tile_kernel), kAttnTileLds);
 		attn_tile_kernel<<<dim3(n_head, q_tiles), dim3(512), kAttnTileLds, s>>>(
 		    q, static_cast<const uint16_t*>(kcache), static_cast<const uint16_t*>(vcache), out, past_dev,
 		    static_cast<int>(past_host), static_cast<int>(m), static_cast<int>(n_head), static_cast<int>(n_kv_head),

@@ -8,7 +8,10 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <mutex>
+#include <set>
 #include <string>
+#include <utility>
 
 #include "../../include/litenn_hip.h"
 
@@ -19,6 +22,25 @@ namespace litenn_hip
 	{
 		const char* v = getenv(name);
 		return (v && *v) ? atoi(v) : fallback;
+	}
+
+	// Lets `kernel` be launched with up to `bytes` of dynamic LDS.  The attribute belongs to the
+	// kernel's instance on one device, so it is set once per (device, kernel), for the device that
+	// is current at the launch.
+	inline void allow_dynamic_lds(const void* kernel, size_t bytes)
+	{
+		static std::mutex mutex;
+		static std::set<std::pair<int, const void*>> done;
+		int dev = 0;
+		if (hipGetDevice(&dev) != hipSuccess)
+		{
+			return; // the launch that follows reports the error
+		}
+		std::lock_guard<std::mutex> lock(mutex);
+		if (done.insert({ dev, kernel }).second)
+		{
+			(void)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes));
+		}
 	}
 
 	// ---- error reporting: status code + thread-local message ---------------

@@ -1205,10 +1205,7 @@ namespace litenn_hip
 		{
 			constexpr size_t lds = gemm_lds_bytes<F, MT, NG, WAVES>();
 			static_assert(lds <= kLdsLimit, "LDS budget");
-			static const hipError_t attr =
-			    hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_q_kernel<F, MT, NG, WAVES>),
-			                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-			(void)attr;
+			allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_q_kernel<F, MT, NG, WAVES>), lds);
 			constexpr int bn = 16 * WAVES * NG;
 			GemmMats mats;
 			mats.partial = c.partial;

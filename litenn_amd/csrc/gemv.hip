@@ -1764,10 +1764,7 @@ namespace litenn_hip
 		template <typename U, int XP>
 		void launch_stream_variant(const GemvArgs& a, int blocks, size_t lds, hipStream_t stream)
 		{
-			static const hipError_t attr =
-			    hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_stream_kernel<U, XP>),
-			                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kStreamLdsLimit));
-			(void)attr;
+			allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U, XP>), kStreamLdsLimit);
 			gemv_stream_kernel<U, XP><<<dim3(blocks), dim3(64 * a.slices * a.groups), lds, stream>>>(a);
 		}
 
