@@ -22,6 +22,8 @@
 //     is issued: a mask produces the operand of v_fma_mix_f32.
 #include "common.hpp"
 
+#include <type_traits>
+
 #include <algorithm>
 #include <cstdlib>
 
@@ -1119,8 +1121,16 @@ namespace litenn_hip
 			return __fmul_rn(__fmul_rn(g, sig), u);
 		}
 
+		// A launch is one or two parts: workgroups [0, blocks0) walk part 0, the rest part 1, whose
+		// matrices may have another block format (q/k in one format and v in another share a launch).
+		struct GemvLaunch
+		{
+			GemvArgs part[2];
+			int blocks0;
+		};
+
 		template <typename U, int XP>
-		__global__ __launch_bounds__(512) void gemv_stream_kernel(const GemvArgs a)
+		__device__ __forceinline__ void gemv_stream_body(const GemvArgs a, const int block)
 		{
 			constexpr int PD = kPrefetchRows;
 			constexpr int kLoadsPerRowMax = (U::kSliceBytes + 1023) / 1024;
@@ -1143,7 +1153,7 @@ namespace litenn_hip
 			const uint32_t rows_base = x_bytes + static_cast<uint32_t>(wave) * (PD * U::kSliceBytes);
 			const uint32_t part_base = x_bytes + static_cast<uint32_t>(nwaves) * (PD * U::kSliceBytes);
 			const uint32_t norm_base = part_base + ((static_cast<uint32_t>(nwaves * rpg) * 4u + 7u) & ~7u);
-			const int row0 = (blockIdx.x * groups + g) * rpg;
+			const int row0 = (block * groups + g) * rpg;
 			const int count = max(0, min(rpg, a.n_total - row0));
 			const uint32_t slice_off = static_cast<uint32_t>(s) * U::kSliceBytes;
 			const uint32_t slice_len = min(static_cast<uint32_t>(U::kSliceBytes), a.row_bytes - slice_off);
@@ -1192,7 +1202,7 @@ namespace litenn_hip
 				{
 					const uint8_t* wm = cursor_m == 0 ? a.w[0] : (cursor_m == 1 ? a.w[1] : a.w[2]);
 					next_a = wm + static_cast<size_t>(local) * a.row_bytes + slice_off;
-					cursor_left = a.n[cursor_m] - local;
+					cursor_left = (cursor_m == 0 ? a.n[0] : (cursor_m == 1 ? a.n[1] : a.n[2])) - local;
 				}
 			}
 			auto issue_row = [&](uint32_t slot_off) {
@@ -1222,7 +1232,7 @@ namespace litenn_hip
 				{
 					++cursor_m;
 					next_a = (cursor_m == 1 ? a.w[1] : a.w[2]) + slice_off;
-					cursor_left = a.n[cursor_m];
+					cursor_left = cursor_m == 1 ? a.n[1] : a.n[2];
 				}
 			};
 			const int first_rows = min(count, PD);
@@ -1391,7 +1401,7 @@ namespace litenn_hip
 				}
 				lds_barrier();
 				const int t = threadIdx.x;
-				vr = blockIdx.x * groups * rpg + t;
+				vr = block * groups * rpg + t;
 				have = t < groups * rpg && vr < a.n_total;
 				res = 0.0f;
 				if (have)
@@ -1427,6 +1437,27 @@ namespace litenn_hip
 					res += a.residual[local];
 				}
 				ym[local] = res;
+			}
+		}
+
+		template <typename U0, typename U1, int XP>
+		__global__ __launch_bounds__(512) void gemv_stream_kernel(const GemvLaunch launch)
+		{
+			if constexpr (std::is_same<U0, U1>::value)
+			{
+				gemv_stream_body<U0, XP>(launch.part[0], static_cast<int>(blockIdx.x));
+			}
+			else
+			{
+				// uniform per workgroup
+				if (static_cast<int>(blockIdx.x) < launch.blocks0)
+				{
+					gemv_stream_body<U0, XP>(launch.part[0], static_cast<int>(blockIdx.x));
+				}
+				else
+				{
+					gemv_stream_body<U1, XP>(launch.part[1], static_cast<int>(blockIdx.x) - launch.blocks0);
+				}
 			}
 		}
 
@@ -1761,16 +1792,18 @@ namespace litenn_hip
 			return cus;
 		}
 
-		template <typename U, int XP>
-		void launch_stream_variant(const GemvArgs& a, int blocks, size_t lds, hipStream_t stream)
+		template <typename U0, typename U1, int XP>
+		void launch_stream_variant(const GemvLaunch& launch, int blocks, int threads, size_t lds, hipStream_t stream)
 		{
-			allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U, XP>), kStreamLdsLimit);
-			gemv_stream_kernel<U, XP><<<dim3(blocks), dim3(64 * a.slices * a.groups), lds, stream>>>(a);
+			allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, U1, XP>), kStreamLdsLimit);
+			gemv_stream_kernel<U0, U1, XP><<<dim3(blocks), dim3(threads), lds, stream>>>(launch);
 		}
 
-		// Returns false when the shape does not fit the streaming kernel.
+		// Fills the launch geometry of one part for a budget of `max_blocks` workgroups (one round, at
+		// most one per CU, every group walking the same number of rows, an even number when gate/up
+		// rows are paired).  Returns false when the shape does not fit the streaming kernel.
 		template <typename U>
-		bool launch_stream(GemvArgs a, hipStream_t stream)
+		bool plan_stream(GemvArgs& a, int max_blocks, int& blocks, size_t& lds)
 		{
 			const int k = a.k;
 			a.slices = (k + 4095) / 4096;
@@ -1795,12 +1828,9 @@ namespace litenn_hip
 			{
 				return false;
 			}
-			// Rows per wavefront group: one round of workgroups, at most one per CU, every group
-			// walking the same number of rows (even when gate/up rows are paired).
 			const size_t x_bytes = sizeof(float) * (static_cast<size_t>(k) / 64) * kLdsUnitStride;
 			static const int forced_rows = env_int("LITENN_HIP_GEMV_ROWS", 0);
-			const int cus = compute_units();
-			int rows = (a.n_total + cus * a.groups - 1) / (cus * a.groups);
+			int rows = (a.n_total + max_blocks * a.groups - 1) / (max_blocks * a.groups);
 			if (forced_rows > 0)
 			{
 				rows = forced_rows;
@@ -1811,31 +1841,94 @@ namespace litenn_hip
 				++rows;
 			}
 			a.rows_per_group = rows;
-			const int blocks = (a.n_total + a.groups * rows - 1) / (a.groups * rows);
-			const size_t lds = x_bytes + static_cast<size_t>(nwaves) * kPrefetchRows * U::kSliceBytes +
-			                   ((sizeof(float) * nwaves * rows + 7) & ~size_t{ 7 }) + sizeof(double) * nwaves;
-			if (lds > kStreamLdsLimit)
-			{
-				return false;
-			}
-			// more than half of the CU's LDS: the dispatcher cannot stack two of these workgroups
-			// on one CU while another CU has none
+			blocks = (a.n_total + a.groups * rows - 1) / (a.groups * rows);
+			lds = x_bytes + static_cast<size_t>(nwaves) * kPrefetchRows * U::kSliceBytes +
+			      ((sizeof(float) * nwaves * rows + 7) & ~size_t{ 7 }) + sizeof(double) * nwaves;
+			return lds <= kStreamLdsLimit;
+		}
+
+		// more than half of the CU's LDS: the dispatcher cannot stack two of these workgroups on one
+		// CU while another CU has none
+		size_t exclusive_lds(size_t lds)
+		{
 			static const int exclusive = env_int("LITENN_HIP_GEMV_EXCLUSIVE", 1);
-			const size_t lds_request = exclusive ? std::max(lds, kStreamLdsLimit / 2 + 1024) : lds;
-			const int threads = 64 * nwaves;
-			const int per_thread = (k / 4 + threads - 1) / threads; // 128-bit activation loads per thread
+			return exclusive ? std::max(lds, kStreamLdsLimit / 2 + 1024) : lds;
+		}
+
+		template <typename U0, typename U1>
+		void launch_stream_xp(const GemvLaunch& launch, int blocks, size_t lds, hipStream_t stream)
+		{
+			const GemvArgs& a = launch.part[0];
+			const int threads = 64 * a.slices * a.groups;
+			const int per_thread = (a.k / 4 + threads - 1) / threads; // 128-bit activation loads per thread
 			if (per_thread <= 2)
 			{
-				launch_stream_variant<U, 2>(a, blocks, lds_request, stream);
+				launch_stream_variant<U0, U1, 2>(launch, blocks, threads, lds, stream);
 			}
 			else if (per_thread <= 4)
 			{
-				launch_stream_variant<U, 4>(a, blocks, lds_request, stream);
+				launch_stream_variant<U0, U1, 4>(launch, blocks, threads, lds, stream);
 			}
 			else
 			{
-				launch_stream_variant<U, kXPerThread>(a, blocks, lds_request, stream);
+				launch_stream_variant<U0, U1, kXPerThread>(launch, blocks, threads, lds, stream);
 			}
+		}
+
+		template <typename U>
+		bool launch_stream(GemvArgs a, hipStream_t stream)
+		{
+			int blocks = 0;
+			size_t lds = 0;
+			if (!plan_stream<U>(a, compute_units(), blocks, lds))
+			{
+				return false;
+			}
+			GemvLaunch launch{};
+			launch.part[0] = a;
+			launch.blocks0 = blocks;
+			launch_stream_xp<U, U>(launch, blocks, exclusive_lds(lds), stream);
+			return true;
+		}
+
+		// Two parts of different block formats over the same activations in one launch.  The CUs are
+		// shared out so that the slower part finishes as early as possible: a group's time goes with
+		// its run length times the bytes of its rows.
+		template <typename U0, typename U1>
+		bool launch_stream_pair(GemvArgs a0, GemvArgs a1, hipStream_t stream)
+		{
+			const int cus = compute_units();
+			long best_cost = -1;
+			int best_b0 = 0;
+			for (int b0 = 1; b0 < cus; ++b0)
+			{
+				GemvArgs t0 = a0, t1 = a1;
+				int blocks0 = 0, blocks1 = 0;
+				size_t lds0 = 0, lds1 = 0;
+				if (!plan_stream<U0>(t0, b0, blocks0, lds0) || !plan_stream<U1>(t1, cus - b0, blocks1, lds1))
+				{
+					return false; // the fit does not depend on the share
+				}
+				const long cost = std::max(static_cast<long>(t0.rows_per_group) * t0.row_bytes,
+				                           static_cast<long>(t1.rows_per_group) * t1.row_bytes);
+				if (best_cost < 0 || cost < best_cost)
+				{
+					best_cost = cost;
+					best_b0 = b0;
+				}
+			}
+			int blocks0 = 0, blocks1 = 0;
+			size_t lds0 = 0, lds1 = 0;
+			if (best_cost < 0 || !plan_stream<U0>(a0, best_b0, blocks0, lds0) ||
+			    !plan_stream<U1>(a1, cus - best_b0, blocks1, lds1) || a0.slices != a1.slices || a0.groups != a1.groups)
+			{
+				return false;
+			}
+			GemvLaunch launch{};
+			launch.part[0] = a0;
+			launch.part[1] = a1;
+			launch.blocks0 = blocks0;
+			launch_stream_xp<U0, U1>(launch, blocks0 + blocks1, exclusive_lds(std::max(lds0, lds1)), stream);
 			return true;
 		}
 
@@ -1888,6 +1981,69 @@ namespace litenn_hip
 			default: return launch_stream<Q6_KUnit>(a, stream);
 			}
 		}
+
+		// the format pairs that share a launch: the K-quant mixes of llama.cpp keep some projections
+		// (attn_v among q/k/v) in Q6_K beside Q4_K or Q5_K ones
+		bool stream_dispatch_pair(int fmt0, int fmt1, const GemvArgs& a0, const GemvArgs& a1, hipStream_t stream)
+		{
+			static const int use_stream = env_int("LITENN_HIP_GEMV_STREAM", 1);
+			static const int use_pairs = env_int("LITENN_HIP_GEMV_PAIRS", 1);
+			if (!use_stream || !use_pairs || a0.k % 256 != 0)
+			{
+				return false;
+			}
+			if (fmt0 == LITENN_FMT_Q4_K && fmt1 == LITENN_FMT_Q6_K)
+			{
+				return launch_stream_pair<Q4_KUnit, Q6_KUnit>(a0, a1, stream);
+			}
+			if (fmt0 == LITENN_FMT_Q5_K && fmt1 == LITENN_FMT_Q6_K)
+			{
+				return launch_stream_pair<Q5_KUnit, Q6_KUnit>(a0, a1, stream);
+			}
+			return false;
+		}
+
+		// arguments of one part: `count` same-format matrices over x
+		bool fill_args(GemvArgs& a, int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
+		               const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul)
+		{
+			if (count < 1 || count > 3 || k > 0x7fffffffu || (silu_mul && (count != 2 || n[0] != n[1])) ||
+			    (residual && count != 1))
+			{
+				return false;
+			}
+			a = GemvArgs{};
+			size_t total = 0;
+			for (int m = 0; m < count; ++m)
+			{
+				if (n[m] == 0 || n[m] > 0x3fffffffu)
+				{
+					return false;
+				}
+				a.w[m] = static_cast<const uint8_t*>(w[m]);
+				a.y[m] = y[m];
+				a.n[m] = static_cast<int>(n[m]);
+				total += n[m];
+			}
+			if (total > 0x7fffffffu)
+			{
+				return false;
+			}
+			const size_t rb = row_bytes(fmt, k);
+			if (rb == 0 || rb > 0xffffffffull)
+			{
+				return false;
+			}
+			a.x = x;
+			a.residual = residual;
+			a.norm_w = norm_w;
+			a.eps = eps;
+			a.n_total = static_cast<int>(total);
+			a.k = static_cast<int>(k);
+			a.row_bytes = static_cast<uint32_t>(rb);
+			a.silu_mul = silu_mul ? 1 : 0;
+			return true;
+		}
 	} // namespace
 
 	// One fused launch over up to three same-format matrices that share x (see GemvArgs).  Returns
@@ -1897,42 +2053,43 @@ namespace litenn_hip
 	                       const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
 	                       hipStream_t stream)
 	{
-		if (count < 1 || count > 3 || k > 0x7fffffffu || (silu_mul && (count != 2 || n[0] != n[1])) ||
-		    (residual && count != 1))
+		GemvArgs a;
+		return fill_args(a, fmt, count, w, y, n, k, x, residual, norm_w, eps, silu_mul) && stream_dispatch(fmt, a, stream);
+	}
+
+	// The same for two or three matrices of two block formats (fmts[i] per matrix, equal formats
+	// adjacent): one launch whose workgroups are shared out between the two formats.  Returns false,
+	// launching nothing, when the formats are not such a pair or the shape does not fit.
+	bool launch_gemv_fused_mixed(const int* fmts, int count, const void* const* w, float* const* y, const size_t* n,
+	                             size_t k, const float* x, const float* norm_w, double eps, hipStream_t stream)
+	{
+		if (count < 2 || count > 3)
 		{
 			return false;
 		}
-		GemvArgs a{};
-		size_t total = 0;
-		for (int m = 0; m < count; ++m)
+		int first = 1; // matrices of the first format
+		while (first < count && fmts[first] == fmts[0])
 		{
-			if (n[m] == 0 || n[m] > 0x3fffffffu)
+			++first;
+		}
+		if (first == count)
+		{
+			return launch_gemv_fused(fmts[0], count, w, y, n, k, x, nullptr, norm_w, eps, false, stream);
+		}
+		for (int i = first + 1; i < count; ++i)
+		{
+			if (fmts[i] != fmts[first])
 			{
-				return false;
+				return false; // three formats
 			}
-			a.w[m] = static_cast<const uint8_t*>(w[m]);
-			a.y[m] = y[m];
-			a.n[m] = static_cast<int>(n[m]);
-			total += n[m];
 		}
-		if (total > 0x7fffffffu)
+		GemvArgs a0, a1;
+		if (!fill_args(a0, fmts[0], first, w, y, n, k, x, nullptr, norm_w, eps, false) ||
+		    !fill_args(a1, fmts[first], count - first, w + first, y + first, n + first, k, x, nullptr, norm_w, eps, false))
 		{
 			return false;
 		}
-		const size_t rb = row_bytes(fmt, k);
-		if (rb == 0 || rb > 0xffffffffull)
-		{
-			return false;
-		}
-		a.x = x;
-		a.residual = residual;
-		a.norm_w = norm_w;
-		a.eps = eps;
-		a.n_total = static_cast<int>(total);
-		a.k = static_cast<int>(k);
-		a.row_bytes = static_cast<uint32_t>(rb);
-		a.silu_mul = silu_mul ? 1 : 0;
-		return stream_dispatch(fmt, a, stream);
+		return stream_dispatch_pair(fmts[0], fmts[first], a0, a1, stream);
 	}
 
 	// y[m, n] = x[m, k] . W^T (+ residual), one activation row at a time.

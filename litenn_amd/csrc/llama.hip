@@ -30,6 +30,8 @@ namespace litenn_hip
 	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
 	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
 	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream);
+	bool launch_gemv_fused_mixed(const int* fmts, int count, const void* const* w, float* const* y, const size_t* n,
+	                             size_t k, const float* x, const float* norm_w, double eps, hipStream_t stream);
 	void launch_get_rows_q(int fmt, const void* table, size_t rows, size_t k, const int32_t* ids, size_t n_ids,
 	                       float* out, int* err_flag, hipStream_t stream);
 	void launch_rmsnorm(const float* x, const float* w, double eps, size_t m, size_t d, float* y, hipStream_t s);
@@ -311,15 +313,26 @@ namespace
 		{
 			const Weight* qkv[3] = { &L.wq, &L.wk, &L.wv };
 			float* qkv_out[3] = { m->q, m->k, m->v };
-			for (int i = 0; i < 3;)
+			// one launch when the three share a format or are one of the two-format mixes the GEMV
+			// takes (q/k in Q4_K or Q5_K beside a Q6_K v); otherwise one per run of equal formats
+			const int qkv_fmt[3] = { L.wq.fmt, L.wk.fmt, L.wv.fmt };
+			const void* qkv_w[3] = { L.wq.data, L.wk.data, L.wv.data };
+			const size_t qkv_n[3] = { L.wq.n, L.wk.n, L.wv.n };
+			const bool mixed = L.wq.fmt != L.wk.fmt || L.wk.fmt != L.wv.fmt;
+			if (!(mixed && L.wq.k == L.wk.k && L.wk.k == L.wv.k &&
+			      launch_gemv_fused_mixed(qkv_fmt, 3, qkv_w, qkv_out, qkv_n, L.wq.k, m->x, L.attn_norm,
+			                              m->p.rms_norm_epsilon, s)))
 			{
-				int j = i + 1;
-				while (j < 3 && qkv[j]->fmt == qkv[i]->fmt)
+				for (int i = 0; i < 3;)
 				{
-					++j;
+					int j = i + 1;
+					while (j < 3 && qkv[j]->fmt == qkv[i]->fmt)
+					{
+						++j;
+					}
+					group(m, j - i, qkv + i, qkv_out + i, m->x, nullptr, L.attn_norm, false, s);
+					i = j;
 				}
-				group(m, j - i, qkv + i, qkv_out + i, m->x, nullptr, L.attn_norm, false, s);
-				i = j;
 			}
 			const size_t rope_dims = m->p.rope_dimension_count;
 			if (attn_step_fusable(m->q, m->k, m->v, L.kcache, L.vcache, hd, rope_dims, m->cos_t, m->sin_t))

@@ -7,7 +7,7 @@ import pytest
 
 from conftest import rel_l2
 from litenn_amd import synth
-from litenn_amd.formats import DT_F16, DT_F32, Q4_0, Q4_K, Q6_K, Q8_0
+from litenn_amd.formats import DT_F16, DT_F32, Q4_0, Q4_K, Q5_K, Q6_K, Q8_0
 from llama_util import hip_model, oracle_model, tiny_reference_archive
 
 pytestmark = pytest.mark.gpu
@@ -87,6 +87,26 @@ def test_mixed_formats_gqa(hip, oracle):
                                     "token_embd": Q8_0})
     toks = synth.prompt_tokens(cfg, 5, 6)
     assert rel_l2(hip_model(hip, cfg, 3).eval(toks), oracle_model(oracle, cfg, 3).eval(toks)) < 1e-4
+
+
+@pytest.mark.parametrize("main_fmt,d_model,ff", [(Q4_K, 512, 768), (Q5_K, 1024, 1024), (Q4_K, 4096, 512)])
+def test_single_token_steps_with_a_q6_k_value_projection(hip, oracle, main_fmt, d_model, ff):
+    """The K-quant mixes keep attn_v in Q6_K beside Q4_K / Q5_K q and k: the single-token step runs
+    the three projections as one launch whose workgroups are shared out between the two formats.
+    Logits of every step and the cache against the checker; the tokens of a greedy run exactly."""
+    cfg = synth.tiny_llama(main_fmt, block_count=2, d_model=d_model, heads=d_model // 128 * 2, kv_heads=2, ff=ff,
+                           vocab=777, formats={"default": main_fmt, "attn_v": Q6_K, "ffn_down": Q6_K, "output": Q6_K})
+    toks = synth.prompt_tokens(cfg, 9, 8)
+    dev, ref = hip_model(hip, cfg, 4), oracle_model(oracle, cfg, 4)
+    for t in toks:
+        assert rel_l2(dev.eval([t])[0], ref.eval([t])[0]) < 1e-4
+    for layer in range(cfg.block_count):
+        for got, want in zip(dev.get_kv(layer), ref.get_kv(layer)):
+            assert rel_l2(got, want) < 1e-3  # fp16 cache: a rounding flip is 2^-11 of the value
+    dev.reset()
+    ref.reset()
+    got, _, _ = dev.generate(toks[:4], 12)
+    assert got.tolist() == ref.generate(toks[:4], 12)[0].tolist()
 
 
 def test_error_paths(hip):
