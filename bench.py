@@ -292,7 +292,7 @@ def main() -> int:
             "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": GEMV_Q4_K_14336x4096_TRAFFIC_BYTES,
             "traffic_unit": "bytes/launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
             "algorithmic_bytes": algo_bytes,
-            "kernel": "gemv_stream_kernel<Q4_KUnit, 2>",
+            "kernel": "gemv_stream_kernel<Q4_KUnit, Q4_KUnit, 2>",
         },
     }
     if not args.no_cpu:
