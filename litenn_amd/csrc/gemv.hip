@@ -1129,335 +1129,32 @@ namespace litenn_hip
 			int blocks0;
 		};
 
+		// The statements live in gemv_stream_body.inc and are compiled into both forms below.
 		template <typename U, int XP>
-		__device__ __forceinline__ void gemv_stream_body(const GemvArgs a, const int block)
+		__global__ __launch_bounds__(512) void gemv_stream_kernel(const GemvArgs a)
 		{
-			constexpr int PD = kPrefetchRows;
-			constexpr int kLoadsPerRowMax = (U::kSliceBytes + 1023) / 1024;
-			static_assert(kLoadsPerRowMax <= 5 && PD * kLoadsPerRowMax <= 63, "vmcnt range");
-			extern __shared__ __attribute__((aligned(16))) uint8_t smem_b[];
-			const uint32_t lds0 = lds_address(smem_b);
-			const int lane = threadIdx.x & 63;
-			// the wavefront index is uniform: keeping it in a scalar register makes every row
-			// address, bound and branch below scalar work
-			const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-			const int slices = a.slices, groups = a.groups, k = a.k;
-			const int s = wave % slices;
-			const int g = wave / slices;
-			const int unit = s * 64 + lane;
-			const int units_per_row = k >> 6;
-			const bool active = unit < units_per_row;
-			const int nwaves = slices * groups;
-			const uint32_t x_bytes = static_cast<uint32_t>(units_per_row) * kLdsUnitStride * 4u;
-			const int rpg = a.rows_per_group;
-			const uint32_t rows_base = x_bytes + static_cast<uint32_t>(wave) * (PD * U::kSliceBytes);
-			const uint32_t part_base = x_bytes + static_cast<uint32_t>(nwaves) * (PD * U::kSliceBytes);
-			const uint32_t norm_base = part_base + ((static_cast<uint32_t>(nwaves * rpg) * 4u + 7u) & ~7u);
-			const int row0 = (block * groups + g) * rpg;
-			const int count = max(0, min(rpg, a.n_total - row0));
-			const uint32_t slice_off = static_cast<uint32_t>(s) * U::kSliceBytes;
-			const uint32_t slice_len = min(static_cast<uint32_t>(U::kSliceBytes), a.row_bytes - slice_off);
-			const int loads_per_row = static_cast<int>((slice_len + 1023u) >> 10);
-			const bool fuse_norm = a.norm_w != nullptr;
-
-			GEMV_TRACE(0);
-			// 1. activations (and norm weights) first: the oldest loads in flight.  XP 128-bit loads
-			// per thread, clamped so that every lane issues every one of them.  They are issued
-			// outside the compiler's view: it may only order them against the direct-to-LDS loads
-			// below by waiting for everything.
-			f32x4 xv[XP], nw[XP];
-#pragma unroll
-			for (int j = 0; j < XP; ++j)
-			{
-				const int i = min(static_cast<int>(threadIdx.x + j * blockDim.x) * 4, k - 4);
-				xv[j] = asm_global_load128(a.x, static_cast<uint32_t>(i) * 4u);
-			}
-			if (fuse_norm)
-			{
-#pragma unroll
-				for (int j = 0; j < XP; ++j)
-				{
-					const int i = min(static_cast<int>(threadIdx.x + j * blockDim.x) * 4, k - 4);
-					nw[j] = asm_global_load128(a.norm_w, static_cast<uint32_t>(i) * 4u);
-				}
-			}
-
-			// 2. the first rows of the wavefront, straight into their LDS slots
-			// The rows are requested strictly in order, so a cursor walks them: `next_a` is the row
-			// about to be requested; with gate/up pairing `next_b` is the one after it and the two
-			// swap roles after every request; otherwise the cursor hops to the next matrix when the
-			// current one runs out.
-			const uint8_t* next_a;
-			const uint8_t* next_b = nullptr;
-			int cursor_m = 0, cursor_left = 0;
-			{
-				int local = 0;
-				locate_row(a, min(row0, a.n_total - 1), cursor_m, local);
-				if (a.silu_mul)
-				{
-					next_a = a.w[0] + static_cast<size_t>(local) * a.row_bytes + slice_off; // row0 is even
-					next_b = a.w[1] + static_cast<size_t>(local) * a.row_bytes + slice_off;
-				}
-				else
-				{
-					const uint8_t* wm = cursor_m == 0 ? a.w[0] : (cursor_m == 1 ? a.w[1] : a.w[2]);
-					next_a = wm + static_cast<size_t>(local) * a.row_bytes + slice_off;
-					cursor_left = (cursor_m == 0 ? a.n[0] : (cursor_m == 1 ? a.n[1] : a.n[2])) - local;
-				}
-			}
-			auto issue_row = [&](uint32_t slot_off) {
-				const uint8_t* grow = next_a;
-				uint8_t* slot = smem_b + rows_base + slot_off;
-#pragma unroll
-				for (int i = 0; i < kLoadsPerRowMax; ++i)
-				{
-					if (i * 1024 < static_cast<int>(slice_len)) // uniform
-					{
-						const uint32_t off = static_cast<uint32_t>(i) * 1024u + static_cast<uint32_t>(lane) * 16u;
-						if (off < slice_len)
-						{
-							__builtin_amdgcn_global_load_lds((global_ptr_t)(grow + off), (lds_ptr_t)(slot + i * 1024),
-							                                 16, 0, 0);
-						}
-					}
-				}
-				next_a += a.row_bytes;
-				if (a.silu_mul)
-				{
-					const uint8_t* t = next_a;
-					next_a = next_b;
-					next_b = t;
-				}
-				else if (--cursor_left == 0 && cursor_m < 2)
-				{
-					++cursor_m;
-					next_a = (cursor_m == 1 ? a.w[1] : a.w[2]) + slice_off;
-					cursor_left = cursor_m == 1 ? a.n[1] : a.n[2];
-				}
-			};
-			const int first_rows = min(count, PD);
-#pragma unroll
-			for (int r = 0; r < PD; ++r)
-			{
-				if (r < first_rows) // uniform
-				{
-					issue_row(static_cast<uint32_t>(r) * U::kSliceBytes);
-				}
-			}
-
-			// 3. activations into LDS as soon as THEY have arrived (the rows issued after them stay
-			// in flight; the activation registers are only read after this wait)
-			wait_rows_outstanding_dyn<PD>(first_rows, loads_per_row);
-			if (fuse_norm)
-			{
-				// RMSNorm with f64 accumulation (ComputePrimitives.h:792-817): every workgroup sums
-				// the whole vector, so no other kernel or pass over x is needed
-				double ss = 0.0;
-#pragma unroll
-				for (int j = 0; j < XP; ++j)
-				{
-					if (static_cast<int>(threadIdx.x + j * blockDim.x) * 4 < k)
-					{
-						const double x0 = xv[j].x, x1 = xv[j].y, x2 = xv[j].z, x3 = xv[j].w;
-						ss += x0 * x0;
-						ss += x1 * x1;
-						ss += x2 * x2;
-						ss += x3 * x3;
-					}
-				}
-				ss = wave_sum_f64(ss);
-				if (lane == 0)
-				{
-					lds_wr64(lds0 + norm_base + static_cast<uint32_t>(wave) * 8u, ss);
-				}
-				lds_barrier();
-				double total = 0.0;
-				for (int wv = 0; wv < nwaves; ++wv)
-				{
-					total += lds_rd_f64(lds0 + norm_base + static_cast<uint32_t>(wv) * 8u);
-				}
-				const double inv = 1.0 / sqrt(total / static_cast<double>(k) + a.eps);
-#pragma unroll
-				for (int j = 0; j < XP; ++j)
-				{
-					xv[j].x = static_cast<float>(static_cast<double>(xv[j].x) * inv * static_cast<double>(nw[j].x));
-					xv[j].y = static_cast<float>(static_cast<double>(xv[j].y) * inv * static_cast<double>(nw[j].y));
-					xv[j].z = static_cast<float>(static_cast<double>(xv[j].z) * inv * static_cast<double>(nw[j].z));
-					xv[j].w = static_cast<float>(static_cast<double>(xv[j].w) * inv * static_cast<double>(nw[j].w));
-				}
-			}
-			// each float4 lands in the slot of the unit that consumes it, units kLdsUnitStride floats
-			// apart so that the per-lane 128-bit reads below fall on distinct banks
-#pragma unroll
-			for (int j = 0; j < XP; ++j)
-			{
-				const int i = (threadIdx.x + j * blockDim.x) * 4;
-				if (i < k)
-				{
-					lds_wr128(lds0 + static_cast<uint32_t>(U::unit_of(i) * kLdsUnitStride + U::index_of(i)) * 4u, xv[j]);
-				}
-			}
-			GEMV_TRACE(1);
-			lds_barrier();
-			GEMV_TRACE(2);
-
-			// 4. the lane's 64 activations move to registers for good
-			float xr[64];
-			if (active)
-			{
-				const uint32_t xb = lds0 + static_cast<uint32_t>(unit) * (kLdsUnitStride * 4u);
-				u32x4 t[16];
-				t[0] = lds_rd128<0>(xb);
-				t[1] = lds_rd128<16>(xb);
-				t[2] = lds_rd128<32>(xb);
-				t[3] = lds_rd128<48>(xb);
-				t[4] = lds_rd128<64>(xb);
-				t[5] = lds_rd128<80>(xb);
-				t[6] = lds_rd128<96>(xb);
-				t[7] = lds_rd128<112>(xb);
-				t[8] = lds_rd128<128>(xb);
-				t[9] = lds_rd128<144>(xb);
-				t[10] = lds_rd128<160>(xb);
-				t[11] = lds_rd128<176>(xb);
-				t[12] = lds_rd128<192>(xb);
-				t[13] = lds_rd128<208>(xb);
-				t[14] = lds_rd128<224>(xb);
-				t[15] = lds_rd128<240>(xb);
-				asm volatile("s_waitcnt lgkmcnt(0)"
-				             : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]),
-				               "+v"(t[7]), "+v"(t[8]), "+v"(t[9]), "+v"(t[10]), "+v"(t[11]), "+v"(t[12]), "+v"(t[13]),
-				               "+v"(t[14]), "+v"(t[15])
-				             :
-				             : "memory");
-#pragma unroll
-				for (int i = 0; i < 16; ++i)
-				{
-					xr[4 * i] = __uint_as_float(t[i].x);
-					xr[4 * i + 1] = __uint_as_float(t[i].y);
-					xr[4 * i + 2] = __uint_as_float(t[i].z);
-					xr[4 * i + 3] = __uint_as_float(t[i].w);
-				}
-			}
-			else
-			{
-#pragma unroll
-				for (int i = 0; i < 64; ++i)
-				{
-					xr[i] = 0.0f;
-				}
-			}
-			const typename U::Prep pz = U::prep(xr);
-			GEMV_TRACE(3);
-
-			// 5. rows in arrival order; lane r keeps the total of row row0 + r.  Row r has landed
-			// once only the rows issued after it are outstanding: min(PD - 1, count - 1 - r) rows of
-			// `loads_per_row` instructions.  The slot is refilled only after the lanes' LDS reads of
-			// it have returned (unit_dot consumes them before the refill is issued).
-			const uint32_t lane_p = lds0 + rows_base + U::lds_lane_offset(lane);
-			float res = 0.0f;
-			uint32_t slot_off = 0;
-			auto consume = [&](int r) {
-#ifdef LITENN_GEMV_TRACE
-				if (r < 11)
-				{
-					GEMV_TRACE(4 + r);
-				}
-#endif
-				const typename U::Raw raw = unit_lds_load<U>(lane_p + slot_off, lane);
-				const float p = active ? unit_dot<U>(raw, xr, pz, unit) : 0.0f;
-				const float total = wave_sum(p);
-				res = (lane == r) ? total : res;
-			};
-			// A loop rather than straight-line code per row: in a decoder every launch meets a cold
-			// instruction cache, and the unrolled form (16 KB and more) measured slower there.
-			int r = 0;
-			for (; r + PD <= count; ++r) // steady state: PD - 1 younger rows stay in flight
-			{
-				wait_rows_outstanding<PD - 1>(loads_per_row);
-				consume(r);
-				if (r + PD < count)
-				{
-					issue_row(slot_off);
-				}
-				slot_off = slot_off + U::kSliceBytes == PD * U::kSliceBytes ? 0u : slot_off + U::kSliceBytes;
-			}
-			for (; r < count; ++r) // the last rows: nothing left to request
-			{
-				wait_rows_outstanding_dyn<(PD >= 2 ? PD - 2 : 0)>(count - 1 - r, loads_per_row);
-				consume(r);
-				slot_off = slot_off + U::kSliceBytes == PD * U::kSliceBytes ? 0u : slot_off + U::kSliceBytes;
-			}
-			GEMV_TRACE(15);
-
-			// 6. slices of one row meet in LDS; afterwards thread t of the workgroup holds row
-			// block_row0 + t in `res`
-			int vr = row0 + lane;
-			bool have = lane < count;
-			if (slices > 1)
-			{
-				if (lane < rpg)
-				{
-					lds_wr32(lds0 + part_base + static_cast<uint32_t>((s * groups + g) * rpg + lane) * 4u, res);
-				}
-				lds_barrier();
-				const int t = threadIdx.x;
-				vr = block * groups * rpg + t;
-				have = t < groups * rpg && vr < a.n_total;
-				res = 0.0f;
-				if (have)
-				{
-					const int gg = t / rpg, rl = t % rpg;
-					for (int ss = 0; ss < slices; ++ss)
-					{
-						float v = __uint_as_float(
-						    lds_rd32<0>(lds0 + part_base + static_cast<uint32_t>((ss * groups + gg) * rpg + rl) * 4u));
-						lds_wait(v);
-						res += v;
-					}
-				}
-			}
-			if (a.silu_mul)
-			{
-				// even lanes hold gate_i, their odd neighbours up_i (row 2i + m); the run length and
-				// every block origin are even, so pairs never straddle wavefronts
-				const float other = dpp_f32<0xB1>(res); // quad_perm [1,0,3,2]
-				if (have && (vr & 1) == 0)
-				{
-					a.y[0][vr >> 1] = silu_mul_value(res, other);
-				}
-				return;
-			}
-			if (have)
-			{
-				int m, local;
-				locate_row(a, vr, m, local);
-				float* ym = m == 0 ? a.y[0] : (m == 1 ? a.y[1] : a.y[2]);
-				if (m == 0 && a.residual)
-				{
-					res += a.residual[local];
-				}
-				ym[local] = res;
-			}
+			const int block = static_cast<int>(blockIdx.x);
+#include "gemv_stream_body.inc"
 		}
 
-		template <typename U0, typename U1, int XP>
-		__global__ __launch_bounds__(512) void gemv_stream_kernel(const GemvLaunch launch)
+		template <typename U, int XP>
+		__device__ __forceinline__ void gemv_stream_part(const GemvArgs a, const int block)
 		{
-			if constexpr (std::is_same<U0, U1>::value)
+#include "gemv_stream_body.inc"
+		}
+
+
+		template <typename U0, typename U1, int XP>
+		__global__ __launch_bounds__(512) void gemv_stream_pair_kernel(const GemvLaunch launch)
+		{
+			// uniform per workgroup
+			if (static_cast<int>(blockIdx.x) < launch.blocks0)
 			{
-				gemv_stream_body<U0, XP>(launch.part[0], static_cast<int>(blockIdx.x));
+				gemv_stream_part<U0, XP>(launch.part[0], static_cast<int>(blockIdx.x));
 			}
 			else
 			{
-				// uniform per workgroup
-				if (static_cast<int>(blockIdx.x) < launch.blocks0)
-				{
-					gemv_stream_body<U0, XP>(launch.part[0], static_cast<int>(blockIdx.x));
-				}
-				else
-				{
-					gemv_stream_body<U1, XP>(launch.part[1], static_cast<int>(blockIdx.x) - launch.blocks0);
-				}
+				gemv_stream_part<U1, XP>(launch.part[1], static_cast<int>(blockIdx.x) - launch.blocks0);
 			}
 		}
 
@@ -1795,8 +1492,16 @@ namespace litenn_hip
 		template <typename U0, typename U1, int XP>
 		void launch_stream_variant(const GemvLaunch& launch, int blocks, int threads, size_t lds, hipStream_t stream)
 		{
-			allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, U1, XP>), kStreamLdsLimit);
-			gemv_stream_kernel<U0, U1, XP><<<dim3(blocks), dim3(threads), lds, stream>>>(launch);
+			if constexpr (std::is_same<U0, U1>::value)
+			{
+				allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, XP>), kStreamLdsLimit);
+				gemv_stream_kernel<U0, XP><<<dim3(blocks), dim3(threads), lds, stream>>>(launch.part[0]);
+			}
+			else
+			{
+				allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_pair_kernel<U0, U1, XP>), kStreamLdsLimit);
+				gemv_stream_pair_kernel<U0, U1, XP><<<dim3(blocks), dim3(threads), lds, stream>>>(launch);
+			}
 		}
 
 		// Fills the launch geometry of one part for a budget of `max_blocks` workgroups (one round, at
