@@ -1130,16 +1130,18 @@ namespace litenn_hip
 		};
 
 		// The statements live in gemv_stream_body.inc and are compiled into both forms below.
-		template <typename U, int XP>
+		template <typename U, int XP, bool WHOLE>
 		__global__ __launch_bounds__(512) void gemv_stream_kernel(const GemvArgs a)
 		{
 			const int block = static_cast<int>(blockIdx.x);
+			constexpr bool kWholeSlices = WHOLE;
 #include "gemv_stream_body.inc"
 		}
 
 		template <typename U, int XP>
 		__device__ __forceinline__ void gemv_stream_part(const GemvArgs a, const int block)
 		{
+			constexpr bool kWholeSlices = false;
 #include "gemv_stream_body.inc"
 		}
 
@@ -1494,8 +1496,17 @@ namespace litenn_hip
 		{
 			if constexpr (std::is_same<U0, U1>::value)
 			{
-				allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, XP>), kStreamLdsLimit);
-				gemv_stream_kernel<U0, XP><<<dim3(blocks), dim3(threads), lds, stream>>>(launch.part[0]);
+				// K = 4096 is most of a decoder's launches: its own instance with the slice geometry folded
+				if (XP == 2 && launch.part[0].k == 4096)
+				{
+					allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, 2, true>), kStreamLdsLimit);
+					gemv_stream_kernel<U0, 2, true><<<dim3(blocks), dim3(threads), lds, stream>>>(launch.part[0]);
+				}
+				else
+				{
+					allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, XP, false>), kStreamLdsLimit);
+					gemv_stream_kernel<U0, XP, false><<<dim3(blocks), dim3(threads), lds, stream>>>(launch.part[0]);
+				}
 			}
 			else
 			{
