@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes one launch of the headline GEMV moves, from the profiler's FETCH_SIZE / WRITE_SIZE
 # counters scaled by a known-size copy (profiles/gemv_q4_k_14336x4096_hbm_traffic.txt); it is a
 # property of the kernel and the shape, not re-measured by this script.
-GEMV_Q4_K_14336x4096_TRAFFIC_BYTES = 33314072
+GEMV_Q4_K_14336x4096_TRAFFIC_BYTES = 33291725
 
 
 def log(*a):
@@ -292,7 +292,7 @@ def main() -> int:
             "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": GEMV_Q4_K_14336x4096_TRAFFIC_BYTES,
             "traffic_unit": "bytes/launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
             "algorithmic_bytes": algo_bytes,
-            "kernel": "gemv_stream_kernel<Q4_KUnit, 2>",
+            "kernel": "gemv_stream_kernel<Q4_KUnit, 2, true>",
         },
     }
     if not args.no_cpu:
