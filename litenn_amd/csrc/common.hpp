@@ -104,9 +104,24 @@ namespace litenn_hip
 	// same way.  Not IEEE round-to-nearest-even, so the hardware converter is not used.
 	__device__ __forceinline__ uint16_t f32_to_f16_bits_litenn(float value)
 	{
+		const uint32_t bits = __float_as_uint(value);
+		// Values that land on normal halves (all of them, in practice) take the hardware converter:
+		// round-to-nearest-even differs from the rule above only on an exact tie whose lower
+		// neighbour is even, where one is added (a carry into the exponent, up to infinity, is
+		// what the reference's sum does too).  One wavefront-uniform branch; any lane outside the
+		// range sends the wavefront through the general form below.
+		{
+			const uint32_t e = (bits >> 23) & 0xffu;
+			const bool plain = e >= 113u && e <= 142u;
+			if (__builtin_amdgcn_ballot_w64(!plain) == 0)
+			{
+				const _Float16 h = static_cast<_Float16>(value);
+				const uint32_t hb = __builtin_bit_cast(uint16_t, h);
+				return static_cast<uint16_t>(hb + ((bits & 0x3fffu) == 0x1000u ? 1u : 0u));
+			}
+		}
 		// branch-free: every range is computed and the result selected, so a wave converting a
 		// handful of values does not serialise through divergent paths
-		const uint32_t bits = __float_as_uint(value);
 		const uint32_t sign = (bits >> 16) & 0x8000u;
 		const uint32_t mag = bits & 0x7fffffffu;
 		const uint32_t exp_field = mag >> 23; // biased by 127

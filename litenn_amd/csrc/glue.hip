@@ -323,6 +323,37 @@ namespace litenn_hip
 			return f16_bits_to_f32(f32_to_f16_bits_litenn(v));
 		}
 
+		// The new row's key / value as the cache will hold them: rounded through the cache type once,
+		// used from registers and stored from the same values.
+		template <typename KV>
+		__device__ __forceinline__ void round_through_cache(float (&v)[8])
+		{
+#pragma unroll
+			for (int e = 0; e < 8; ++e)
+			{
+				v[e] = through_cache<KV>(v[e]);
+			}
+		}
+		// values already representable in the cache type: the hardware conversion is exact for them
+		__device__ __forceinline__ void store8_exact(float* dst, const float (&v)[8])
+		{
+			reinterpret_cast<float4*>(dst)[0] = make_float4(v[0], v[1], v[2], v[3]);
+			reinterpret_cast<float4*>(dst)[1] = make_float4(v[4], v[5], v[6], v[7]);
+		}
+		__device__ __forceinline__ void store8_exact(uint16_t* dst, const float (&v)[8])
+		{
+			typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+			typedef float float2v __attribute__((ext_vector_type(2)));
+			uint32_t w[4];
+#pragma unroll
+			for (int i = 0; i < 4; ++i)
+			{
+				const float2v f = { v[2 * i], v[2 * i + 1] };
+				w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, half2v));
+			}
+			*reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+		}
+
 		__device__ __forceinline__ void store8(float* dst, const float (&v)[8])
 		{
 			reinterpret_cast<float4*>(dst)[0] = make_float4(v[0], v[1], v[2], v[3]);
@@ -445,10 +476,15 @@ namespace litenn_hip
 					rotate8(qv, cos4, sin4);
 					rotate8(kn, cos4, sin4);
 				}
-				if (new_key_here && h % (n_head / n_kv_head) == 0)
+				if (new_key_here)
 				{
-					store8(kcache + static_cast<size_t>(pos) * kvw + kvh * head_dim + first, kn);
-					store8(vcache + static_cast<size_t>(pos) * kvw + kvh * head_dim + first, vn);
+					round_through_cache<KV>(kn);
+					round_through_cache<KV>(vn);
+					if (h % (n_head / n_kv_head) == 0)
+					{
+						store8_exact(kcache + static_cast<size_t>(pos) * kvw + kvh * head_dim + first, kn);
+						store8_exact(vcache + static_cast<size_t>(pos) * kvw + kvh * head_dim + first, vn);
+					}
 				}
 			}
 
@@ -519,7 +555,7 @@ namespace litenn_hip
 #pragma unroll
 					for (int e = 0; e < E; ++e)
 					{
-						acc = fmaf(qv[e], through_cache<KV>(kn[e]), acc);
+						acc = fmaf(qv[e], kn[e], acc);
 					}
 					const float sc = row16_sum(acc) * scale;
 					const float step_m = fmaxf(run_m, sc);
@@ -529,7 +565,7 @@ namespace litenn_hip
 #pragma unroll
 					for (int e = 0; e < E; ++e)
 					{
-						o[e] = fmaf(pw, through_cache<KV>(vn[e]), o[e] * corr);
+						o[e] = fmaf(pw, vn[e], o[e] * corr);
 					}
 					run_m = step_m;
 				}

@@ -63,6 +63,18 @@ def test_kv_append_f16_uses_litenn_rounding(hip, oracle, golden):
     raw = cache.numpy()  # float16 view
     assert np.array_equal(raw[3:5].reshape(-1).view(np.uint16), oracle.f32_to_f16_bits(cur))
     assert np.all(raw[:3] == 0) and np.all(raw[5:] == 0)
+    # whole wavefronts of values that land on normal halves (the converter's short path): exact
+    # ties over even and odd lower neighbours, near-ties one f32 ulp to either side, both signs,
+    # every half exponent, and the run up to the overflow boundary
+    exp = rng.integers(113, 143, 8192).astype(np.uint32)
+    kept = rng.integers(0, 1024, 8192).astype(np.uint32)
+    dropped = rng.choice(np.array([0x1000, 0x0fff, 0x1001, 0x0000, 0x1fff], np.uint32), 8192)
+    sign = rng.integers(0, 2, 8192).astype(np.uint32) << 31
+    ties = (sign | (exp << 23) | (kept << 13) | dropped).view(np.float32)
+    ties[:64] = np.linspace(65472.0, 65535.0, 64, dtype=np.float32)
+    cache = hip.Tensor((2, ties.size), DT_F16)
+    hip.kv_append(cache, 1, T(hip, ties), ties.size)
+    assert np.array_equal(cache.numpy()[1].view(np.uint16), oracle.f32_to_f16_bits(ties))
     g = golden["kv_append"]
     c32 = hip.Tensor((3, 2), DT_F32)
     hip.kv_append(c32, 0, T(hip, g["past_k"]), 2)
