@@ -9,6 +9,7 @@ import pytest
 
 import gguf_writer as gw
 from litenn_amd import synth
+from litenn_amd import _lib
 from litenn_amd._lib import LiteNNHipError
 from litenn_amd.formats import Q4_0, Q4_K, Q6_K, Q8_0
 from litenn_amd.gguf import GGUFFile
@@ -133,3 +134,67 @@ def test_broken_files_are_refused(tmp_path):
     bad.write_bytes(bytes(patched))
     with pytest.raises(LiteNNHipError, match="Unsupported ggml tensor type '99' for tensor 'q'"):
         GGUFFile(bad)
+
+
+@pytest.mark.parametrize("kind", ["gguf", "ltnn"])
+def test_mutated_images_are_refused_or_read_never_crash(tmp_path, kind):
+    """Both container readers parse files from outside: truncations anywhere, random bytes and huge
+    counts in the header region, single bit flips.  Every mutant either opens (and every accessor
+    then works on it) or is refused with an error; a fault in the reader would take the test
+    process down.  (The same mutations, tens of thousands per format, were also run once against
+    a host-sanitizer build of the reader.)"""
+    import ltnn_writer as lw
+    cfg = synth.tiny_llama(Q4_K, block_count=1, d_model=256, heads=2, kv_heads=1, ff=256, vocab=64,
+                           formats={"default": Q4_K, "attn_v": Q6_K, "token_embd": Q8_0})
+    base = tmp_path / ("base." + kind)
+    (gw.llama_gguf if kind == "gguf" else lw.llama_ltnn)(base, cfg, 3)
+    image = open(base, "rb").read()
+    rng = np.random.default_rng(17)
+    head = min(len(image), 8192)
+    opened = 0
+    for it in range(400):
+        m = bytearray(image)
+        how = it % 5
+        if how == 0:
+            m = m[:int(rng.integers(0, len(m) + 1))]
+        elif how == 1:
+            m = m[:int(rng.integers(0, head + 1))]
+        elif how == 2:
+            for _ in range(int(rng.integers(1, 9))):
+                m[int(rng.integers(0, head))] = int(rng.integers(0, 256))
+        elif how == 3:
+            at = int(rng.integers(0, head - 8))
+            value = (1 << 64) - 1 if it % 4 == 0 else int(rng.integers(0, 1 << 62)) >> int(rng.integers(0, 62))
+            m[at:at + 8] = value.to_bytes(8, "little")
+        else:
+            for _ in range(int(rng.integers(1, 5))):
+                m[int(rng.integers(0, len(m)))] ^= 1 << int(rng.integers(0, 8))
+        p = tmp_path / "mutant.bin"
+        p.write_bytes(bytes(m))
+        try:
+            with GGUFFile(p) as f:
+                opened += 1
+                for i in range(f.tensor_count):
+                    try:
+                        t = f.tensor(i)
+                        assert len(f.payload(i)) == t.bytes
+                    except (LiteNNHipError, UnicodeDecodeError):
+                        pass
+                for i in range(f.metadata_count):
+                    raw_key = _lib.load().litenn_gguf_metadata_key(f._h, i)
+                    try:
+                        key = raw_key.decode()
+                    except UnicodeDecodeError:
+                        continue
+                    for get in (f.get_size, f.get_double, f.get_string, f.get_bool, f.get_array_info):
+                        try:
+                            get(key)
+                        except (LiteNNHipError, UnicodeDecodeError):
+                            pass
+                try:
+                    f.llama_params()
+                except LiteNNHipError:
+                    pass
+        except LiteNNHipError:
+            pass
+    assert 0 < opened < 400
