@@ -228,12 +228,27 @@ namespace litenn_hip
 		template <> struct IsInt<uint8_t> { static constexpr bool value = true; };
 		template <> struct IsInt<bool> { static constexpr bool value = true; };
 
+		// The float a Float16 / BFloat16 constructor receives: integers convert to float in one
+		// rounding (a detour through double would round an Int64 beyond 2^53 twice).
+		template <typename S>
+		__device__ __forceinline__ float load_as_float(const S* p, size_t i)
+		{
+			if constexpr (IsInt<S>::value)
+			{
+				return static_cast<float>(p[i]);
+			}
+			else
+			{
+				return static_cast<float>(load_as_double<S>(p, i));
+			}
+		}
+
 		// static_cast<Dst>(src) for every pair, with LiteNN's own Float16 / BFloat16 constructors
 		// (via float; DType.h:63-110, :136-141).
 		template <typename S, typename D>
 		__device__ __forceinline__ void convert_one(const S* src, D* dst, size_t i)
 		{
-			if constexpr (IsInt<S>::value && IsInt<D>::value)
+			if constexpr (IsInt<S>::value)
 			{
 				dst[i] = static_cast<D>(src[i]);
 			}
@@ -245,12 +260,12 @@ namespace litenn_hip
 		template <typename S>
 		__device__ __forceinline__ void convert_one(const S* src, F16* dst, size_t i)
 		{
-			dst[i].bits = f32_to_f16_bits_litenn(static_cast<float>(load_as_double<S>(src, i)));
+			dst[i].bits = f32_to_f16_bits_litenn(load_as_float<S>(src, i));
 		}
 		template <typename S>
 		__device__ __forceinline__ void convert_one(const S* src, BF16* dst, size_t i)
 		{
-			const uint32_t bits = __float_as_uint(static_cast<float>(load_as_double<S>(src, i)));
+			const uint32_t bits = __float_as_uint(load_as_float<S>(src, i));
 			const uint32_t lsb = (bits >> 16) & 1u;
 			dst[i].bits = static_cast<uint16_t>((bits + 0x7fffu + lsb) >> 16);
 		}
@@ -354,6 +369,10 @@ extern "C" int litenn_hip_alloc(int dev, int dtype, size_t n, void** out)
 	{
 		return fail("HIP allocate", "bad dtype or null output pointer");
 	}
+	if (n > SIZE_MAX / es)
+	{
+		return fail("HIP allocate", "element count overflows the byte size");
+	}
 	GUARD("HIP allocate", dev);
 	*out = nullptr;
 	// zero-element tensors still get a distinct, freeable pointer
@@ -385,6 +404,10 @@ extern "C" int litenn_hip_zero(int dev, void* ptr, int dtype, size_t n)
 	{
 		return 0;
 	}
+	if (!ptr)
+	{
+		return fail("HIP zero fill", "null operand");
+	}
 	GUARD("HIP zero fill", dev);
 	LITENN_HIP_TRY("HIP zero fill", hipMemset(ptr, 0, n * es));
 	return 0;
@@ -396,6 +419,10 @@ extern "C" int litenn_hip_convert(int dev, int src_dtype, const void* src, size_
 	if (dtype_size(src_dtype) == 0 || dtype_size(dst_dtype) == 0)
 	{
 		return fail("HIP convert", "bad dtype");
+	}
+	if (n && (!src || !dst))
+	{
+		return fail("HIP convert", "null operand");
 	}
 	GUARD("HIP convert", dev);
 	if (src_dtype == dst_dtype)
@@ -423,6 +450,10 @@ extern "C" int litenn_hip_copy_to_host(int dev, int src_dtype, const void* src, 
 	if (n == 0)
 	{
 		return 0;
+	}
+	if (!src || !dst)
+	{
+		return fail("HIP copy to host", "null operand");
 	}
 	GUARD("HIP copy to host", dev);
 	hipStream_t s = stream_of(opts);
@@ -462,6 +493,10 @@ extern "C" int litenn_hip_copy_from_host(int dev, int dst_dtype, void* dst, int 
 	if (n == 0)
 	{
 		return 0;
+	}
+	if (!src || !dst)
+	{
+		return fail("HIP copy from host", "null operand");
 	}
 	GUARD("HIP copy from host", dev);
 	hipStream_t s = stream_of(opts);
@@ -673,6 +708,10 @@ extern "C" int litenn_hip_dequantize(int dev, int fmt, const void* wq, size_t ro
 	{
 		return fail(action, "dimension exceeds 2^31-1");
 	}
+	if (!wq || !dst)
+	{
+		return fail(action, "null operand");
+	}
 	GUARD(action, dev);
 	launch_dequantize(fmt, wq, rows, k, static_cast<float*>(dst), stream_of(opts));
 	return finish(action, opts);
@@ -693,6 +732,10 @@ extern "C" int litenn_hip_get_rows_q(int dev, int fmt, const void* table, size_t
 	if (k > 0x7fffffffu || rows > 0x7fffffffu || n_ids > 0x7fffffffu)
 	{
 		return fail(action, "dimension exceeds 2^31-1");
+	}
+	if (!table || !ids || !out)
+	{
+		return fail(action, "null operand");
 	}
 	GUARD(action, dev);
 	hipStream_t s = stream_of(opts);
@@ -739,6 +782,10 @@ extern "C" int litenn_hip_rmsnorm(int dev, const void* x, const void* w, double 
 	{
 		return fail(action, "dimension exceeds 2^31-1");
 	}
+	if (!x || !y) // w may be null: a norm without a weight
+	{
+		return fail(action, "null operand");
+	}
 	GUARD(action, dev);
 	launch_rmsnorm(static_cast<const float*>(x), static_cast<const float*>(w), eps, m, d, static_cast<float*>(y),
 	               stream_of(opts));
@@ -769,6 +816,10 @@ extern "C" int litenn_hip_rope_interleaved(int dev, const void* x, void* y, size
 	if (m * n_heads * head_dim > 0x7fffffffu)
 	{
 		return fail(action, "tensor too large");
+	}
+	if (!x || !y)
+	{
+		return fail(action, "null operand");
 	}
 	GUARD(action, dev);
 	hipStream_t s = stream_of(opts);
@@ -810,6 +861,10 @@ extern "C" int litenn_hip_kv_append(int dev, void* cache, int cache_dtype, size_
 	{
 		return 0;
 	}
+	if (!cache || !cur)
+	{
+		return fail(action, "null operand");
+	}
 	GUARD(action, dev);
 	launch_kv_append(cache, cache_dtype, past * width, static_cast<const float*>(cur), m * width, stream_of(opts));
 	return finish(action, opts);
@@ -843,6 +898,10 @@ static int attn_rows_impl(int dev, const void* q, const void* kcache, const void
 	if (m > 65535 || n_head > 65535)
 	{
 		return fail(action, "too many query rows or heads");
+	}
+	if (!q || !kcache || !vcache || !out)
+	{
+		return fail(action, "null operand");
 	}
 	GUARD(action, dev);
 	if (matrix_cores && m >= 16 &&
@@ -907,6 +966,10 @@ extern "C" int litenn_hip_silu_mul(int dev, const void* gate, const void* up, vo
 	{
 		return 0;
 	}
+	if (!gate || !up || !y)
+	{
+		return fail(action, "null operand");
+	}
 	GUARD(action, dev);
 	launch_silu_mul(static_cast<const float*>(gate), static_cast<const float*>(up), static_cast<float*>(y), n,
 	                stream_of(opts));
@@ -924,6 +987,10 @@ extern "C" int litenn_hip_argmax(int dev, const void* x, size_t rows, size_t n, 
 	if (n == 0 || n > 0x7fffffffu)
 	{
 		return fail(action, "row length must be in [1, 2^31-1]");
+	}
+	if (!x || !out_index)
+	{
+		return fail(action, "null operand");
 	}
 	GUARD(action, dev);
 	launch_argmax(static_cast<const float*>(x), rows, n, static_cast<int32_t*>(out_index), stream_of(opts));

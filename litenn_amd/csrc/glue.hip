@@ -72,12 +72,15 @@ namespace litenn_hip
 			sin_t[idx] = static_cast<float>(sin(angle));
 		}
 
-		// f32 rotation with separately rounded products (RoPE.h:93-111): the fused forms are
-		// avoided on purpose so the four multiplies round like the reference's Multiply nodes.
+		// f32 rotation with separately rounded products (RoPE.h:93-111), so the four multiplies
+		// round like the reference's Multiply nodes.  The pragma is what keeps them apart: the
+		// compiler contracts a * c - b * s into a fused multiply-add by default.
 		__device__ __forceinline__ void rotate(float a, float b, float c, float s, float& o0, float& o1)
 		{
-			o0 = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, s));
-			o1 = __fadd_rn(__fmul_rn(a, s), __fmul_rn(b, c));
+#pragma clang fp contract(off)
+			const float ac = a * c, bs = b * s, as = a * s, bc = b * c;
+			o0 = ac - bs;
+			o1 = as + bc;
 		}
 
 		// x,y [m, n_heads, head_dim]; tables indexed by row (positions start at the table's origin)

@@ -8,6 +8,7 @@
 // run sequentially along the reduced axis).
 #include "common.hpp"
 
+#include <type_traits>
 #include <vector>
 
 namespace litenn_hip
@@ -112,7 +113,17 @@ namespace litenn_hip
 			case LITENN_BIN_SUBTRACT: return a - b;
 			case LITENN_BIN_MULTIPLY: return a * b;
 			case LITENN_BIN_DIVIDE: return a / b;
-			case LITENN_BIN_POW: return static_cast<T>(pow(static_cast<double>(a), static_cast<double>(b)));
+			case LITENN_BIN_POW: {
+				const double p = pow(static_cast<double>(a), static_cast<double>(b));
+				if constexpr (std::is_integral<T>::value)
+				{
+					// std::pow(int, int) on the host returns the exact integer for a non-negative
+					// exponent (while it fits a double); the device routine may land one unit in
+					// the last place below it, which the cast would turn into the next integer down
+					return static_cast<T>(b >= T(0) ? rint(p) : p);
+				}
+				return static_cast<T>(p);
+			}
 			case LITENN_BIN_MAX: return a < b ? b : a; // std::max(a, b)
 			case LITENN_BIN_MIN: return b < a ? b : a; // std::min(a, b)
 			default: return a;
@@ -166,17 +177,15 @@ namespace litenn_hip
 		// ---------------- MatMul: bit-for-bit the i-k-j loop of Device.h:645-658 --------------
 		// One thread per output element; k ascends; multiply and add round separately, so the
 		// result equals the host loop exactly.  A and B tiles are staged through LDS.
+		// The compiler contracts a * b + c into a fused multiply-add by default, also through the
+		// *_rn intrinsics (they are plain operators here); the pragma keeps the two roundings of
+		// the host loop (x86-64 without FMA).
 		template <typename T>
-		__device__ __forceinline__ T mul_then_add(T acc, T a, T b) { return acc + a * b; }
-		template <>
-		__device__ __forceinline__ float mul_then_add<float>(float acc, float a, float b)
+		__device__ __forceinline__ T mul_then_add(T acc, T a, T b)
 		{
-			return __fadd_rn(acc, __fmul_rn(a, b));
-		}
-		template <>
-		__device__ __forceinline__ double mul_then_add<double>(double acc, double a, double b)
-		{
-			return __dadd_rn(acc, __dmul_rn(a, b));
+#pragma clang fp contract(off)
+			const T product = a * b;
+			return acc + product;
 		}
 
 		template <typename T>
@@ -330,6 +339,10 @@ extern "C" int litenn_hip_permute(int dev, void* dst, int dtype, const size_t* s
                                   const size_t* perm, const litenn_hip_exec* opts)
 {
 	const char* action = "HIP permute";
+	if ((rank && (!src_shape || !perm)))
+	{
+		return fail(action, "null shape");
+	}
 	const size_t es = dtype_size(dtype);
 	if (es == 0)
 	{
@@ -352,6 +365,10 @@ extern "C" int litenn_hip_permute(int dev, void* dst, int dtype, const size_t* s
 	if (total == 0)
 	{
 		return 0;
+	}
+	if (!dst || !src || !perm)
+	{
+		return fail(action, "null operand");
 	}
 	GUARD(action, dev);
 	hipStream_t s = stream_of(opts);
@@ -384,6 +401,10 @@ extern "C" int litenn_hip_unary(int dev, int op, void* dst, int dtype, const siz
                                 const void* src, const litenn_hip_exec* opts)
 {
 	const char* action = "HIP unary op";
+	if ((rank && !shape))
+	{
+		return fail(action, "null shape");
+	}
 	if (dtype_size(dtype) == 0)
 	{
 		return fail(action, "bad dtype");
@@ -408,6 +429,10 @@ extern "C" int litenn_hip_unary(int dev, int op, void* dst, int dtype, const siz
 		{
 			return 0;
 		}
+		if (!dst || !src)
+		{
+			return fail(action, "null operand");
+		}
 		GUARD(action, dev);
 		logical_not_kernel<<<grid_for(n), 256, 0, stream_of(opts)>>>(static_cast<const bool*>(src),
 		                                                              static_cast<bool*>(dst), n);
@@ -424,6 +449,10 @@ extern "C" int litenn_hip_unary(int dev, int op, void* dst, int dtype, const siz
 	if (n == 0)
 	{
 		return 0;
+	}
+	if (!dst || !src)
+	{
+		return fail(action, "null operand");
 	}
 	GUARD(action, dev);
 	hipStream_t s = stream_of(opts);
@@ -443,6 +472,10 @@ extern "C" int litenn_hip_binary(int dev, int op, void* dst, int dtype1, const s
                                  const litenn_hip_exec* opts)
 {
 	const char* action = "HIP binary op";
+	if (((rank1 && !shape1) || (rank2 && !shape2)))
+	{
+		return fail(action, "null shape");
+	}
 	if (dtype1 != dtype2)
 	{
 		return fail(action, op == LITENN_BIN_MATMUL ? "MatMul requires both inputs to have the same data type"
@@ -474,6 +507,10 @@ extern "C" int litenn_hip_binary(int dev, int op, void* dst, int dtype1, const s
 		if (m == 0 || n == 0)
 		{
 			return 0;
+		}
+		if (!dst || !src1 || !src2)
+		{
+			return fail(action, "null operand");
 		}
 		GUARD(action, dev);
 		hipStream_t s = stream_of(opts);
@@ -553,6 +590,10 @@ extern "C" int litenn_hip_binary(int dev, int op, void* dst, int dtype1, const s
 	{
 		return 0;
 	}
+	if (!dst || !src1 || !src2)
+	{
+		return fail(action, "null operand");
+	}
 	GUARD(action, dev);
 	hipStream_t s = stream_of(opts);
 	const bool compare = op >= LITENN_BIN_LESS;
@@ -584,6 +625,10 @@ extern "C" int litenn_hip_reduce(int dev, int op, void* dst, int dtype, const si
                                  const void* src, size_t axis, const litenn_hip_exec* opts)
 {
 	const char* action = "HIP reduce op";
+	if ((rank && !shape))
+	{
+		return fail(action, "null shape");
+	}
 	if (axis >= rank)
 	{
 		return fail(action, "ReduceOp axis out of range");
@@ -605,6 +650,10 @@ extern "C" int litenn_hip_reduce(int dev, int op, void* dst, int dtype, const si
 	{
 		return fail(action, "cannot reduce over an empty axis");
 	}
+	if (!dst || !src)
+	{
+		return fail(action, "null operand");
+	}
 	GUARD(action, dev);
 	hipStream_t s = stream_of(opts);
 	const bool ok = dispatch_numeric(dtype, [&](auto tag) {
@@ -623,6 +672,10 @@ extern "C" int litenn_hip_concat(int dev, void* dst, int dtype, const void* cons
                                  size_t rank, size_t input_count, size_t axis, const litenn_hip_exec* opts)
 {
 	const char* action = "HIP concat";
+	if ((rank && input_count && !shapes) || !srcs)
+	{
+		return fail(action, "null shape");
+	}
 	const size_t es = dtype_size(dtype);
 	if (es == 0)
 	{
@@ -648,6 +701,17 @@ extern "C" int litenn_hip_concat(int dev, void* dst, int dtype, const void* cons
 	{
 		total_axis += shapes[i * rank + axis];
 	}
+	if (!dst)
+	{
+		return fail(action, "null operand");
+	}
+	for (size_t i = 0; i < input_count; ++i)
+	{
+		if (!srcs[i] && outer * inner * shapes[i * rank + axis] != 0)
+		{
+			return fail(action, "null operand");
+		}
+	}
 	GUARD(action, dev);
 	hipStream_t s = stream_of(opts);
 	size_t axis_off = 0;
@@ -669,6 +733,10 @@ extern "C" int litenn_hip_slice(int dev, void* dst, int dtype, const size_t* src
                                 size_t axis, size_t start, size_t length, const litenn_hip_exec* opts)
 {
 	const char* action = "HIP slice";
+	if ((rank && !src_shape))
+	{
+		return fail(action, "null shape");
+	}
 	const size_t es = dtype_size(dtype);
 	if (es == 0)
 	{
@@ -684,6 +752,10 @@ extern "C" int litenn_hip_slice(int dev, void* dst, int dtype, const size_t* src
 	{
 		return 0;
 	}
+	if (!dst || !src)
+	{
+		return fail(action, "null operand");
+	}
 	GUARD(action, dev);
 	chunk_copy_kernel<<<grid_for(outer * chunk), 256, 0, stream_of(opts)>>>(
 	    static_cast<const uint8_t*>(src) + start * inner * es, static_cast<uint8_t*>(dst), outer, chunk,
@@ -696,6 +768,10 @@ extern "C" int litenn_hip_get_rows(int dev, void* dst, int dtype, const size_t* 
                                    const void* indices, const litenn_hip_exec* opts)
 {
 	const char* action = "HIP GetRows";
+	if (((data_rank && !data_shape) || (index_rank && !index_shape)))
+	{
+		return fail(action, "null shape");
+	}
 	const size_t es = dtype_size(dtype);
 	if (es == 0)
 	{
@@ -714,6 +790,14 @@ extern "C" int litenn_hip_get_rows(int dev, void* dst, int dtype, const size_t* 
 	if (n_idx == 0)
 	{
 		return 0;
+	}
+	if (n_idx > 0x7fffffffu)
+	{
+		return fail(action, "index count exceeds 2^31-1");
+	}
+	if (!dst || !data || !indices)
+	{
+		return fail(action, "null operand");
 	}
 	GUARD(action, dev);
 	hipStream_t s = stream_of(opts);

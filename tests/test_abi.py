@@ -42,3 +42,41 @@ def test_device_count_never_fails_and_errors_are_reported_without_a_device():
     assert b"block size" in lib.litenn_hip_last_error()
     assert lib.litenn_hip_mul_mat_q(0, 6, None, 4, 32, None, 0, 1, None, None, 0, None) != 0  # Q8_1: no dequantizer
     assert b"unsupported block format" in lib.litenn_hip_last_error()
+
+
+def test_null_operands_are_refused_before_any_device_work():
+    """A null data or shape pointer with work to do is an error return, never a launch."""
+    lib = _lib.load()
+    sz = ctypes.c_size_t
+    shape = (sz * 2)(4, 8)
+    one = ctypes.c_void_p(256)  # never dereferenced on the host: every call below fails in validation
+    ptrs = (ctypes.c_void_p * 2)(None, None)
+    calls = [
+        lambda: lib.litenn_hip_zero(0, None, 0, 16),
+        lambda: lib.litenn_hip_convert(0, 0, None, 16, 5, one, None),
+        lambda: lib.litenn_hip_copy_to_host(0, 0, None, 16, 0, one, None),
+        lambda: lib.litenn_hip_copy_from_host(0, 0, one, 0, None, 16, None),
+        lambda: lib.litenn_hip_unary(0, 0, None, 0, shape, 2, one, None),
+        lambda: lib.litenn_hip_unary(0, 0, one, 0, None, 2, one, None),
+        lambda: lib.litenn_hip_binary(0, 0, one, 0, shape, 2, None, 0, shape, 2, one, None),
+        lambda: lib.litenn_hip_reduce(0, 0, one, 0, shape, 2, None, 1, None),
+        lambda: lib.litenn_hip_concat(0, one, 0, ptrs, shape, 2, 1, 0, None),
+        lambda: lib.litenn_hip_slice(0, None, 0, shape, 2, one, 0, 0, 2, None),
+        lambda: lib.litenn_hip_get_rows(0, one, 0, shape, 2, one, 2, shape, 1, None, None),
+        lambda: lib.litenn_hip_permute(0, one, 0, shape, 2, one, None, None),
+        lambda: lib.litenn_hip_mul_mat_q(0, 9, None, 4, 256, one, 0, 1, one, None, 0, None),
+        lambda: lib.litenn_hip_dequantize(0, 9, None, 4, 256, one, None),
+        lambda: lib.litenn_hip_get_rows_q(0, 9, one, 4, 256, None, 1, one, None),
+        lambda: lib.litenn_hip_rmsnorm(0, None, one, 1e-5, 1, 64, one, None),
+        lambda: lib.litenn_hip_rope_interleaved(0, None, one, 1, 1, 64, 64, 1e4, 1.0, 0, None),
+        lambda: lib.litenn_hip_kv_append(0, None, 5, 0, one, 1, 64, None),
+        lambda: lib.litenn_hip_attn_decode(0, one, None, one, 5, 1, 3, 2, 2, 64, one, None),
+        lambda: lib.litenn_hip_attn_rows(0, one, one, one, 5, 16, 0, 2, 2, 128, None, 0, None),
+        lambda: lib.litenn_hip_silu_mul(0, one, None, one, 8, None),
+        lambda: lib.litenn_hip_argmax(0, None, 1, 8, one, None),
+    ]
+    for i, call in enumerate(calls):
+        assert call() != 0, i
+        assert b"null" in lib.litenn_hip_last_error(), (i, lib.litenn_hip_last_error())
+    assert lib.litenn_hip_alloc(0, 1, (1 << 63), ctypes.byref(ctypes.c_void_p())) != 0
+    assert b"overflows" in lib.litenn_hip_last_error()
