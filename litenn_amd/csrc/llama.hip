@@ -503,7 +503,10 @@ extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* p
 		litenn_hip_llama_free(m);
 		return fail_hip(kAction, e);
 	};
-	hipError_t e = hipStreamCreate(&m->stream);
+	// Non-blocking: a stream that synchronises with the legacy default stream would, while its
+	// decode step is being captured, make every default-stream call of another host thread fail
+	// ("would make the legacy stream depend on a capturing blocking stream").
+	hipError_t e = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking);
 	if (e != hipSuccess)
 	{
 		m->stream = nullptr;
@@ -544,9 +547,9 @@ extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* p
 	if ((e = hipMalloc(reinterpret_cast<void**>(&m->d_counters), 2 * sizeof(int))) != hipSuccess ||
 	    (e = hipMalloc(reinterpret_cast<void**>(&m->d_err), sizeof(int))) != hipSuccess ||
 	    (e = hipMalloc(reinterpret_cast<void**>(&m->d_next), sizeof(int32_t))) != hipSuccess ||
-	    (e = hipMemset(m->d_counters, 0, 2 * sizeof(int))) != hipSuccess ||
-	    (e = hipMemset(m->d_err, 0, sizeof(int))) != hipSuccess ||
-	    (e = hipMemset(m->d_next, 0, sizeof(int32_t))) != hipSuccess)
+	    (e = hipMemsetAsync(m->d_counters, 0, 2 * sizeof(int), m->stream)) != hipSuccess ||
+	    (e = hipMemsetAsync(m->d_err, 0, sizeof(int), m->stream)) != hipSuccess ||
+	    (e = hipMemsetAsync(m->d_next, 0, sizeof(int32_t), m->stream)) != hipSuccess)
 	{
 		return bail(e);
 	}
@@ -561,7 +564,7 @@ extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* p
 		const size_t floats = attn_partial_floats(1, heads, static_cast<size_t>(head_dim), m->attn_splits);
 		if ((e = hipMalloc(reinterpret_cast<void**>(&m->attn_partial), sizeof(float) * floats)) != hipSuccess ||
 		    (e = hipMalloc(reinterpret_cast<void**>(&m->attn_counters), sizeof(int) * heads)) != hipSuccess ||
-		    (e = hipMemset(m->attn_counters, 0, sizeof(int) * heads)) != hipSuccess)
+		    (e = hipMemsetAsync(m->attn_counters, 0, sizeof(int) * heads, m->stream)) != hipSuccess)
 		{
 			return bail(e);
 		}
