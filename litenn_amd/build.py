@@ -54,7 +54,8 @@ def build(verbose: bool = True, jobs: int = 6) -> str:
             print(out)
     if failed:
         raise RuntimeError("hipcc failed")
-    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", LIB_PATH]
+    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc",
+           "-Wl,--version-script=" + os.path.join(CSRC, "exports.map"), *objs, "-o", LIB_PATH]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)

@@ -965,7 +965,10 @@ extern "C" int litenn_gguf_llama_params(const litenn_gguf* g, litenn_hip_llama_p
 
 // ---- loader: GGUF file -> resident decoder -----------------------------------------------------
 
-extern "C" int litenn_hip_llama_adopt(litenn_hip_llama* model, void* device_ptr); // llama.hip: frees it with the model
+namespace litenn_hip
+{
+	int llama_adopt(litenn_hip_llama* model, void* device_ptr); // llama.hip: frees it with the model
+}
 
 namespace
 {
@@ -1033,7 +1036,7 @@ namespace
 		{
 			return 1;
 		}
-		if (litenn_hip_llama_adopt(model, dptr) != 0)
+		if (litenn_hip::llama_adopt(model, dptr) != 0)
 		{
 			(void)hipFree(dptr);
 			return 1;

@@ -573,16 +573,20 @@ extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* p
 	return 0;
 }
 
-// Hands a device allocation to the model: it is released by litenn_hip_llama_free.
-extern "C" int litenn_hip_llama_adopt(litenn_hip_llama* m, void* device_ptr)
+// Hands a device allocation to the model: it is released by litenn_hip_llama_free.  Used by
+// the GGUF loader; not part of the C ABI.
+namespace litenn_hip
 {
-	if (!m || !device_ptr)
+	int llama_adopt(litenn_hip_llama* m, void* device_ptr)
 	{
-		return fail(kAction, "null argument");
+		if (!m || !device_ptr)
+		{
+			return fail(kAction, "null argument");
+		}
+		m->owned.push_back(device_ptr);
+		return 0;
 	}
-	m->owned.push_back(device_ptr);
-	return 0;
-}
+} // namespace litenn_hip
 
 extern "C" int litenn_hip_llama_free(litenn_hip_llama* m)
 {
