@@ -123,7 +123,9 @@ int litenn_hip_permute(int dev, void* dst, int dtype, const size_t* src_shape, s
 /* y[m, n] (f32) = x[m, k] . deq(wq)[n, k]^T with f32 accumulation, i.e. the value
  * AddLinear produces after the lowering's dequantise + transpose
  * (tools/gguf/LLaMABuilder.cpp:144-150,225-230; src/LiteNN/Layer/Linear.h:67-95).
- * wq is the raw GGUF payload: n rows of k/block blocks.  x_dtype is F32.
+ * wq is the raw GGUF payload: n rows of k/block blocks.  x_dtype is F32; F16 and BF16
+ * activations are accepted too and widened exactly into a Float32 copy first (the copy is
+ * allocated and freed by the call, which therefore always synchronises).
  * residual (f32 [m, n]) may be NULL; when given, y = residual + x.W
  * (the Add at tools/gguf/LLaMABuilder.cpp:652-653,661-663).  residual may alias y.
  * m == 1..15 runs the streaming GEMV.  m >= 16 (with k a multiple of 256) runs on the matrix

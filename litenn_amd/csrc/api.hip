@@ -555,9 +555,9 @@ extern "C" int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t 
 	{
 		return fail(action, "unsupported block format");
 	}
-	if (x_dtype != LITENN_F32)
+	if (x_dtype != LITENN_F32 && x_dtype != LITENN_F16 && x_dtype != LITENN_BF16)
 	{
-		return fail(action, "activations must be Float32");
+		return fail(action, "activations must be Float32, Float16 or BFloat16");
 	}
 	if (row_bytes(fmt, k) == 0)
 	{
@@ -581,7 +581,32 @@ extern "C" int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t 
 	}
 	GUARD(action, dev);
 	hipStream_t s = stream_of(opts);
+	// 16-bit activations are widened (exactly) into a Float32 copy that this call owns; the copy
+	// is released after the stream has drained, so such a call always blocks
+	struct Widened
+	{
+		void* p = nullptr;
+		hipStream_t s = nullptr;
+		~Widened()
+		{
+			if (p)
+			{
+				(void)hipStreamSynchronize(s);
+				(void)hipFree(p);
+			}
+		}
+	} widened;
 	const float* xf = static_cast<const float*>(x);
+	if (x_dtype != LITENN_F32)
+	{
+		widened.s = s;
+		LITENN_HIP_TRY(action, hipMalloc(&widened.p, sizeof(float) * m * k));
+		if (!launch_convert(x_dtype, x, m * k, LITENN_F32, widened.p, s))
+		{
+			return fail(action, "activation dtype is not supported on the device");
+		}
+		xf = static_cast<const float*>(widened.p);
+	}
 	float* yf = static_cast<float*>(y);
 	const float* rf = static_cast<const float*>(residual);
 	const bool quant = fmt != LITENN_FMT_F16 && fmt != LITENN_FMT_F32;

@@ -194,3 +194,27 @@ def test_gemv_properties_at_full_size(hip):
         assert np.array_equal(y(e)[0], deq[:, col]), col
     # all-ones input: row sums (f32 summation order differs: tolerance, not equality)
     assert rel_l2(y(np.ones((1, k), np.float32))[0], deq.astype(np.float64).sum(axis=1).astype(np.float32)) <= 1e-5
+
+
+@pytest.mark.parametrize("fmt", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("m", [1, 3, 32])
+def test_sixteen_bit_activations_are_widened_exactly(hip, oracle, fmt, m):
+    """Float16 / BFloat16 activations give what their exact Float32 values give."""
+    from litenn_amd.formats import DT_BF16
+    n, k = 96, 1024
+    wq = synth.quant_weights(fmt, n, k, 5, 1)
+    x = synth.activations(m, k, 5, 2)
+    w = hip.Tensor.from_numpy(wq)
+    half = x.astype(np.float16)
+    want = hip.mul_mat_q(fmt, w, n, k, hip.Tensor.from_numpy(half.astype(np.float32))).numpy()
+    got = hip.mul_mat_q(fmt, w, n, k, hip.Tensor.from_numpy(half)).numpy()
+    assert np.array_equal(got, want)
+    assert rel_l2(got, oracle.mul_mat_q(fmt, wq, n, k, half.astype(np.float32))) <= TOL
+    bits = (x.view(np.uint32) >> 16).astype(np.uint16)  # BFloat16 by truncation: exactly representable
+    bf = hip.Tensor((m, k), DT_BF16)
+    hip.DeviceTraits.CopyFromCPU(bf.device, DT_BF16, bf.ptr, DT_BF16, bits, bits.size)
+    wide = (bits.astype(np.uint32) << 16).view(np.float32)
+    want = hip.mul_mat_q(fmt, w, n, k, hip.Tensor.from_numpy(wide)).numpy()
+    assert np.array_equal(hip.mul_mat_q(fmt, w, n, k, bf).numpy(), want)
+    with pytest.raises(hip.LiteNNHipError, match="Float32, Float16 or BFloat16"):
+        hip.mul_mat_q(fmt, w, n, k, hip.Tensor.from_numpy(np.zeros((1, k), np.float64)))
