@@ -916,8 +916,10 @@ namespace litenn_hip
 			};
 
 			// ---- weight requests: piece p = 64 i + lane of the slot is piece p % P of row p / P; a
-			// row's pieces start at the 16-byte boundary at or below its chunk.  Rows past the end
-			// re-read the last row; their results are never stored.
+			// row's pieces start at the 16-byte boundary at or below its chunk (an aligned piece that
+			// holds a byte of the tensor lies in that byte's page, so nothing outside the tensor's
+			// pages is touched).  Rows past the end re-read the last row; their results are never
+			// stored.
 			const uint8_t* w_src[kWLoads]; // the row's chunk 0
 			int w_piece[kWLoads];          // 16 j
 #pragma unroll
@@ -935,8 +937,18 @@ namespace litenn_hip
 					if (64 * (i + 1) <= NG * 16 * P || 64 * i + lane < NG * 16 * P)
 					{
 						const uintptr_t chunk = reinterpret_cast<uintptr_t>(w_src[i] + static_cast<size_t>(c) * F::kChunkBytes);
-						const uint8_t* src =
-						    reinterpret_cast<const uint8_t*>((F::kAligned16 ? chunk : (chunk & ~uintptr_t{ 15 })) + w_piece[i]);
+						uintptr_t from = chunk + w_piece[i];
+						if constexpr (!F::kAligned16)
+						{
+							// P counts the pieces of the worst misalignment; with a smaller one the last
+							// piece holds no byte of this chunk, and behind the tensor's last chunk it
+							// can be the first 16 bytes of a page that is not mapped.  Such a piece
+							// fetches the chunk's first piece again (its slot bytes are never read).
+							const uintptr_t base = chunk & ~uintptr_t{ 15 };
+							from = base + w_piece[i];
+							from = from >= chunk + F::kChunkBytes ? base : from;
+						}
+						const uint8_t* src = reinterpret_cast<const uint8_t*>(from);
 						const uint32_t dst = slot_lds + i * 1024;
 						asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
 						             :

@@ -173,3 +173,18 @@ def test_prefill_through_the_matrix_cores(hip, oracle, fmt):
     # go row by row through the GEMV
     for lo, hi in ((36, 40), (40, 47), (47, 49)):
         assert rel_l2(dev.eval(toks[lo:hi], precise=False), ref.eval(toks[lo:hi])) < 5e-3
+
+
+@pytest.mark.parametrize("fmt,n,k", [(Q2_K, 512, 512), (Q3_K, 1024, 512), (Q6_K, 1024, 512), (Q2_K, 1024, 256)])
+def test_weights_that_end_on_a_page_boundary(hip, oracle, fmt, n, k):
+    """Blocks of 84, 110 and 210 bytes are fetched as 16-byte pieces from the boundary below them;
+    no piece may lie wholly behind the tensor, where the next page need not be mapped (these
+    tensors are a whole number of 4 KB pages)."""
+    from litenn_amd.formats import row_bytes
+    assert (n * row_bytes(fmt, k)) % 4096 == 0
+    wq = synth.quant_weights(fmt, n, k, 9, 1)
+    w = hip.Tensor.from_numpy(wq)
+    for m in (16, 40):
+        x = synth.activations(m, k, 9, m)
+        y = hip.mul_mat_q(fmt, w, n, k, hip.Tensor.from_numpy(x)).numpy()
+        assert rel_l2(y, oracle.mul_mat_q(fmt, wq, n, k, x)) <= 1e-3

