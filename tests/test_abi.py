@@ -80,3 +80,16 @@ def test_null_operands_are_refused_before_any_device_work():
         assert b"null" in lib.litenn_hip_last_error(), (i, lib.litenn_hip_last_error())
     assert lib.litenn_hip_alloc(0, 1, (1 << 63), ctypes.byref(ctypes.c_void_p())) != 0
     assert b"overflows" in lib.litenn_hip_last_error()
+
+
+def test_nothing_but_the_declared_entry_points_is_exported():
+    """The dynamic symbol table holds the header's functions only (linker version script)."""
+    import shutil
+    import subprocess
+    import pytest
+    nm = shutil.which("nm")
+    if nm is None:
+        pytest.skip("nm is not installed")
+    out = subprocess.run([nm, "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = sorted(line.split()[-1] for line in out.splitlines() if line.split()[-2:-1] and line.split()[-2] in "TDBR")
+    assert exported == declared_symbols(), sorted(set(exported) ^ set(declared_symbols()))
