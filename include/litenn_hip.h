@@ -191,6 +191,21 @@ int litenn_hip_kv_append(int dev, void* cache, int cache_dtype, size_t past, con
 int litenn_hip_attn_decode(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
                            size_t past, size_t n_head, size_t n_kv_head, size_t head_dim, void* out,
                            const litenn_hip_exec* opts);
+/* litenn_hip_attn_decode for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): same operands and the same
+ * result, bit for bit, but the chunk triples and arrival counters that a single row against a
+ * long cache needs live in a fixed array of 1 MiB + 4 KiB inside the library's code object (one copy per
+ * GPU, held until the process ends) instead of memory allocated and freed by the call.  No
+ * counterpart in the reference.  The call allocates nothing, records no memset node, and honours
+ * opts->synchronize like every other entry point.  It refuses a launch whose chunks do not fit:
+ * a single row (m == 1) is cut into c = min(16, ceil(keys / 64), ceil(1024 / n_head)) chunks and
+ * needs n_head * c * (head_dim + 2) <= 262144 floats, which holds for every head_dim <= 128 and
+ * e.g. for 48 heads of 256 features but not for 64.  Every call on one GPU shares that GPU's array:
+ * calls that overlap on one GPU (two streams, two threads) race and must be serialised by the
+ * caller. */
+int litenn_hip_attn_decode_noalloc(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype,
+                                   size_t m, size_t past, size_t n_head, size_t n_kv_head, size_t head_dim, void* out,
+                                   const litenn_hip_exec* opts);
 /* The same attention for a prompt's rows (the multi-row lowering of
  * tools/gguf/LLaMABuilder.cpp:350-404,502-557; mask of src/LiteNN/Layer/CausalMask.h:16-56):
  * with m >= 16, an F16 cache, 128-wide heads and 16-byte aligned buffers both contractions

@@ -67,6 +67,7 @@ SIGNATURES = {
     "litenn_hip_rope_interleaved": [_i, _vp, _vp, _sz, _sz, _sz, _sz, _d, _d, _sz, _ex],
     "litenn_hip_kv_append": [_i, _vp, _i, _sz, _vp, _sz, _sz, _ex],
     "litenn_hip_attn_decode": [_i, _vp, _vp, _vp, _i, _sz, _sz, _sz, _sz, _sz, _vp, _ex],
+    "litenn_hip_attn_decode_noalloc": [_i, _vp, _vp, _vp, _i, _sz, _sz, _sz, _sz, _sz, _vp, _ex],
     "litenn_hip_attn_rows": [_i, _vp, _vp, _vp, _i, _sz, _sz, _sz, _sz, _sz, _vp, _u, _ex],
     "litenn_hip_silu_mul": [_i, _vp, _vp, _vp, _sz, _ex],
     "litenn_hip_argmax": [_i, _vp, _sz, _sz, _vp, _ex],

@@ -38,6 +38,11 @@ namespace litenn_hip
 	void launch_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
 	                        const int* past_dev, size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim,
 	                        float* out, size_t splits, float* partial, int* counters, hipStream_t s);
+	bool attn_static_fits(size_t m, size_t n_head, size_t head_dim, size_t splits);
+	size_t attn_static_scratch_bytes();
+	hipError_t launch_attn_decode_static(const float* q, const void* kcache, const void* vcache, int cache_dtype,
+	                                     size_t m, size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim,
+	                                     float* out, size_t splits, hipStream_t s);
 	void launch_silu_mul(const float* gate, const float* up, float* y, size_t n, hipStream_t s);
 	void launch_argmax(const float* x, size_t rows, size_t n, int32_t* out, hipStream_t s);
 
@@ -895,11 +900,11 @@ extern "C" int litenn_hip_kv_append(int dev, void* cache, int cache_dtype, size_
 	return finish(action, opts);
 }
 
-static int attn_rows_impl(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
-                          size_t past, size_t n_head, size_t n_kv_head, size_t head_dim, void* out, bool matrix_cores,
-                          const litenn_hip_exec* opts)
+// Operand checks shared by the attention entry points; returns 0, a failure status, or -1 when
+// there is nothing to do (m == 0).
+static int attn_check(const char* action, const void* q, const void* kcache, const void* vcache, int cache_dtype,
+                      size_t m, size_t past, size_t n_head, size_t n_kv_head, size_t head_dim, const void* out)
 {
-	const char* action = "HIP attention";
 	if (cache_dtype != LITENN_F16 && cache_dtype != LITENN_F32)
 	{
 		return fail(action, "cache dtype must be Float16 or Float32");
@@ -914,7 +919,7 @@ static int attn_rows_impl(int dev, const void* q, const void* kcache, const void
 	}
 	if (m == 0)
 	{
-		return 0;
+		return -1;
 	}
 	if (past + m > (size_t{ 1 } << 30))
 	{
@@ -927,6 +932,18 @@ static int attn_rows_impl(int dev, const void* q, const void* kcache, const void
 	if (!q || !kcache || !vcache || !out)
 	{
 		return fail(action, "null operand");
+	}
+	return 0;
+}
+
+static int attn_rows_impl(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
+                          size_t past, size_t n_head, size_t n_kv_head, size_t head_dim, void* out, bool matrix_cores,
+                          const litenn_hip_exec* opts)
+{
+	const char* action = "HIP attention";
+	if (const int rc = attn_check(action, q, kcache, vcache, cache_dtype, m, past, n_head, n_kv_head, head_dim, out))
+	{
+		return rc < 0 ? 0 : rc;
 	}
 	GUARD(action, dev);
 	if (matrix_cores && m >= 16 &&
@@ -973,6 +990,29 @@ extern "C" int litenn_hip_attn_decode(int dev, const void* q, const void* kcache
                                       void* out, const litenn_hip_exec* opts)
 {
 	return attn_rows_impl(dev, q, kcache, vcache, cache_dtype, m, past, n_head, n_kv_head, head_dim, out, false, opts);
+}
+
+extern "C" int litenn_hip_attn_decode_noalloc(int dev, const void* q, const void* kcache, const void* vcache,
+                                              int cache_dtype, size_t m, size_t past, size_t n_head, size_t n_kv_head,
+                                              size_t head_dim, void* out, const litenn_hip_exec* opts)
+{
+	const char* action = "HIP attention (no allocation)";
+	if (const int rc = attn_check(action, q, kcache, vcache, cache_dtype, m, past, n_head, n_kv_head, head_dim, out))
+	{
+		return rc < 0 ? 0 : rc;
+	}
+	const size_t splits = attn_splits(m, past + m, n_head);
+	if (!attn_static_fits(m, n_head, head_dim, splits))
+	{
+		return fail(action, "a single row cut into key chunks needs more than the static scratch of " +
+		                        std::to_string(attn_static_scratch_bytes()) +
+		                        " bytes: heads * chunks * (head_dim + 2) must not exceed 262144 floats");
+	}
+	GUARD(action, dev);
+	LITENN_HIP_TRY(action, launch_attn_decode_static(static_cast<const float*>(q), kcache, vcache, cache_dtype, m, past,
+	                                                 n_head, n_kv_head, head_dim, static_cast<float*>(out), splits,
+	                                                 stream_of(opts)));
+	return finish(action, opts);
 }
 
 extern "C" int litenn_hip_attn_rows(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype,

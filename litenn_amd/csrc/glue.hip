@@ -7,10 +7,33 @@
 
 #include <algorithm>
 
+// Scratch of the allocation-free attention entry point (litenn_hip_attn_decode_noalloc): the
+// chunk triples {running maximum, sum, head_dim outputs} of one query row cut into key chunks,
+// followed by one arrival counter per head.  1 MiB of triples: a row is cut into
+// min(16, ceil(1024 / heads)) chunks at most, so heads * chunks < 2048 and every launch with heads
+// of up to 128 features fits; wider heads fit up to heads * chunks * (head_dim + 2) <= 262144
+// (e.g. 48 heads of 256 features, not 64).  Only rows that are cut (m == 1, heads <= 1024) use the
+// array at all.  Every GPU the library runs on holds its own copy (1 MiB + 4 KiB) until the
+// process ends.  Host code never uses the
+// array's name as an address: static_attn_scratch() asks the runtime for the device address once
+// per device and hands that pointer to the launches.
+constexpr size_t kStaticAttnPartialFloats = size_t{ 256 } * 1024;
+constexpr size_t kStaticAttnCounters = 1024;
+static __device__ __align__(256) float scratch[kStaticAttnPartialFloats + kStaticAttnCounters];
+
 namespace litenn_hip
 {
 	namespace
 	{
+		__global__ void zero_ints_kernel(int* p, int n)
+		{
+			const int i = blockIdx.x * blockDim.x + threadIdx.x;
+			if (i < n)
+			{
+				p[i] = 0;
+			}
+		}
+
 		// ---------------- RMSNorm (f64 accumulate, ComputePrimitives.h:792-817) -------------
 		__global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__ x,
 		                                                        const float* __restrict__ w, double eps, int d,
@@ -948,6 +971,80 @@ namespace litenn_hip
 	{
 		launch_attn_any(q, const_cast<void*>(kcache), const_cast<void*>(vcache), cache_dtype, m, past_dev, past_host,
 		                n_head, n_kv_head, head_dim, out, splits, partial, counters, nullptr, s);
+	}
+
+	// Device address of this file's `scratch` array on the CURRENT device, looked up once per device
+	// (each GPU holds its own copy at its own address).  No allocation: the array is part of the
+	// code object.
+	static hipError_t static_attn_scratch(float** base)
+	{
+		constexpr int kMaxDevices = 64;
+		static std::mutex mutex;
+		static float* per_device[kMaxDevices] = {};
+		int dev = 0;
+		hipError_t e = hipGetDevice(&dev);
+		if (e != hipSuccess)
+		{
+			return e;
+		}
+		if (dev < 0 || dev >= kMaxDevices)
+		{
+			return hipErrorInvalidDevice;
+		}
+		std::lock_guard<std::mutex> lock(mutex);
+		if (!per_device[dev])
+		{
+			void* ptr = nullptr;
+			e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+			if (e != hipSuccess)
+			{
+				return e;
+			}
+			if (!ptr)
+			{
+				return hipErrorInvalidSymbol;
+			}
+			per_device[dev] = static_cast<float*>(ptr);
+		}
+		*base = per_device[dev];
+		return hipSuccess;
+	}
+
+	// Whether a launch of that geometry fits the static scratch (always true without chunks).
+	bool attn_static_fits(size_t m, size_t n_head, size_t head_dim, size_t splits)
+	{
+		return splits <= 1 || (attn_partial_floats(m, n_head, head_dim, splits) <= kStaticAttnPartialFloats &&
+		                       m * n_head <= kStaticAttnCounters);
+	}
+
+	size_t attn_static_scratch_bytes() { return sizeof(float) * (kStaticAttnPartialFloats + kStaticAttnCounters); }
+
+	// launch_attn_decode with the chunk triples and counters in the static scratch of the current
+	// device.  The counters are cleared by a small kernel first (not a memset node: a caller may be
+	// capturing), so a launch that was cut short earlier cannot leave a stale count behind.  Calls
+	// that overlap on one GPU share the array and race.
+	hipError_t launch_attn_decode_static(const float* q, const void* kcache, const void* vcache, int cache_dtype,
+	                                     size_t m, size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim,
+	                                     float* out, size_t splits, hipStream_t s)
+	{
+		float* partial = nullptr;
+		int* counters = nullptr;
+		if (splits > 1)
+		{
+			float* base = nullptr;
+			const hipError_t e = static_attn_scratch(&base);
+			if (e != hipSuccess)
+			{
+				return e;
+			}
+			partial = base;
+			counters = reinterpret_cast<int*>(base + kStaticAttnPartialFloats);
+			const int n = static_cast<int>(m * n_head);
+			zero_ints_kernel<<<dim3((n + 255) / 256), dim3(256), 0, s>>>(counters, n);
+		}
+		launch_attn_decode(q, kcache, vcache, cache_dtype, m, nullptr, past_host, n_head, n_kv_head, head_dim, out,
+		                   splits, partial, counters, s);
+		return hipSuccess;
 	}
 
 	// Whether one new row's rotation, cache append and attention can run as a single launch.

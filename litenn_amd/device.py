@@ -263,6 +263,15 @@ def attn_decode(q: Tensor, kcache: Tensor, vcache: Tensor, m: int, past: int, n_
     return out
 
 
+def attn_decode_noalloc(q: Tensor, kcache: Tensor, vcache: Tensor, m: int, past: int, n_head: int, n_kv_head: int,
+                        head_dim: int, out: Tensor) -> Tensor:
+    """attn_decode through the entry point that allocates nothing: the caller brings `out`."""
+    check(_lib.load().litenn_hip_attn_decode_noalloc(q.device.deviceIndex, q.ptr, kcache.ptr, vcache.ptr,
+                                                     kcache.dtype, m, past, n_head, n_kv_head, head_dim, out.ptr,
+                                                     None))
+    return out
+
+
 def attn_rows(q: Tensor, kcache: Tensor, vcache: Tensor, m: int, past: int, n_head: int, n_kv_head: int,
               head_dim: int, precise: bool = False) -> Tensor:
     """attn_decode for a prompt's rows: on the matrix cores when the shape allows and precise is False."""
@@ -288,5 +297,5 @@ def argmax(x: Tensor) -> Tensor:
 
 __all__ = ["HIP", "HIPDeviceCount", "IsHIPDeviceAvailable", "DeviceTraits", "Tensor", "mul_mat_q", "linear_group",
            "dequantize",
-           "get_rows_q", "rmsnorm", "rope_interleaved", "kv_append", "attn_decode", "silu_mul", "argmax",
+           "get_rows_q", "rmsnorm", "rope_interleaved", "kv_append", "attn_decode", "attn_decode_noalloc", "silu_mul", "argmax",
            "MATMUL_PRECISE", "LiteNNHipError", "F32"]
