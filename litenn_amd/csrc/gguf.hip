@@ -239,12 +239,29 @@ namespace
 		return fail(kReadAction, "GGUF metadata key '" + key + "' must be numeric");
 	}
 
-	// Byte size of every tensor from its type and shape, checked against the file
-	int finish_tensors(litenn_gguf* g, const char* what)
+	// Byte size of every tensor from its type and shape, checked against the file.  All arithmetic on
+	// sizes and offsets read from the file is done without wrapping: a product or sum that would not
+	// fit is a tensor that cannot lie inside the file.  `alignment` (0: none) is what every tensor
+	// offset must be a multiple of (ggml refuses a GGUF whose tensor data is not aligned).
+	int finish_tensors(litenn_gguf* g, const char* what, uint64_t alignment)
 	{
 		const std::string kind = what;
+		if (g->data_offset > g->size)
+		{
+			return fail(kReadAction, "Failed to open GGUF file '" + g->path + "'");
+		}
+		const uint64_t data_bytes = g->size - g->data_offset;
 		for (TensorEntry& t : g->tensors)
 		{
+			const TypeInfo* ti = find_type(t.ggml_type);
+			if (!ti)
+			{
+				return fail(kReadAction, "Unsupported ggml tensor type '" + std::to_string(t.ggml_type) + "' for tensor '" +
+				                             t.name + "'");
+			}
+			// no tensor inside the file has more elements than the file has bytes times the elements a
+			// block holds (a block takes at least one byte)
+			const uint64_t element_limit = data_bytes * static_cast<uint64_t>(ti->block_elements) + 1;
 			uint64_t elements = 1;
 			for (uint64_t n : t.ne)
 			{
@@ -252,24 +269,28 @@ namespace
 				{
 					return fail(kReadAction, kind + " tensor '" + t.name + "' has non-positive dimension " + std::to_string(n));
 				}
+				if (elements > element_limit / n)
+				{
+					return fail(kReadAction, "Failed to read the payload of " + kind + " tensor '" + t.name +
+					                             "': its shape holds more elements than the file has room for");
+				}
 				elements *= n;
-			}
-			const TypeInfo* ti = find_type(t.ggml_type);
-			if (!ti)
-			{
-				return fail(kReadAction, "Unsupported ggml tensor type '" + std::to_string(t.ggml_type) + "' for tensor '" +
-				                             t.name + "'");
 			}
 			const uint64_t row = t.ne.empty() ? 1 : t.ne[0];
 			if (row % static_cast<uint64_t>(ti->block_elements) != 0)
 			{
 				return fail(kReadAction, kind + " tensor '" + t.name + "' has an invalid serialized byte size");
 			}
-			t.bytes = elements / ti->block_elements * ti->block_bytes;
-			if (g->data_offset + t.offset + t.bytes > g->size)
+			t.bytes = elements / ti->block_elements * ti->block_bytes; // elements <= data_bytes * block + 1: no wrap
+			if (t.offset > data_bytes || t.bytes > data_bytes - t.offset)
 			{
 				return fail(kReadAction, "Failed to read " + std::to_string(t.bytes) + " bytes for " + kind + " tensor '" +
 				                             t.name + "'");
+			}
+			if (alignment != 0 && t.offset % alignment != 0)
+			{
+				return fail(kReadAction, kind + " tensor '" + t.name + "' has offset " + std::to_string(t.offset) +
+				                             ", which is not a multiple of the alignment " + std::to_string(alignment));
 			}
 		}
 		return 0;
@@ -371,7 +392,7 @@ namespace
 			}
 		}
 		g->data_offset = (c.pos + alignment - 1) / alignment * alignment;
-		return finish_tensors(g, "GGUF");
+		return finish_tensors(g, "GGUF", alignment);
 	}
 
 	// ---- LiteNN model archive (.ltnn) ---------------------------------------------------------
@@ -616,7 +637,7 @@ namespace
 		{
 			payloads.push_back(t.bytes);
 		}
-		if (finish_tensors(g, "LiteNN model") != 0)
+		if (finish_tensors(g, "LiteNN model", 0) != 0)
 		{
 			return 1;
 		}

@@ -198,3 +198,58 @@ def test_mutated_images_are_refused_or_read_never_crash(tmp_path, kind):
         except LiteNNHipError:
             pass
     assert 0 < opened < 400
+
+
+def _raw_gguf(path, tensors, pad_to=0, tail=b""):
+    """A version-3 image with a hand-made tensor directory: tensors = (name, ne fastest first, ggml type id, offset)."""
+    import struct
+    head = struct.pack("<IIQQ", 0x46554747, 3, len(tensors), 0)
+    for name, ne, type_id, offset in tensors:
+        head += struct.pack("<Q", len(name)) + name.encode() + struct.pack("<I", len(ne))
+        for n in ne:
+            head += struct.pack("<Q", n)
+        head += struct.pack("<IQ", type_id, offset)
+    start = (len(head) + 31) // 32 * 32
+    with open(path, "wb") as f:
+        f.write(head + b"\0" * (start - len(head)) + tail + b"\0" * pad_to)
+    return path, start
+
+
+def test_offsets_and_shapes_that_wrap_64_bits_are_refused(tmp_path):
+    """Directory entries whose offset + size, or whose element count, does not fit 64 bits must not
+    pass a bound check through wrap-around (the reference reads through ggml's checked reader)."""
+    data = np.arange(16, dtype=np.float32).tobytes()
+    # one f32[4] tensor at an offset just below 2^64: data_offset + offset + 16 wraps to a small number
+    for offset in (2 ** 64 - 72, 2 ** 64 - 64, 2 ** 64 - 32, 2 ** 63):
+        path, start = _raw_gguf(tmp_path / "wrap.gguf", [("t", (4,), 0, offset)], tail=data)
+        with pytest.raises(LiteNNHipError) as e:
+            GGUFFile(path)
+        assert "Failed to read" in str(e.value), str(e.value)
+    # a 2^32 x 2^32 f32 tensor: the element count wraps to 0
+    path, _ = _raw_gguf(tmp_path / "big.gguf", [("t", (2 ** 32, 2 ** 32), 0, 0)], tail=data)
+    with pytest.raises(LiteNNHipError) as e:
+        GGUFFile(path)
+    assert "more elements than the file has room for" in str(e.value)
+    # four dimensions of 2^40: far past any wrap
+    path, _ = _raw_gguf(tmp_path / "big4.gguf", [("t", (2 ** 40,) * 4, 0, 0)], tail=data)
+    with pytest.raises(LiteNNHipError):
+        GGUFFile(path)
+    # a quantised shape whose element count wraps to a whole number of blocks
+    path, _ = _raw_gguf(tmp_path / "bigq.gguf", [("t", (2 ** 40, 2 ** 24), 12, 0)], tail=data)
+    with pytest.raises(LiteNNHipError):
+        GGUFFile(path)
+    # the honest neighbour still opens: same tensor at offset 32
+    path, start = _raw_gguf(tmp_path / "ok.gguf", [("t", (4,), 0, 32)], tail=b"\0" * 32 + data[:16])
+    with GGUFFile(path) as f:
+        t = f.tensor("t")
+        assert t.file_offset == start + 32 and t.bytes == 16
+        assert np.array_equal(f.payload("t").view(np.float32), np.arange(4, dtype=np.float32))
+
+
+def test_unaligned_tensor_offsets_are_refused(tmp_path):
+    """ggml refuses a file whose tensor data does not start on a multiple of general.alignment."""
+    data = np.arange(16, dtype=np.float32).tobytes()
+    path, _ = _raw_gguf(tmp_path / "unaligned.gguf", [("t", (4,), 0, 8)], tail=data)
+    with pytest.raises(LiteNNHipError) as e:
+        GGUFFile(path)
+    assert "not a multiple of the alignment" in str(e.value)
