@@ -80,6 +80,24 @@ def build_cpp_host_test(verbose: bool = True) -> str:
     return CPP_TEST_BIN
 
 
+FETCH_TEST_SRC = os.path.join(os.path.dirname(HERE), "tests", "cpp", "fetch_bounds_test.cpp")
+FETCH_TEST_BIN = os.path.join(os.path.dirname(HERE), "tests", "cpp", "fetch_bounds_test")
+
+
+def build_fetch_bounds_test(verbose: bool = True) -> str:
+    """Compile the host-side bounds model of the kernels' fetch patterns (plain g++: it includes
+    csrc/fetch_model.hpp, the address arithmetic the kernels themselves call)."""
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if not cxx:
+        raise RuntimeError("g++ not found; the fetch bounds test cannot be built")
+    cmd = [cxx, "-std=c++17", "-O2", "-Wall", FETCH_TEST_SRC, "-o", FETCH_TEST_BIN]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return FETCH_TEST_BIN
+
+
 if __name__ == "__main__":
     build()
     build_cpp_host_test()
+    build_fetch_bounds_test()

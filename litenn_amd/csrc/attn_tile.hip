@@ -26,6 +26,7 @@
 #include <cstdint>
 
 #include "common.hpp"
+#include "fetch_model.hpp"
 
 namespace litenn_hip
 {
@@ -79,8 +80,7 @@ namespace litenn_hip
 			const uint16_t* vbase = vcache + static_cast<size_t>(kvh) * kDim;
 
 			const int q_first = tile * kQTile;
-			const int q_last = min(m, q_first + kQTile) - 1;
-			const int kv_len = past + q_last + 1; // keys any row of this tile may see
+			const int kv_len = fetch::attn_tile_kv_len(past, q_first, kQTile, m); // keys any row of this tile may see
 			const int n_key_tiles = (kv_len + kKeyTile - 1) / kKeyTile;
 			const int n_steps = (n_key_tiles + 1) >> 1; // both halves make the same number of steps
 
@@ -110,10 +110,10 @@ namespace litenn_hip
 				for (int i = 0; i < 4; ++i)
 				{
 					const int c = tid + 256 * i;
-					const int key = min(kt * kKeyTile + (c >> 4), kv_len - 1);
+					const int key = fetch::attn_tile_key(kt, kKeyTile, c >> 4, kv_len);
 					k_reg[i] = *reinterpret_cast<const u32x4*>(kbase + static_cast<size_t>(key) * kvw + (c & 15) * 8);
 				}
-				const int key = min(kt * kKeyTile + v_key, kv_len - 1);
+				const int key = fetch::attn_tile_key(kt, kKeyTile, v_key, kv_len);
 				const uint16_t* vr = vbase + static_cast<size_t>(key) * kvw + v_part0 * 8;
 #pragma unroll
 				for (int i = 0; i < 4; ++i)

@@ -20,6 +20,7 @@
 // everywhere.  Chunk c + 1 (activation tile by direct-to-LDS loads, weights into a second
 // register set) is fetched while chunk c is multiplied.
 #include "common.hpp"
+#include "fetch_model.hpp"
 
 #include <algorithm>
 #include <type_traits>
@@ -835,7 +836,7 @@ namespace litenn_hip
 		template <typename F>
 		constexpr int weight_pieces() // 16-byte pieces per row and chunk in the LDS slot
 		{
-			return F::kAligned16 ? F::kChunkBytes / 16 : (F::kChunkBytes + 14 + 15) / 16;
+			return fetch::gemm_weight_pieces(F::kChunkBytes, F::kAligned16);
 		}
 
 		constexpr size_t kLdsLimit = 160 * 1024;
@@ -920,35 +921,27 @@ namespace litenn_hip
 			// holds a byte of the tensor lies in that byte's page, so nothing outside the tensor's
 			// pages is touched).  Rows past the end re-read the last row; their results are never
 			// stored.
+			// The address arithmetic lives in fetch_model.hpp, where a host test runs it for every
+			// thread of a launch.
 			const uint8_t* w_src[kWLoads]; // the row's chunk 0
 			int w_piece[kWLoads];          // 16 j
+			bool w_issued[kWLoads];
 #pragma unroll
 			for (int i = 0; i < kWLoads; ++i)
 			{
-				const int piece = min(64 * i + lane, NG * 16 * P - 1);
-				const int row = piece / P;
-				w_piece[i] = 16 * (piece - row * P);
-				w_src[i] = w + static_cast<size_t>(min(n_base + row, n - 1)) * row_bytes;
+				const fetch::GemmWeightRequest rq = fetch::gemm_weight_request(i, lane, NG, P);
+				w_piece[i] = rq.offset;
+				w_issued[i] = rq.issued;
+				w_src[i] = w + static_cast<size_t>(fetch::gemm_weight_row(n_base, rq.row, n)) * row_bytes;
 			}
 			const auto issue_w = [&](int c) {
 #pragma unroll
 				for (int i = 0; i < kWLoads; ++i)
 				{
-					if (64 * (i + 1) <= NG * 16 * P || 64 * i + lane < NG * 16 * P)
+					if (64 * (i + 1) <= NG * 16 * P || w_issued[i])
 					{
-						const uintptr_t chunk = reinterpret_cast<uintptr_t>(w_src[i] + static_cast<size_t>(c) * F::kChunkBytes);
-						uintptr_t from = chunk + w_piece[i];
-						if constexpr (!F::kAligned16)
-						{
-							// P counts the pieces of the worst misalignment; with a smaller one the last
-							// piece holds no byte of this chunk, and behind the tensor's last chunk it
-							// can be the first 16 bytes of a page that is not mapped.  Such a piece
-							// fetches the chunk's first piece again (its slot bytes are never read).
-							const uintptr_t base = chunk & ~uintptr_t{ 15 };
-							from = base + w_piece[i];
-							from = from >= chunk + F::kChunkBytes ? base : from;
-						}
-						const uint8_t* src = reinterpret_cast<const uint8_t*>(from);
+						const uint8_t* src = reinterpret_cast<const uint8_t*>(fetch::gemm_weight_piece(
+						    reinterpret_cast<uintptr_t>(w_src[i]), c, F::kChunkBytes, F::kAligned16, w_piece[i]));
 						const uint32_t dst = slot_lds + i * 1024;
 						asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
 						             :
@@ -968,7 +961,7 @@ namespace litenn_hip
 #pragma unroll
 			for (int q = 0; q < NG; ++q)
 			{
-				lane_rows[q] = w + static_cast<size_t>(min(n_base + 16 * q + r, n - 1)) * row_bytes;
+				lane_rows[q] = w + static_cast<size_t>(fetch::gemm_weight_row(n_base, 16 * q + r, n)) * row_bytes;
 			}
 
 			floatx4 acc[NG][MT];
@@ -1004,10 +997,8 @@ namespace litenn_hip
 #pragma unroll
 				for (int q = 0; q < NG; ++q)
 				{
-					const int mis =
-					    F::kAligned16
-					        ? 0
-					        : static_cast<int>(reinterpret_cast<uintptr_t>(lane_rows[q] + static_cast<size_t>(c) * F::kChunkBytes) & 15);
+					const int mis = fetch::gemm_weight_misalignment(reinterpret_cast<uintptr_t>(lane_rows[q]), c,
+					                                                F::kChunkBytes, F::kAligned16);
 					raw[q] = F::load(slot_rows[q] + mis, g);
 					sc[q] = F::prep(raw[q], g);
 				}

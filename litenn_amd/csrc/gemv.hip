@@ -21,6 +21,7 @@
 //   * quants enter the FMA as binary16 subnormals (value * 2^-24), so no int->float conversion
 //     is issued: a mask produces the operand of v_fma_mix_f32.
 #include "common.hpp"
+#include "fetch_model.hpp"
 
 #include <type_traits>
 

@@ -1,0 +1,353 @@
+// Host-side bounds model of the hot kernels' fetch patterns (plain g++, no GPU): runs the address
+// arithmetic of litenn_amd/csrc/fetch_model.hpp -- the very functions the kernels call -- for every
+// thread of a launch over page-exact, ragged and minimal shapes, and checks
+//   * every requested 16-byte piece is 16-byte aligned and holds at least one byte of its tensor
+//     (so it lies in a page the tensor occupies);
+//   * the pieces a kernel consumes are fetched from the right addresses and cover what it reads;
+//   * rows, activation elements and cache rows are each covered, none outside its array.
+// It also shows that the checker has teeth: the matrix-core GEMM's piece arithmetic as it was before
+// its over-fetch was fixed (no redirection of a piece that holds no byte of its chunk) fails on the
+// Q2_K 512 x 512 tensor that once faulted a GPU.
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <map>
+#include <vector>
+
+#include "../../litenn_amd/csrc/fetch_model.hpp"
+
+namespace fm = litenn_hip::fetch;
+
+static int g_failures = 0;
+#define CHECK(cond, ...)                                                                                               \
+	do                                                                                                                 \
+	{                                                                                                                  \
+		if (!(cond))                                                                                                   \
+		{                                                                                                              \
+			if (++g_failures <= 20)                                                                                    \
+			{                                                                                                          \
+				std::printf("FAIL %s:%d %s: ", __FILE__, __LINE__, #cond);                                             \
+				std::printf(__VA_ARGS__);                                                                              \
+				std::printf("\n");                                                                                     \
+			}                                                                                                          \
+		}                                                                                                              \
+	} while (0)
+
+struct Format
+{
+	const char* name;
+	int chunk_bytes;   // bytes of 256 elements
+	bool aligned16;    // the GEMM's view: chunks start on 16-byte boundaries
+	int base_align;    // what the GEMM launcher demands of the tensor's address
+	int stream_slice;  // bytes of 4096 elements (one wavefront's slice in the streaming GEMV)
+};
+static const Format kFormats[] = {
+	{ "Q4_0", 144, true, 16, 2304 }, { "Q4_1", 160, true, 16, 2560 }, { "Q5_0", 176, true, 16, 2816 },
+	{ "Q5_1", 192, true, 16, 3072 }, { "Q8_0", 272, true, 16, 4352 }, { "Q4_K", 144, true, 16, 2304 },
+	{ "Q5_K", 176, true, 16, 2816 }, { "Q2_K", 84, false, 4, 1344 },  { "Q3_K", 110, false, 2, 1760 },
+	{ "Q6_K", 210, false, 2, 3360 },
+};
+
+constexpr uintptr_t kPage = 4096;
+
+// ---- matrix-core GEMM weight pieces -------------------------------------------------------------
+typedef uintptr_t (*PieceFn)(uintptr_t, int, int, bool, int);
+
+static uintptr_t piece_without_redirection(uintptr_t row_start, int c, int chunk_bytes, bool aligned16, int offset)
+{
+	const uintptr_t chunk = row_start + static_cast<size_t>(c) * chunk_bytes;
+	return (aligned16 ? chunk : (chunk & ~uintptr_t{ 15 })) + offset;
+}
+
+// returns the number of pieces that touch no byte of [base, base + bytes)
+static long gemm_case(const Format& f, int ng, int waves, int n, int chunks, uintptr_t base, PieceFn piece_fn,
+                      bool check_contents)
+{
+	const size_t row_bytes = static_cast<size_t>(chunks) * f.chunk_bytes;
+	const uintptr_t end = base + static_cast<size_t>(n) * row_bytes;
+	const int pieces = fm::gemm_weight_pieces(f.chunk_bytes, f.aligned16);
+	const int loads = (ng * 16 * pieces + 63) / 64;
+	const int bn = 16 * waves * ng;
+	long outside = 0;
+	for (int block = 0; block < (n + bn - 1) / bn; ++block)
+	{
+		for (int wave = 0; wave < waves; ++wave)
+		{
+			const int n_base = (block * waves + wave) * 16 * ng;
+			for (int c = 0; c < chunks; ++c)
+			{
+				std::map<int, uintptr_t> slot; // slot byte offset of a piece -> where it was fetched from
+				for (int i = 0; i < loads; ++i)
+				{
+					for (int lane = 0; lane < 64; ++lane)
+					{
+						const fm::GemmWeightRequest rq = fm::gemm_weight_request(i, lane, ng, pieces);
+						if (!(64 * (i + 1) <= ng * 16 * pieces || rq.issued))
+						{
+							continue;
+						}
+						CHECK(rq.row >= 0 && rq.row < 16 * ng && rq.offset >= 0 && rq.offset < 16 * pieces, "%s row %d off %d",
+						      f.name, rq.row, rq.offset);
+						const uintptr_t row_start = base + static_cast<size_t>(fm::gemm_weight_row(n_base, rq.row, n)) * row_bytes;
+						const uintptr_t from = piece_fn(row_start, c, f.chunk_bytes, f.aligned16, rq.offset);
+						if (check_contents)
+						{
+							CHECK(from % 16 == 0, "%s n %d: piece at %#zx is not aligned", f.name, n, static_cast<size_t>(from));
+						}
+						if (!(from < end && from + 16 > base))
+						{
+							++outside;
+						}
+						// the i-th instruction writes 1 KB of the slot: lane l at 1024 i + 16 l
+						slot[1024 * i + 16 * lane] = from;
+					}
+				}
+				if (!check_contents)
+				{
+					continue;
+				}
+				// what the decoders read: row r of the wavefront at slot offset r * 16 pieces + mis,
+				// chunk_bytes bytes, which must be the chunk's own bytes
+				for (int r = 0; r < 16 * ng; ++r)
+				{
+					const uintptr_t row_start = base + static_cast<size_t>(fm::gemm_weight_row(n_base, r, n)) * row_bytes;
+					const uintptr_t chunk = row_start + static_cast<size_t>(c) * f.chunk_bytes;
+					const int mis = fm::gemm_weight_misalignment(row_start, c, f.chunk_bytes, f.aligned16);
+					for (int b = 0; b < f.chunk_bytes; ++b)
+					{
+						const int at = r * 16 * pieces + mis + b;
+						const auto it = slot.find(at & ~15);
+						CHECK(it != slot.end() && it->second + (at & 15) == chunk + b, "%s n %d chunk %d row %d byte %d", f.name, n, c,
+						      r, b);
+					}
+				}
+			}
+		}
+	}
+	return outside;
+}
+
+static void test_gemm_weight_pieces()
+{
+	const int tiles[][2] = { { 2, 8 }, { 1, 8 }, { 1, 4 } }; // weight groups per wavefront, wavefronts
+	long cases = 0;
+	for (const Format& f : kFormats)
+	{
+		for (const auto& t : tiles)
+		{
+			for (int n : { 1, 15, 16, 17, 33, 128, 129, 512 })
+			{
+				for (int chunks : { 1, 2, 3, 8 })
+				{
+					const size_t bytes = static_cast<size_t>(n) * chunks * f.chunk_bytes;
+					std::vector<uintptr_t> bases;
+					for (int mis = 0; mis < 16; mis += f.base_align)
+					{
+						bases.push_back(64 * kPage + mis); // every misalignment the launcher accepts
+					}
+					const uintptr_t ends_on_page = 1024 * kPage - bytes; // the tensor's last byte is a page's last
+					if (ends_on_page % f.base_align == 0)
+					{
+						bases.push_back(ends_on_page);
+					}
+					for (uintptr_t base : bases)
+					{
+						const long outside = gemm_case(f, t[0], t[1], n, chunks, base, fm::gemm_weight_piece, true);
+						CHECK(outside == 0, "%s ng %d waves %d n %d chunks %d base %#zx: %ld pieces outside the tensor", f.name, t[0],
+						      t[1], n, chunks, static_cast<size_t>(base), outside);
+						++cases;
+					}
+				}
+			}
+		}
+	}
+	std::printf("gemm weight pieces: %ld launches walked\n", cases);
+	// the arithmetic as it was before the fix, on the tensor that faulted: Q2_K, 512 rows of 512
+	// elements = 21 pages exactly; the last piece of the last rows' last chunk lies in the next page
+	const Format& q2k = kFormats[7];
+	const size_t bytes = 512 * 2 * 84;
+	CHECK(bytes == 21 * kPage, "Q2_K 512 x 512 is 21 pages");
+	const long before = gemm_case(q2k, 1, 4, 512, 2, 512 * kPage, piece_without_redirection, false);
+	const long after = gemm_case(q2k, 1, 4, 512, 2, 512 * kPage, fm::gemm_weight_piece, false);
+	CHECK(before > 0, "the pre-fix arithmetic must be caught");
+	CHECK(after == 0, "the current arithmetic stays inside");
+	std::printf("Q2_K 512 x 512, page-exact: %ld pieces behind the tensor before the fix, %ld now\n", before, after);
+}
+
+// ---- streaming GEMV ------------------------------------------------------------------------------
+static void test_stream_rows_and_pieces()
+{
+	long cases = 0;
+	for (const Format& f : kFormats)
+	{
+		for (int k : { 256, 512, 1024, 4096, 4352, 8192, 11008, 12288, 14336, 28672, 32768 })
+		{
+			const uint32_t row_bytes = static_cast<uint32_t>(k / 256 * f.chunk_bytes);
+			const int slices = (k + 4095) / 4096;
+			if (slices > 8 || row_bytes % 16 != 0)
+			{
+				continue; // the launcher sends such a shape to the register kernel
+			}
+			const int groups = 8 / slices;
+			if (k > 64 * slices * groups * 4 * 8)
+			{
+				continue; // more than eight 128-bit activation loads per thread: register kernel as well
+			}
+			const int loads = (f.stream_slice + 1023) / 1024;
+			for (int whole = 0; whole < 2; ++whole)
+			{
+				if (whole && k != 4096)
+				{
+					continue; // the whole-slice instance exists for K = 4096 only
+				}
+				std::vector<int> covered(row_bytes, 0);
+				for (int s = 0; s < slices; ++s)
+				{
+					const uint32_t slice_off = static_cast<uint32_t>(s) * f.stream_slice;
+					CHECK(slice_off < row_bytes, "%s k %d slice %d starts behind the row", f.name, k, s);
+					const uint32_t len = fm::stream_slice_len(whole != 0, f.stream_slice, row_bytes, slice_off);
+					CHECK(len >= 16 && len % 16 == 0 && slice_off + len <= row_bytes, "%s k %d slice %d len %u", f.name, k, s, len);
+					for (int i = 0; i < loads; ++i)
+					{
+						for (int lane = 0; lane < 64; ++lane)
+						{
+							const fm::StreamPiece p = fm::stream_row_piece(i, lane, len, whole != 0);
+							if (!p.issued)
+							{
+								continue;
+							}
+							CHECK(p.offset + 16 <= len, "%s k %d: piece %u + 16 > %u", f.name, k, p.offset, len);
+							if (1024u * i + 16u * lane < len) // a consumed piece sits where the unit reads it
+							{
+								CHECK(p.offset == 1024u * i + 16u * lane, "%s k %d: piece misplaced", f.name, k);
+								for (int b = 0; b < 16; ++b)
+								{
+									++covered[slice_off + p.offset + b];
+								}
+							}
+						}
+					}
+				}
+				for (uint32_t b = 0; b < row_bytes; ++b)
+				{
+					CHECK(covered[b] == 1, "%s k %d: row byte %u fetched %d times", f.name, k, b, covered[b]);
+				}
+				// activations: 128-bit loads, clamped so that every thread issues every one of them
+				const int threads = 64 * slices * groups;
+				const int per_thread = (k / 4 + threads - 1) / threads;
+				const int xp = per_thread <= 2 ? 2 : (per_thread <= 4 ? 4 : 8);
+				CHECK(per_thread <= xp, "%s k %d: %d loads per thread", f.name, k, per_thread);
+				std::vector<int> x_seen(k, 0);
+				for (int tid = 0; tid < threads; ++tid)
+				{
+					for (int j = 0; j < xp; ++j)
+					{
+						const int at = fm::stream_x_index(tid, j, threads, k);
+						CHECK(at >= 0 && at + 4 <= k && at % 4 == 0, "%s k %d: x load at %d", f.name, k, at);
+						if ((tid + j * threads) * 4 < k)
+						{
+							for (int e = 0; e < 4; ++e)
+							{
+								++x_seen[at + e];
+							}
+						}
+					}
+				}
+				for (int e = 0; e < k; ++e)
+				{
+					CHECK(x_seen[e] == 1, "%s k %d: activation %d staged %d times", f.name, k, e, x_seen[e]);
+				}
+				// rows: one round of workgroups, every row walked by exactly one wavefront group
+				for (int n_total : { 1, 2, 7, 100, 4096, 11008, 32000, 128256 })
+				{
+					for (int max_blocks : { 256, 64, 1 })
+					{
+						int rows = (n_total + max_blocks * groups - 1) / (max_blocks * groups);
+						rows = rows < 1 ? 1 : (rows > 64 ? 64 : rows);
+						const int blocks = (n_total + groups * rows - 1) / (groups * rows);
+						std::vector<int> walked(n_total, 0);
+						for (int block = 0; block < blocks; ++block)
+						{
+							for (int g = 0; g < groups; ++g)
+							{
+								const fm::StreamRows r = fm::stream_group_rows(block, g, groups, rows, n_total);
+								CHECK(r.count >= 0 && r.count <= rows, "count %d", r.count);
+								for (int q = 0; q < r.count; ++q)
+								{
+									CHECK(r.row0 + q < n_total, "%s k %d n %d: row %d", f.name, k, n_total, r.row0 + q);
+									if (r.row0 + q < n_total)
+									{
+										++walked[r.row0 + q];
+									}
+								}
+							}
+						}
+						for (int r = 0; r < n_total; ++r)
+						{
+							CHECK(walked[r] == 1, "%s k %d n %d: row %d walked %d times", f.name, k, n_total, r, walked[r]);
+						}
+						++cases;
+					}
+				}
+			}
+		}
+	}
+	std::printf("streaming gemv: %ld launch geometries walked\n", cases);
+}
+
+// ---- tiled prompt attention -----------------------------------------------------------------------
+static void test_attention_tiles()
+{
+	constexpr int q_tile = 64, key_tile = 64;
+	long cases = 0;
+	for (int m : { 16, 17, 63, 64, 65, 100, 512, 2048 })
+	{
+		for (int past : { 0, 1, 5, 63, 64, 1000 })
+		{
+			const int cache_rows = past + m; // rows the cache is guaranteed to hold
+			for (int tile = 0; tile < (m + q_tile - 1) / q_tile; ++tile)
+			{
+				const int kv_len = fm::attn_tile_kv_len(past, tile * q_tile, q_tile, m);
+				CHECK(kv_len >= 1 && kv_len <= cache_rows, "m %d past %d tile %d: kv_len %d", m, past, tile, kv_len);
+				// the last row of the tile sees keys 0 .. past + row
+				const int last_row = (tile * q_tile + q_tile < m ? tile * q_tile + q_tile : m) - 1;
+				CHECK(kv_len == past + last_row + 1, "kv_len %d", kv_len);
+				const int n_key_tiles = (kv_len + key_tile - 1) / key_tile;
+				std::vector<int> seen(kv_len, 0);
+				for (int kt = 0; kt < n_key_tiles + 2; ++kt) // the kernel re-reads the last tile past the end
+				{
+					const int t = fm::imin(kt, n_key_tiles - 1);
+					for (int idx = 0; idx < key_tile; ++idx)
+					{
+						const int key = fm::attn_tile_key(t, key_tile, idx, kv_len);
+						CHECK(key >= 0 && key < kv_len, "m %d past %d: key %d of %d", m, past, key, kv_len);
+						if (kt < n_key_tiles && t * key_tile + idx < kv_len)
+						{
+							++seen[key];
+						}
+					}
+				}
+				for (int key = 0; key < kv_len; ++key)
+				{
+					CHECK(seen[key] == 1, "m %d past %d: key %d staged %d times", m, past, key, seen[key]);
+				}
+				++cases;
+			}
+		}
+	}
+	std::printf("attention tiles: %ld query tiles walked\n", cases);
+}
+
+int main()
+{
+	test_gemm_weight_pieces();
+	test_stream_rows_and_pieces();
+	test_attention_tiles();
+	if (g_failures)
+	{
+		std::printf("%d checks failed\n", g_failures);
+		return 1;
+	}
+	std::printf("fetch bounds ok\n");
+	return 0;
+}

@@ -31,3 +31,16 @@ def test_cpp_device_traits_on_the_gpu():
     for name in ("MatMul reference vector", "Q4_0 fixture block . x", "Q4_0 fixture block dequantised",
                  "RMSNorm closed form", "Reduce Sum"):
         assert f"ok   {name}" in p.stdout, p.stdout
+
+
+def test_fetch_patterns_stay_inside_their_tensors():
+    """tests/cpp/fetch_bounds_test.cpp (CPU only): the address arithmetic the kernels call
+    (litenn_amd/csrc/fetch_model.hpp) walked for every thread of a launch -- matrix-core GEMM weight
+    pieces for every format, tile and misalignment including page-exact tensors, streaming GEMV rows
+    with the lane-0 fill-in, activation loads, attention key tiles -- and the GEMM's arithmetic as
+    it was before its over-fetch was fixed, which must be caught."""
+    assert os.path.exists(hip_build.FETCH_TEST_BIN), "run `python -m litenn_amd.build` (or __graft_entry__.build())"
+    p = subprocess.run([hip_build.FETCH_TEST_BIN], capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stdout[-3000:] + p.stderr
+    assert "fetch bounds ok" in p.stdout and "FAIL" not in p.stdout
+    assert "pieces behind the tensor before the fix, 0 now" in p.stdout
