@@ -110,3 +110,41 @@ def test_error_paths(oracle):
         missing.eval([0])
     with pytest.raises(oracle.OracleError, match="shape"):
         m.set_tensor(2, 0, Q4_0, np.zeros(18, np.uint8), 1, 32)
+
+
+@pytest.mark.parametrize("fmt,heads,kv_heads,rope_dims,freq_scale", [
+    (Q4_0, 8, 2, 0, 1.0), (Q8_0, 6, 3, 0, 1.0), (Q4_K, 4, 1, 32, 0.5), (Q6_K, 4, 4, 0, 1.0)])
+def test_block_wiring_against_a_numpy_recomposition_of_the_lowering(oracle, fmt, heads, kv_heads, rope_dims, freq_scale):
+    """The checker's decoder against tests/np_llama.py, a float64 recomposition of
+    AddLLaMADecoderBlockDecode written from tools/gguf/LLaMABuilder.cpp:568-668 with its own block
+    decoders: random non-zero weights, grouped KV heads, several calls so that rows sit at
+    positions past + i against a filled cache.  Then the power of the comparison: five plausible
+    wiring mistakes planted in the numpy model must all be far outside the tolerance."""
+    from np_llama import NumpyLLaMA
+    d = 64 * heads if fmt in (Q4_0, Q8_0) else 256
+    cfg = synth.LLaMAConfig("wiring", 2, d, heads, kv_heads, 512, 96, 32, formats={"default": fmt},
+                            rope_freq_scale=freq_scale, rope_dimension_count=rope_dims)
+    if fmt in (Q4_K, Q6_K):
+        cfg.feed_forward_length = 512
+    tensors = list(synth.llama_tensors(cfg, 31))
+    toks = synth.prompt_tokens(cfg, 9, 6)
+    pieces = [toks[:5], toks[5:8], toks[8:]]
+
+    def run(model):
+        return np.concatenate([np.asarray(model.eval(p), np.float64).reshape(len(p), -1) for p in pieces])
+
+    ref = oracle_model(oracle, cfg, 31, kv_f16=False, tensors=tensors)
+    want = run(NumpyLLaMA(cfg, tensors))
+    got = run(ref)
+    assert rel_l2(got, want) < 1e-5
+    # the cache holds rotated keys and plain values at rows 0 .. past
+    nm = NumpyLLaMA(cfg, tensors)
+    run(nm)
+    for layer in range(cfg.block_count):
+        k, v = ref.get_kv(layer)
+        assert rel_l2(k, nm.k[layer]) < 1e-5 and rel_l2(v, nm.v[layer]) < 1e-5
+    mistakes = ["keys_not_rotated", "residual_from_norm", "gate_up_swapped", "positions_from_zero"]
+    if kv_heads not in (1, heads):
+        mistakes.append("kv_head_modulo")
+    for mistake in mistakes:
+        assert rel_l2(run(NumpyLLaMA(cfg, tensors, mistake=mistake)), want) > 1e-2, mistake
