@@ -1398,3 +1398,32 @@ int oracle_llama_get_kv(const oracle_llama* m, int layer, float* k, float* v)
 	memcpy(v, m->layers[layer].vcache, sizeof(float) * (size_t)m->past * kvw);
 	return 0;
 }
+
+/* Test-harness convenience (no counterpart in the reference): puts back cache rows that
+ * oracle_llama_get_kv returned earlier and sets the position, so that a long checker run can be
+ * resumed from a saved state.  Rows are copied bit for bit. */
+int oracle_llama_set_kv(oracle_llama* m, int layer, int rows, const float* k, const float* v)
+{
+	if (layer < 0 || layer >= m->n_layer)
+	{
+		return fail("layer index out of range");
+	}
+	if (rows < 0 || rows > m->ctx)
+	{
+		return fail("row count exceeds the context length");
+	}
+	const size_t kvw = (size_t)m->n_kv_head * (size_t)m->head_dim;
+	memcpy(m->layers[layer].kcache, k, sizeof(float) * (size_t)rows * kvw);
+	memcpy(m->layers[layer].vcache, v, sizeof(float) * (size_t)rows * kvw);
+	return 0;
+}
+
+int oracle_llama_set_past(oracle_llama* m, int past)
+{
+	if (past < 0 || past > m->ctx)
+	{
+		return fail("position exceeds the context length");
+	}
+	m->past = past;
+	return 0;
+}

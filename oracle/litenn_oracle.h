@@ -163,6 +163,10 @@ int oracle_llama_generate(oracle_llama* m, const int32_t* prompt, int n_prompt, 
                           float* margins);
 /* copy of the cache: k,v [past, n_kv_head*head_dim] f32 (rounded values if kv_f16) */
 int oracle_llama_get_kv(const oracle_llama* m, int layer, float* k, float* v);
+/* Harness convenience, no counterpart in the reference: restore `rows` cache rows saved with
+ * oracle_llama_get_kv, and set the position (resuming a long checker run). */
+int oracle_llama_set_kv(oracle_llama* m, int layer, int rows, const float* k, const float* v);
+int oracle_llama_set_past(oracle_llama* m, int past);
 
 const char* oracle_last_error(void);
 void oracle_set_threads(int n);

@@ -74,6 +74,8 @@ def lib() -> C.CDLL:
         L.oracle_llama_eval.argtypes = [vp, vp, i32, vp, vp]
         L.oracle_llama_generate.argtypes = [vp, vp, i32, i32, vp, vp]
         L.oracle_llama_get_kv.argtypes = [vp, i32, vp, vp]
+        L.oracle_llama_set_kv.argtypes = [vp, i32, i32, vp, vp]
+        L.oracle_llama_set_past.argtypes = [vp, i32]
         L.oracle_set_threads.argtypes = [i32]
         _lib = L
     return _lib
@@ -280,3 +282,11 @@ class LLaMA:
         v = np.empty((self.past, w), np.float32)
         _check(lib().oracle_llama_get_kv(self._h, layer, _p(k), _p(v)))
         return k, v
+
+    def set_kv(self, layer: int, k, v) -> None:
+        """Puts back rows that get_kv returned (bit for bit); set_past then sets the position."""
+        k, v = _f32(k), _f32(v)
+        _check(lib().oracle_llama_set_kv(self._h, layer, k.shape[0], _p(k), _p(v)))
+
+    def set_past(self, past: int) -> None:
+        _check(lib().oracle_llama_set_past(self._h, past))

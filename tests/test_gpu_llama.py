@@ -97,12 +97,24 @@ def test_single_token_steps_with_a_q6_k_value_projection(hip, oracle, main_fmt, 
     cfg = synth.tiny_llama(main_fmt, block_count=2, d_model=d_model, heads=d_model // 128 * 2, kv_heads=2, ff=ff,
                            vocab=777, formats={"default": main_fmt, "attn_v": Q6_K, "ffn_down": Q6_K, "output": Q6_K})
     toks = synth.prompt_tokens(cfg, 9, 8)
+    # Float32 cache: the whole step is held to the checker at a few 1e-6.  Float16 cache: a key or value
+    # within an f32 rounding of a half's midpoint lands on the other half on the device (a handful of
+    # the 1152 values of a layer do), and this random two-block model amplifies each such 2^-11 about
+    # six times per block, so the logits agree to 1e-3 only; what the cache holds is pinned bit for bit
+    # by tests/test_gpu_glue.py::test_kv_append_f16_uses_litenn_rounding instead.
+    dev32, ref32 = hip_model(hip, cfg, 4, kv_dtype=DT_F32), oracle_model(oracle, cfg, 4, kv_f16=False)
+    for t in toks:
+        assert rel_l2(dev32.eval([t])[0], ref32.eval([t])[0]) < 3e-5
+    for layer in range(cfg.block_count):
+        for got, want in zip(dev32.get_kv(layer), ref32.get_kv(layer)):
+            assert rel_l2(got, want) < 3e-5
+    dev32.close()
     dev, ref = hip_model(hip, cfg, 4), oracle_model(oracle, cfg, 4)
     for t in toks:
-        assert rel_l2(dev.eval([t])[0], ref.eval([t])[0]) < 1e-4
+        assert rel_l2(dev.eval([t])[0], ref.eval([t])[0]) < 2e-3
     for layer in range(cfg.block_count):
         for got, want in zip(dev.get_kv(layer), ref.get_kv(layer)):
-            assert rel_l2(got, want) < 1e-3  # fp16 cache: a rounding flip is 2^-11 of the value
+            assert rel_l2(got, want) < 1e-3
     dev.reset()
     ref.reset()
     got, _, _ = dev.generate(toks[:4], 12)
@@ -124,36 +136,54 @@ def test_error_paths(hip):
         hip.LLaMA(1, 64, 4, 3, 64, 10, 8)
 
 
+def _step_figures(logits, probe_indices):
+    best = int(np.argmax(logits))
+    rest = logits.copy()
+    rest[best] = -np.inf
+    return best, float(logits[best] - rest.max()), float(np.abs(logits).max()), logits[probe_indices].astype(np.float64)
+
+
 def test_llama7b_q4_0_greedy_matches_committed_fixture(hip):
     """BASELINE config 4 at full size: the 7B-shape Q4_0 model, prompt 128, 256 greedy tokens, fp16
     KV cache, against tests/golden/llama7b_q4_0_tokens.json (written from the CPU checker by
-    tests/golden/make_llama7b_tokens.py; the model and the prompt are rebuilt from the seed).
-    Tokens must be identical; the top-2 logit margin of the first step must agree to 1e-3 relative,
-    which is what makes the identity meaningful for this random-init model (its margins are ~1.9)."""
+    tests/golden/make_llama7b_tokens.py; the model and the prompt are rebuilt from the seeds).
+    The fixture's continuation is varied (dozens of distinct tokens) and none of its steps is decided
+    by less than 1e-3 of the largest logit, so:
+      * the device's greedy loop (captured single-token step) must return the same 256 tokens;
+      * fed the fixture's tokens step by step, every step's arg-max, top-2 margin and the logits at
+        eight fixed vocabulary indices must agree with the checker's to 1e-3 of the largest logit: a
+        wrong position, cache row or head mapping at any step shows there even where it would not
+        change the token;
+      * after a prompt pass on the matrix cores (Float16 operands, about 1e-3 of the logits) the
+        same walk holds to 2e-2, and the arg-max wherever the checker's margin is wider than that."""
     import json
     import os
     fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "llama7b_q4_0_tokens.json")))
     assert fx["complete"] and fx["new_tokens"] == 256
+    tokens, margins = fx["tokens"], np.array(fx["margins"])
+    absmax, probes, idx = np.array(fx["logit_absmax"]), np.array(fx["probes"]), fx["probe_indices"]
+    # the fixture bites: a varied sequence, no step near a tie
+    assert len(set(tokens)) >= 32 and float((margins / absmax).min()) >= 1e-3
     cfg = synth.llama_7b_q4_0(context_length=fx["context_length"])
     assert cfg.name == fx["model"]
-    prompt = synth.prompt_tokens(cfg, fx["prompt_length"], fx["seed"])
+    prompt = synth.prompt_tokens(cfg, fx["prompt_length"], fx["prompt_seed"])
     assert prompt[:8].tolist() == fx["prompt_head"]
     dev = hip_model(hip, cfg, fx["seed"])
     # f32-operand prefill (GEMV path), then the captured single-token step
     got, _, _ = dev.generate(prompt, 256)
-    assert got.tolist() == fx["tokens"]
-    # prefill on the matrix cores (fp16 operands), same continuation
-    dev.reset()
-    again, _, _ = dev.generate(prompt, 256, precise=False)
-    assert again.tolist() == fx["tokens"]
-    # margins: first generated step, from the logits of the last prompt position
-    dev.reset()
-    logits = dev.eval(prompt, all_logits=False)
-    best = int(np.argmax(logits))
-    rest = logits.copy()
-    rest[best] = -np.inf
-    assert best == fx["tokens"][0]
-    assert abs(float(logits[best] - rest.max()) - fx["margins"][0]) <= 1e-3 * abs(fx["margins"][0])
+    assert got.tolist() == tokens, np.nonzero(got != np.array(tokens))[0][:4]
+    for precise, tol in ((True, 1e-3), (False, 2e-2)):
+        dev.reset()
+        logits = dev.eval(prompt, all_logits=False, precise=precise)
+        for step in range(256):
+            best, margin, top, pr = _step_figures(logits, idx)
+            bar = tol * absmax[step]
+            assert abs(top - absmax[step]) <= bar, (precise, step)
+            assert np.all(np.abs(pr - probes[step]) <= bar), (precise, step, pr, probes[step])
+            if margins[step] > 2 * bar:
+                assert best == tokens[step] and abs(margin - margins[step]) <= 2 * bar, (precise, step)
+            if step < 255:
+                logits = dev.eval([tokens[step]], all_logits=False)
     dev.close()
 
 
@@ -236,4 +266,22 @@ def test_linear_rope_scaling_and_partial_rotation(hip, oracle, tmp_path):
     dev.reset()
     assert np.array_equal(loaded.eval(toks), dev.eval(toks))
     loaded.close()
+    dev.close()
+
+
+def test_a_context_of_forty_thousand_positions(hip, oracle):
+    """Nothing in the runtime holds per-key storage, so the context is bounded by the caches' memory
+    only: a model declared with 40000 positions (beyond what an earlier score buffer held) is created,
+    evaluates a prompt and single steps like any other, and its attention is cut into key chunks
+    sized for the declared context from the first token on."""
+    cfg = synth.tiny_llama(Q4_0, block_count=2, d_model=256, heads=4, kv_heads=2, ff=512, vocab=300,
+                           context_length=40000)
+    toks = synth.prompt_tokens(cfg, 24, 12)
+    dev, ref = hip_model(hip, cfg, 5, kv_dtype=DT_F32), oracle_model(oracle, cfg, 5, kv_f16=False)
+    assert rel_l2(dev.eval(toks[:20]), ref.eval(toks[:20])) < 5e-5
+    for t in toks[20:]:
+        assert rel_l2(dev.eval([t])[0], ref.eval([t])[0]) < 5e-5
+    dev.reset()
+    ref.reset()
+    assert dev.generate(toks[:5], 10)[0].tolist() == ref.generate(toks[:5], 10)[0].tolist()
     dev.close()

@@ -67,10 +67,13 @@ def test_random_model_matches_checker(hip, oracle, seed):
     for piece in pieces:
         want = ref.eval(piece)
         got = dev.eval(piece)
-        # With the Float16 cache a key or value that lands within rounding distance of a half's
-        # midpoint can round the other way on the device (one unit of a half, 5e-4 relative, on one
-        # element); in these one- and two-block models a single such flip shows in the logits.
-        assert rel_l2(got, want) < (2e-3 if kv == DT_F16 else 2e-4), (what, len(piece), dev.past)
+        # With the Float16 cache a key or value that lands within an f32 rounding of a half's
+        # midpoint rounds the other way on the device (one unit of a half, 5e-4 relative, on a few
+        # elements per thousand), and a random block amplifies such a difference several times: the
+        # Float32-cache cases carry the sharp bar, the Float16 ones the rounding-tolerant one.
+        err = rel_l2(got, want)
+        print("piece of %d rows: %.2e" % (len(piece), err), flush=True)
+        assert err < (2e-3 if kv == DT_F16 else 5e-5), (what, len(piece), dev.past)
     assert dev.past == ref.past
     kd, vd = dev.get_kv(cfg.block_count - 1)
     kr, vr = ref.get_kv(cfg.block_count - 1)
@@ -80,12 +83,13 @@ def test_random_model_matches_checker(hip, oracle, seed):
     fast = dev.eval(toks[:first + 3 + later], precise=False)
     ref.reset()
     full = ref.eval(toks[:first + 3 + later])
-    # (per row: these synthetic weights are large, attention scores reach the hundreds, and the
-    # softmax turns the 3e-4 of the Float16 operands into a few 1e-3 per block; a row whose two
-    # best keys score alike gets a different mixture altogether -- such a row may stand out, the
-    # rest may not.  A wrong tile, row or format shows as errors of order one.)
+    # (per row, and every row: the model's attention scores are of order one -- see
+    # tests/test_synth_conditioning.py -- so the 3e-4 of the Float16 operands stays a few 1e-4 per
+    # matmul and block and no row may stand out.  A wrong tile, row or format shows as errors of
+    # order one.)
     rows = np.array([rel_l2(fast[i], full[i]) for i in range(len(full))])
-    assert np.median(rows) < 1e-2 and np.sum(rows >= 5e-2) <= max(1, len(rows) // 10), (what, rows)
+    print("matrix-core rows: median %.2e max %.2e" % (np.median(rows), rows.max()), flush=True)
+    assert np.median(rows) < 2e-3 and rows.max() < 5e-3, (what, rows)
     # greedy continuation: device loop and step-by-step evaluation agree with each other
     dev.reset()
     generated = dev.generate(toks[:first], 6)[0]
