@@ -25,8 +25,13 @@
  *  - tensors are row-major and contiguous.
  *  - `opts` mirrors CUDAExecutionOptions (src/LiteNN/Device/CUDA.h:70-74):
  *    NULL means stream 0 and synchronise before returning.
- *  - all entry points are thread-safe; each call selects `dev` for its own
- *    duration (cf. CUDADeviceGuard, src/LiteNN/Device/CUDA.cpp:734-761).
+ *  - the entry points of groups 1, 2 and 4 may be called from several host threads at
+ *    once; each call selects `dev` for its own duration (cf. CUDADeviceGuard,
+ *    src/LiteNN/Device/CUDA.cpp:734-761).  A litenn_hip_llama handle (group 3) is a
+ *    mutable object -- cache position, scratch buffers, the captured step -- and must
+ *    not be used by two threads at the same time; separate handles run side by side.
+ *    litenn_hip_attn_decode_noalloc shares one scratch array per GPU between all its
+ *    calls (see there).
  */
 #ifndef LITENN_HIP_H
 #define LITENN_HIP_H
@@ -235,7 +240,9 @@ enum litenn_llama_tensor {
 };
 
 /* Hyper-parameters as ParseLLaMAHyperparameters yields them
- * (tools/gguf/GGUFImporter.cpp:505-642).  kv_dtype is F16 or F32. */
+ * (tools/gguf/GGUFImporter.cpp:505-642).  kv_dtype is F16 or F32.  context_length is bounded by
+ * 2^30 positions and by the memory of the caches it sizes
+ * (2 * block_count * context_length * head_count_kv * head_dim elements of kv_dtype). */
 typedef struct litenn_hip_llama_params {
 	int32_t block_count, embedding_length, head_count, head_count_kv, feed_forward_length, vocab_size,
 	    context_length, rope_dimension_count;

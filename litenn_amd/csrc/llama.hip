@@ -480,9 +480,12 @@ extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* p
 	{
 		return fail(kAction, "head dimension must be even and at most 256");
 	}
-	if (p.context_length > 15360)
+	// The attention kernels keep no per-key storage (online softmax), so the context is bounded only
+	// by the 2^30 positions their int arithmetic takes and by the memory the caches need (an
+	// allocation failure below reports that).
+	if (p.context_length > (1 << 30))
 	{
-		return fail(kAction, "context length exceeds the 15360 positions the attention score buffer holds");
+		return fail(kAction, "context length exceeds 2^30 positions");
 	}
 	if (p.kv_dtype != LITENN_F16 && p.kv_dtype != LITENN_F32)
 	{
@@ -525,12 +528,17 @@ extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* p
 	if (half)
 	{
 		std::vector<float> c(static_cast<size_t>(p.context_length) * half), s(c.size());
+		std::vector<double> inv_freqs(half);
+		for (size_t dim = 0; dim < half; ++dim)
+		{
+			const double exponent = -2.0 * static_cast<double>(dim) / static_cast<double>(half * 2);
+			inv_freqs[dim] = std::pow(p.rope_freq_base, exponent);
+		}
 		for (size_t pos = 0; pos < static_cast<size_t>(p.context_length); ++pos)
 		{
 			for (size_t dim = 0; dim < half; ++dim)
 			{
-				const double exponent = -2.0 * static_cast<double>(dim) / static_cast<double>(half * 2);
-				const double inv_freq = std::pow(p.rope_freq_base, exponent);
+				const double inv_freq = inv_freqs[dim];
 				const double angle = static_cast<double>(pos) * inv_freq * p.rope_freq_scale;
 				c[pos * half + dim] = static_cast<float>(std::cos(angle));
 				s[pos * half + dim] = static_cast<float>(std::sin(angle));
@@ -824,24 +832,39 @@ extern "C" int litenn_hip_llama_generate(litenn_hip_llama* m, const int32_t* pro
 		m->cap_out = n_new;
 	}
 	hipStream_t s = m->stream;
-	hipEvent_t ev[3];
-	for (hipEvent_t& e : ev)
-	{
-		LITENN_HIP_TRY(kAction, hipEventCreate(&e));
-	}
-	int rc = 0;
+	// the events exist before any work is queued and are destroyed on every way out
+	hipEvent_t ev[3] = { nullptr, nullptr, nullptr };
 	auto cleanup = [&]() {
 		for (hipEvent_t& e : ev)
 		{
-			(void)hipEventDestroy(e);
+			if (e)
+			{
+				(void)hipEventDestroy(e);
+				e = nullptr;
+			}
 		}
 	};
+	for (hipEvent_t& e : ev)
+	{
+		const hipError_t ce = hipEventCreate(&e);
+		if (ce != hipSuccess)
+		{
+			e = nullptr;
+			cleanup();
+			return fail_hip(kAction, ce);
+		}
+	}
+	int rc = 0;
+	// A failure part-way leaves `past` as it was: the rows a failed run appended lie beyond it, are
+	// never read (every pass takes its position from `past`) and are overwritten by the next call.
+	// The stream is drained first so that nothing of the failed run is still in flight afterwards.
 #define GEN_TRY(expr)                                                                                                  \
 	do                                                                                                                 \
 	{                                                                                                                  \
 		const hipError_t e_ = (expr);                                                                                  \
 		if (e_ != hipSuccess)                                                                                          \
 		{                                                                                                              \
+			(void)hipStreamSynchronize(s);                                                                             \
 			cleanup();                                                                                                 \
 			return fail_hip(kAction, e_);                                                                              \
 		}                                                                                                              \
