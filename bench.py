@@ -170,6 +170,125 @@ def bench_prefill_gemm(ln, hiprt, only=None):
     return out
 
 
+def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=125):
+    """What the headline GEMV's time is made of, measured on the same card with the same rotation of
+    weight buffers and the same graph replay (lib/liblitenn_hip_trace.so: the library with timeline
+    stamps compiled into the streaming kernel, plus csrc/microbench.hip):
+      * a kernel that does nothing, per graph node;
+      * a kernel that only reads the same 33 MB per launch (best of several geometries);
+      * the streaming kernel's own timeline: per wavefront, on the card's shared 100 MHz clock, when
+        it started, had its activations in registers, saw each of its rows land and finished."""
+    import ctypes as C
+    from litenn_amd import synth
+    from litenn_amd import build as hip_build
+    from litenn_amd._lib import Exec
+    from litenn_amd.formats import row_bytes
+    tl = C.CDLL(hip_build.TRACE_LIB_PATH)
+    tl.litenn_hip_last_error.restype = C.c_char_p
+    vp, sz = C.c_void_p, C.c_size_t
+    tl.litenn_hip_mul_mat_q.argtypes = [C.c_int, C.c_int, vp, sz, sz, vp, C.c_int, sz, vp, vp, C.c_uint, C.POINTER(Exec)]
+    tl.litenn_hip_mb_empty.argtypes = [vp]
+    tl.litenn_hip_mb_read.argtypes = [vp, sz, C.c_int, C.c_int, vp, vp]
+    tl.litenn_hip_gemv_trace_read.argtypes = [vp, sz]
+    tl.litenn_hip_gemv_trace_skip_arithmetic.argtypes = [C.c_int]
+
+    def ok(rc):
+        if rc != 0:
+            raise RuntimeError(tl.litenn_hip_last_error().decode())
+
+    wq_host = synth.quant_weights(fmt, n, k, 1)
+    weights = [ln.Tensor.from_numpy(np.roll(wq_host, b, axis=0).reshape(-1)) for b in range(n_buffers)]
+    w_bytes = n * row_bytes(fmt, k)
+    x = ln.Tensor.from_numpy(synth.activations(1, k, 2))
+    y = ln.Tensor((1, n))
+    sink = ln.Tensor((4,))
+    stream = hiprt.Stream()
+    opts = Exec(stream.handle, 0)
+
+    def per_launch_us(launch):
+        """One rotation captured as a graph, replayed; HIP events on the stream."""
+        for i in range(n_buffers):
+            launch(i)
+        stream.synchronize()
+        stream.begin_capture()
+        for i in range(n_buffers):
+            launch(i)
+        graph = stream.end_capture()
+        graph.launch(stream)
+        stream.synchronize()
+        e0, e1 = hiprt.Event(), hiprt.Event()
+        e0.record(stream)
+        for _ in range(replays):
+            graph.launch(stream)
+        e1.record(stream)
+        stream.synchronize()
+        us = e0.elapsed_ms(e1) * 1e3 / (replays * n_buffers)
+        graph.destroy()
+        return us
+
+    out = {"rotation": f"{n_buffers} buffers x {w_bytes} B, graph of {n_buffers} launches replayed {replays} times"}
+    out["empty_kernel_us"] = round(per_launch_us(lambda i: ok(tl.litenn_hip_mb_empty(stream.handle))), 3)
+    reads = []
+    for blocks in (256, 512, 1024, 2048):
+        for depth in (2, 4, 8):
+            us = per_launch_us(lambda i: ok(tl.litenn_hip_mb_read(weights[i % n_buffers].ptr, w_bytes, blocks, depth,
+                                                                  sink.ptr, stream.handle)))
+            reads.append({"blocks": blocks, "loads_in_flight_per_lane": depth, "us": round(us, 3),
+                          "gbps": round(w_bytes / us / 1e3, 1)})
+    best = min(reads, key=lambda r: r["us"])
+    out["read_kernel_best"] = best
+    out["read_kernel_all"] = reads
+    log(f"[bench] microbench: empty kernel {out['empty_kernel_us']} us/launch; read-only kernel best "
+        f"{best['us']} us = {best['gbps']} GB/s ({best['blocks']} workgroups, {best['loads_in_flight_per_lane']} loads/lane)")
+
+    def gemv(i):
+        ok(tl.litenn_hip_mul_mat_q(0, fmt, weights[i % n_buffers].ptr, n, k, x.ptr, 0, 1, y.ptr, None, 0, C.byref(opts)))
+
+    out["gemv_with_stamps_us"] = round(per_launch_us(gemv), 3)
+    # the same kernel fetching its rows and reading them from LDS without multiplying them
+    ok(tl.litenn_hip_gemv_trace_skip_arithmetic(1))
+    out["gemv_with_stamps_no_arithmetic_us"] = round(per_launch_us(gemv), 3)
+    ok(tl.litenn_hip_gemv_trace_skip_arithmetic(0))
+    log(f"[bench] microbench: streaming kernel with stamps {out['gemv_with_stamps_us']} us/launch, its row traffic "
+        f"alone (no arithmetic) {out['gemv_with_stamps_no_arithmetic_us']} us/launch")
+    # the timeline of one launch in the middle of a replay: stamps are cleared by the read, then one
+    # rotation runs and the last launch's stamps (every launch overwrites them) are read back
+    slots = 16
+    waves = 256 * 8
+    buf = (C.c_ulonglong * (waves * slots))()
+    ok(tl.litenn_hip_gemv_trace_read(buf, waves * slots))
+    acc = []
+    for _ in range(8):
+        for i in range(n_buffers):
+            gemv(i)
+        ok(tl.litenn_hip_gemv_trace_read(buf, waves * slots))
+        t = np.frombuffer(buf, np.uint64).reshape(waves, slots).astype(np.float64)
+        t = np.where(t == 0, np.nan, t)
+        acc.append((t - np.nanmin(t[:, 0])) * 0.01)  # 100 MHz ticks -> us after the first wavefront's entry
+    t = np.stack(acc)  # [launch, wavefront, slot]
+    names = ["entry", "activations written to LDS", "barrier passed", "activations in registers"] + \
+            [f"row {r} landed" for r in range(11)] + ["last row consumed"]
+    timeline = []
+    for slot, name in enumerate(names):
+        col = t[:, :, slot]
+        if np.all(np.isnan(col)):
+            continue
+        timeline.append({"point": name, "mean_us": round(float(np.nanmean(col)), 2),
+                         "earliest_us": round(float(np.nanmean(np.nanmin(col, axis=1))), 2),
+                         "latest_us": round(float(np.nanmean(np.nanmax(col, axis=1))), 2)})
+        log(f"[bench] microbench: {name:28s} mean {timeline[-1]['mean_us']:5.2f} us  earliest "
+            f"{timeline[-1]['earliest_us']:5.2f}  latest {timeline[-1]['latest_us']:5.2f}")
+    out["gemv_timeline"] = timeline
+    out["gemv_timeline_note"] = ("us after the launch's first wavefront entered the kernel, averaged over 8 launches x "
+                                 "2048 wavefronts; earliest / latest are the per-launch extremes, averaged")
+    for w in weights:
+        w.free()
+    for tns in (x, y, sink):
+        tns.free()
+    stream.destroy()
+    return out
+
+
 def bench_cpu_baseline(fmt, n, k, budget_s=12.0):
     """The reference CPU path for the same GEMV, restated by the CPU checker: weights dequantised
     once to f32 [k, n] (the lowering's one-off cost, not timed), then the single-threaded i-k-j
@@ -240,6 +359,8 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill (batched matmul) measurements")
     ap.add_argument("--gemm-case", default=None, help="run only this prefill case, e.g. Q4_K:512")
+    ap.add_argument("--microbench", action="store_true",
+                    help="also measure an empty kernel, a read-only kernel and the GEMV's in-kernel timeline")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch a known-size streaming kernel (profiler counter calibration)")
     args = ap.parse_args()
@@ -295,6 +416,8 @@ def main() -> int:
             "kernel": "gemv_stream_kernel<Q4_KUnit, 2, true>",
         },
     }
+    if args.microbench:
+        line["microbench"] = microbench(ln, hiprt, Q4_K, n, k, args.buffers)
     if not args.no_cpu:
         s_per_call, calls = bench_cpu_baseline(Q4_K, n, k)
         line["cpu_baseline"] = {

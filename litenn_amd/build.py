@@ -10,6 +10,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "liblitenn_hip.so")
+# the same library with the streaming GEMV's timeline stamps compiled in, plus the measurement
+# kernels of csrc/microbench.hip; only bench.py --microbench loads it
+TRACE_LIB_PATH = os.path.join(LIB_DIR, "liblitenn_hip_trace.so")
 
 SOURCES = ["api.hip", "gemv.hip", "gemm.hip", "glue.hip", "attn_tile.hip", "primitives.hip", "llama.hip", "gguf.hip"]
 
@@ -34,10 +37,12 @@ def build(verbose: bool = True, jobs: int = 6) -> str:
     obj_dir = os.path.join(HERE, "build")
     os.makedirs(obj_dir, exist_ok=True)
     procs, objs = [], []
-    for src in SOURCES:
-        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
-        objs.append(obj)
-        cmd = [hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    trace_units = [("gemv.hip", "gemv_trace.o", ["-DLITENN_GEMV_TRACE"]), ("microbench.hip", "microbench.o", [])]
+    for src, obj_name, extra in [(s, s.replace(".hip", ".o"), []) for s in SOURCES] + trace_units:
+        obj = os.path.join(obj_dir, obj_name)
+        if not extra and src in SOURCES:
+            objs.append(obj)
+        cmd = [hipcc(), *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
@@ -56,6 +61,13 @@ def build(verbose: bool = True, jobs: int = 6) -> str:
         raise RuntimeError("hipcc failed")
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc",
            "-Wl,--version-script=" + os.path.join(CSRC, "exports.map"), *objs, "-o", LIB_PATH]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    trace_objs = [os.path.join(obj_dir, "gemv_trace.o") if o.endswith(os.sep + "gemv.o") else o for o in objs]
+    trace_objs.append(os.path.join(obj_dir, "microbench.o"))
+    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc",
+           "-Wl,--version-script=" + os.path.join(CSRC, "exports.map"), *trace_objs, "-o", TRACE_LIB_PATH]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)

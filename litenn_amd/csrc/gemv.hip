@@ -972,11 +972,17 @@ namespace litenn_hip
 		constexpr size_t kStreamLdsLimit = 160 * 1024;
 
 #ifdef LITENN_GEMV_TRACE
-		__device__ unsigned long long g_trace[4096 * 16];
+		// Timeline build (lib/liblitenn_hip_trace.so only): lane 0 of every wavefront stamps the
+		// card's constant 100 MHz clock, which all compute units share, at fixed points of the
+		// streaming kernel.  Slots: 0 entry, 1 activations written to LDS, 2 barrier passed,
+		// 3 activations in registers, 4 + r row r landed (r < 11), 15 last row consumed.
+		constexpr int kTraceWaves = 4096, kTraceSlots = 16;
+		__device__ unsigned long long g_trace[kTraceWaves * kTraceSlots];
+		__device__ int g_trace_skip_arithmetic = 0; // 1: rows are fetched and read from LDS, not multiplied
 #define GEMV_TRACE(slot)                                                                                               \
 	if (lane == 0)                                                                                                     \
 	{                                                                                                                  \
-		g_trace[(blockIdx.x * 8 + wave) % 4096 * 16 + (slot)] = __builtin_readcyclecounter();                          \
+		g_trace[(blockIdx.x * 8 + wave) % kTraceWaves * kTraceSlots + (slot)] = __builtin_amdgcn_s_memrealtime();      \
 	}
 #else
 #define GEMV_TRACE(slot)
@@ -1926,3 +1932,36 @@ namespace litenn_hip
 		                                                          row_bytes(fmt, k), ids, out, err_flag);
 	}
 } // namespace litenn_hip
+
+#ifdef LITENN_GEMV_TRACE
+// Timeline build only: copies the stamps of the last streaming launch to the host
+// ([wavefront][slot] of 100 MHz clock ticks, 0 where a slot was not reached) and clears them.
+extern "C" int litenn_hip_gemv_trace_read(unsigned long long* dst, size_t entries)
+{
+	using namespace litenn_hip;
+	constexpr size_t total = static_cast<size_t>(kTraceWaves) * kTraceSlots;
+	if (!dst || entries > total)
+	{
+		return fail("read the GEMV timeline", "destination is null or asks for more than 4096 x 16 entries");
+	}
+	LITENN_HIP_TRY("read the GEMV timeline", hipDeviceSynchronize());
+	LITENN_HIP_TRY("read the GEMV timeline",
+	               hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_trace), entries * sizeof(unsigned long long)));
+	void* dev = nullptr;
+	LITENN_HIP_TRY("read the GEMV timeline", hipGetSymbolAddress(&dev, HIP_SYMBOL(g_trace)));
+	LITENN_HIP_TRY("read the GEMV timeline", hipMemset(dev, 0, total * sizeof(unsigned long long)));
+	return 0;
+}
+
+// Timeline build only: 1 makes the streaming kernel fetch its rows and read them from LDS without
+// multiplying them (results are then meaningless), which times the row traffic alone; 0 restores it.
+extern "C" int litenn_hip_gemv_trace_skip_arithmetic(int skip)
+{
+	using namespace litenn_hip;
+	const int value = skip ? 1 : 0;
+	LITENN_HIP_TRY("set the GEMV timeline switch", hipDeviceSynchronize());
+	LITENN_HIP_TRY("set the GEMV timeline switch",
+	               hipMemcpyToSymbol(HIP_SYMBOL(g_trace_skip_arithmetic), &value, sizeof(value)));
+	return 0;
+}
+#endif
