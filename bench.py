@@ -4,11 +4,22 @@
 Headline (`value`): the Q4_K decode GEMV at K=4096, N=14336, batch 1, as algorithmic HBM GB/s.
 One "step" is one GEMV launch.  The steps rotate over distinct weight buffers (> 512 MB in
 total) so every launch streams its 33 MB from HBM rather than from the 256 MB last-level cache.
-The same JSON line carries the roofline object of that kernel, the CPU baseline (the CPU
-checker's restatement of the reference path, timed on this host) and the greedy decode rate of
-the random-init 7B-shape Q4_0 model (prompt 128, 256 new tokens).
+The same JSON line carries
+  * `roofline`: that kernel against the 8 TB/s HBM peak;
+  * `cpu_baseline`: the CPU checker's restatement of the reference path timed on this host (one
+    thread; with the Interpreter's weight copy; the one-off dequantisation; an all-cores form
+    that is not the reference);
+  * `gemv_configs`: the Q8_0 4096 x 4096 and the Q4_0 / Q4_K FFN-shape GEMVs, each with a roofline;
+  * `prefill_gemm`: the matrix-core GEMM at M = 16 / 64 / 512;
+  * `decode`: greedy decode of the random-init 7B-shape Q4_0 model (prompt 128, 256 new tokens),
+    with the CPU checker's tokens per second beside it;
+  * `decode_8b`: the 8B GQA shape with mixed Q4_K / Q6_K weights, prompt 512 + 512 tokens at
+    context 4096;
+  * with --microbench, `microbench`: an empty kernel, a read-only kernel and the GEMV's in-kernel
+    timeline.
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-decode] [--no-cpu]
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-decode] [--no-cpu] [--no-gemm]
+       [--no-configs] [--microbench]
 """
 from __future__ import annotations
 
@@ -24,10 +35,20 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
-# HBM bytes one launch of the headline GEMV moves, from the profiler's FETCH_SIZE / WRITE_SIZE
-# counters scaled by a known-size copy (profiles/gemv_q4_k_14336x4096_hbm_traffic.txt); it is a
-# property of the kernel and the shape, not re-measured by this script.
-GEMV_Q4_K_14336x4096_TRAFFIC_BYTES = 33291725
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "gemv_q4_k_14336x4096_hbm_traffic.txt")
+
+
+def measured_traffic_bytes():
+    """HBM bytes one launch of the headline GEMV moves, as the committed profiler summary states
+    them (rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a known-size copy); a property of the kernel
+    and the shape, not re-measured by this script.  None when the summary is not there."""
+    import re
+    try:
+        with open(TRAFFIC_SUMMARY) as f:
+            m = re.search(r"GEMV traffic per launch:.*= (\d+) bytes", f.read())
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
 
 
 def log(*a):
@@ -289,38 +310,81 @@ def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=125):
     return out
 
 
-def bench_cpu_baseline(fmt, n, k, budget_s=12.0):
-    """The reference CPU path for the same GEMV, restated by the CPU checker: weights dequantised
-    once to f32 [k, n] (the lowering's one-off cost, not timed), then the single-threaded i-k-j
-    MatMul of src/LiteNN/Device.h:645-658 per call."""
+def bench_cpu_baseline(fmt, n, k, budget_s=8.0):
+    """The reference CPU path for the same GEMV, restated by the CPU checker, timed on this host:
+      * one-off: block dequantisation to f32 [n, k] and the transpose to [k, n] that the lowering does
+        once per graph (tools/gguf/LLaMABuilder.cpp:144-150, 225-230);
+      * per call, one thread: the i-k-j MatMul of src/LiteNN/Device.h:645-658 on that f32 matrix;
+      * per call, one thread, with the copy of the weight variable the Interpreter makes at every
+        VariableRefNode first (src/LiteNN/Runtime/Interpreter.h:325-329);
+      * not the reference: the checker's OpenMP form (rows dequantised on the fly, all cores)."""
     from litenn_amd import synth
     from oracle import oracle as orc
     orc.set_threads(1)
     wq = synth.quant_weights(fmt, n, k, 1)
     x = synth.activations(1, k, 2)
+    t0 = time.perf_counter()
     w_kn = orc.transpose(orc.dequantize(fmt, wq, n, k))
+    dequant_s = time.perf_counter() - t0
     orc.matmul_ikj(x, w_kn)  # warm
-    calls, t0 = 0, time.perf_counter()
-    while True:
-        orc.matmul_ikj(x, w_kn)
-        calls += 1
-        dt = time.perf_counter() - t0
-        if dt > budget_s or calls >= 2000:
-            break
-    return dt / calls, calls
+
+    def timed(fn, budget):
+        calls, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            calls += 1
+            dt = time.perf_counter() - t0
+            if dt > budget or calls >= 2000:
+                return dt / calls, calls
+
+    s_per_call, calls = timed(lambda: orc.matmul_ikj(x, w_kn), budget_s)
+    s_with_copy, calls_copy = timed(lambda: orc.matmul_ikj(x, w_kn.copy()), budget_s / 2)
+    cores = os.cpu_count() or 1
+    orc.set_threads(cores)
+    orc.mul_mat_q(fmt, wq, n, k, x, rowwise=True)
+    s_omp, calls_omp = timed(lambda: orc.mul_mat_q(fmt, wq, n, k, x, rowwise=True), budget_s / 2)
+    return {"s_per_call": s_per_call, "calls": calls, "s_with_copy": s_with_copy, "calls_copy": calls_copy,
+            "dequant_s": dequant_s, "s_omp": s_omp, "calls_omp": calls_omp, "omp_threads": cores}
 
 
-def bench_decode(ln, n_prompt=128, n_new=256, seed=4, model_name="7b"):
+ORACLE_TENSOR_IDS = {"token_embd": 0, "output": 1, "attn_q": 2, "attn_k": 3, "attn_v": 4, "attn_output": 5,
+                     "ffn_gate": 6, "ffn_up": 7, "ffn_down": 8, "output_norm": 9, "attn_norm": 10, "ffn_norm": 11}
+
+
+def cpu_decode_rate(cfg, tensors, prompt, steps=4):
+    """Tokens per second of the CPU checker's decoder on the same model (all cores, rows
+    dequantised on the fly; the reference's own interpreter is single-threaded on f32 weights
+    dequantised at lowering): `steps` single-token evaluations behind a two-token prompt."""
+    from oracle import oracle as orc
+    cores = os.cpu_count() or 1
+    orc.set_threads(cores)
+    m = orc.LLaMA(cfg.block_count, cfg.embedding_length, cfg.head_count, cfg.head_count_kv, cfg.feed_forward_length,
+                  cfg.vocab, cfg.context_length, rms_eps=cfg.rms_eps, rope_base=cfg.rope_freq_base,
+                  rope_freq_scale=cfg.rope_freq_scale, rope_dims=cfg.rope_dimension_count, kv_f16=True)
+    for kind, layer, fmt, payload, n, k in tensors:
+        m.set_tensor(ORACLE_TENSOR_IDS[kind], layer, fmt, payload, n, k)
+    logits = m.eval([int(prompt[0])], all_logits=False)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        logits = m.eval([int(np.argmax(logits))], all_logits=False)
+    dt = time.perf_counter() - t0
+    return steps / dt, cores
+
+
+def bench_decode(ln, n_prompt=128, n_new=256, seed=4, model_name="7b", cpu_steps=0):
     from litenn_amd import synth
     from litenn_amd.formats import DT_F16
     if model_name == "8b":
-        cfg = synth.llama_8b_gqa_mixed(context_length=n_prompt + n_new)
+        cfg = synth.llama_8b_gqa_mixed(context_length=max(4096, n_prompt + n_new))
     else:
         cfg = synth.llama_7b_q4_0(context_length=n_prompt + n_new)
     t0 = time.perf_counter()
     model = ln.LLaMA.from_config(cfg, kv_dtype=DT_F16)
+    tensors = []
     for item in synth.llama_tensors(cfg, seed):
         model.set_tensor(*item)
+        if cpu_steps:
+            tensors.append(item)
     log(f"[bench] {cfg.name} resident after {time.perf_counter() - t0:.1f} s")
     prompt = synth.prompt_tokens(cfg, n_prompt, seed)
     model.generate(prompt, 8, precise=False)  # warm-up: captures the step graph
@@ -332,8 +396,9 @@ def bench_decode(ln, n_prompt=128, n_new=256, seed=4, model_name="7b"):
     kv_bytes_mean = 2 * cfg.block_count * cfg.head_count_kv * cfg.head_dim * 2 * (n_prompt + n_new / 2)
     tok_s = steps / (decode_ms / 1e3)
     model.close()
-    return {
-        "workload": f"{cfg.name}: prompt {n_prompt} + {n_new} greedy tokens, fp16 KV cache, f32 activations",
+    out = {
+        "workload": f"{cfg.name}: prompt {n_prompt} + {n_new} greedy tokens, context {cfg.context_length}, "
+                    f"fp16 KV cache, f32 activations",
         "tokens_per_s": round(tok_s, 2),
         "ms_per_token": round(decode_ms / steps, 4),
         "prefill_ms": round(prefill_ms, 3),
@@ -341,8 +406,38 @@ def bench_decode(ln, n_prompt=128, n_new=256, seed=4, model_name="7b"):
         "weight_bytes_per_token": weight_bytes,
         "roofline_tokens_per_s": round(HBM_PEAK_GBPS * 1e9 / (weight_bytes + kv_bytes_mean), 1),
         "frac_of_hbm_roofline": round(tok_s * (weight_bytes + kv_bytes_mean) / (HBM_PEAK_GBPS * 1e9), 4),
+        "distinct_tokens": int(len(set(tokens.tolist()))),
         "first_tokens": tokens[:8].tolist(),
     }
+    if cpu_steps:
+        rate, cores = cpu_decode_rate(cfg, tensors, prompt, cpu_steps)
+        out["cpu_tokens_per_s"] = round(rate, 3)
+        out["cpu_baseline"] = {"value": round(rate, 3), "unit": "tokens/s", "cores": cores,
+                               "kind": "port-omp (not the reference)",
+                               "sample": f"{cpu_steps} single-token steps of the CPU checker's decoder on the same "
+                                         f"model, rows dequantised on the fly, {cores} threads"}
+    return out
+
+
+def bench_gemv_configs(ln, hiprt, steps=1600, warmup=64):
+    """The other single-row configurations: Q8_0 4096 x 4096 and the Q4_0 / Q4_K FFN shapes, each
+    with its own roofline object (rotating buffers of more than 512 MB in total)."""
+    from litenn_amd.formats import Q4_0, Q4_K, Q8_0, row_bytes
+    out = []
+    for name, fmt, n, k in (("Q8_0", Q8_0, 4096, 4096), ("Q4_0", Q4_0, 11008, 4096), ("Q4_0", Q4_0, 4096, 11008),
+                            ("Q4_K", Q4_K, 11008, 4096), ("Q4_K", Q4_K, 4096, 11008)):
+        w_bytes = n * row_bytes(fmt, k)
+        buffers = max(16, -(-540_000_000 // w_bytes))
+        ms, _ = bench_gemv(ln, hiprt, fmt, n, k, steps // buffers * buffers, warmup, buffers)
+        algo = w_bytes + 4 * k + 4 * n
+        gbps = algo / (ms * 1e-3) / 1e9
+        out.append({"format": name, "n": n, "k": k, "batch": 1, "us": round(ms * 1e3, 3), "buffers": buffers,
+                    "algorithmic_bytes": algo,
+                    "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                 "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None}})
+        log(f"[bench] {name} GEMV {n}x{k}: {ms * 1e3:.2f} us/launch, {gbps:.0f} GB/s = "
+            f"{100 * gbps / HBM_PEAK_GBPS:.1f}% of HBM peak")
+    return out
 
 
 def main() -> int:
@@ -352,6 +447,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--buffers", type=int, default=16)
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="skip the other single-row GEMV configurations")
     ap.add_argument("--decode-prompt", type=int, default=128, help="prompt length of the decode run")
     ap.add_argument("--decode-new", type=int, default=256, help="tokens generated by the decode run")
     ap.add_argument("--decode-model", choices=["7b", "8b"], default="7b",
@@ -410,7 +506,7 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": GEMV_Q4_K_14336x4096_TRAFFIC_BYTES,
+            "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": measured_traffic_bytes(),
             "traffic_unit": "bytes/launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
             "algorithmic_bytes": algo_bytes,
             "kernel": "gemv_stream_kernel<Q4_KUnit, 2, true>",
@@ -419,20 +515,42 @@ def main() -> int:
     if args.microbench:
         line["microbench"] = microbench(ln, hiprt, Q4_K, n, k, args.buffers)
     if not args.no_cpu:
-        s_per_call, calls = bench_cpu_baseline(Q4_K, n, k)
+        c = bench_cpu_baseline(Q4_K, n, k)
         line["cpu_baseline"] = {
-            "value": round(algo_bytes / s_per_call / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{calls} calls of the same {n}x{k} GEMV: weights dequantised once to f32 [k,n], then the "
-                      f"single-threaded i-k-j MatMul ({s_per_call * 1e3:.1f} ms/call); host has {os.cpu_count()} "
-                      f"logical CPUs",
-            "ms_per_step": round(s_per_call * 1e3, 3),
+            "value": round(algo_bytes / c["s_per_call"] / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{c['calls']} calls of the same {n}x{k} GEMV: weights dequantised once to f32 [k,n], then the "
+                      f"single-threaded i-k-j MatMul ({c['s_per_call'] * 1e3:.1f} ms/call); host has "
+                      f"{os.cpu_count()} logical CPUs",
+            "ms_per_step": round(c["s_per_call"] * 1e3, 3),
+            "with_weight_copy": {"value": round(algo_bytes / c["s_with_copy"] / 1e9, 4), "unit": "GB/s", "cores": 1,
+                                 "ms_per_step": round(c["s_with_copy"] * 1e3, 3),
+                                 "sample": f"{c['calls_copy']} calls, each preceded by the copy of the f32 weight "
+                                           f"the reference's Interpreter makes per VariableRefNode"},
+            "dequantise_once_ms": round(c["dequant_s"] * 1e3, 1),
+            "all_cores": {"value": round(algo_bytes / c["s_omp"] / 1e9, 4), "unit": "GB/s", "cores": c["omp_threads"],
+                          "kind": "port-omp (not the reference)", "ms_per_step": round(c["s_omp"] * 1e3, 3),
+                          "sample": f"{c['calls_omp']} calls of the checker's OpenMP form (rows dequantised on the "
+                                    f"fly, same arithmetic per output)"},
         }
-        log(f"[bench] CPU baseline: {s_per_call * 1e3:.1f} ms/call over {calls} calls")
+        log(f"[bench] CPU baseline: {c['s_per_call'] * 1e3:.1f} ms/call on one thread, "
+            f"{c['s_with_copy'] * 1e3:.1f} ms with the weight copy, dequantisation once {c['dequant_s'] * 1e3:.0f} ms, "
+            f"{c['s_omp'] * 1e3:.1f} ms/call on {c['omp_threads']} threads (not the reference)")
+    if not args.no_configs:
+        line["gemv_configs"] = bench_gemv_configs(ln, hiprt)
     if not args.no_gemm:
         line["prefill_gemm"] = bench_prefill_gemm(ln, hiprt, args.gemm_case)
     if not args.no_decode:
-        line["decode"] = bench_decode(ln, args.decode_prompt, args.decode_new, model_name=args.decode_model)
-        log(f"[bench] decode: {line['decode']['tokens_per_s']} tok/s")
+        cpu_steps = 0 if args.no_cpu else 4
+        if args.decode_model == "8b":
+            line["decode_8b"] = bench_decode(ln, args.decode_prompt, args.decode_new, model_name="8b")
+        else:
+            line["decode"] = bench_decode(ln, args.decode_prompt, args.decode_new, model_name="7b",
+                                          cpu_steps=cpu_steps)
+            log(f"[bench] decode: {line['decode']['tokens_per_s']} tok/s"
+                + (f" (CPU checker: {line['decode']['cpu_tokens_per_s']} tok/s)" if cpu_steps else ""))
+            line["decode_8b"] = bench_decode(ln, 512, 512, model_name="8b")
+        log(f"[bench] decode 8B shape: {line['decode_8b']['tokens_per_s']} tok/s, prompt pass "
+            f"{line['decode_8b']['prefill_ms']} ms")
     print(json.dumps(line), flush=True)
     return 0
 
