@@ -300,6 +300,11 @@ def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=125):
         log(f"[bench] microbench: {name:28s} mean {timeline[-1]['mean_us']:5.2f} us  earliest "
             f"{timeline[-1]['earliest_us']:5.2f}  latest {timeline[-1]['latest_us']:5.2f}")
     out["gemv_timeline"] = timeline
+    # wavefronts 0-3 of a workgroup are the first on their SIMD, 4-7 share it with them
+    by_wave = np.nanmean(t[:, :, 15].reshape(len(acc), -1, 8), axis=(0, 1))
+    out["last_row_consumed_by_wavefront_index_us"] = [round(float(v), 2) for v in by_wave]
+    log("[bench] microbench: last row consumed, by wavefront index within the workgroup: "
+        + " ".join(f"{v:.2f}" for v in by_wave))
     out["gemv_timeline_note"] = ("us after the launch's first wavefront entered the kernel, averaged over 8 launches x "
                                  "2048 wavefronts; earliest / latest are the per-launch extremes, averaged")
     for w in weights:
