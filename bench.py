@@ -80,28 +80,45 @@ def bench_gemv(ln, hiprt, fmt, n, k, steps, warmup, n_buffers, seed=1):
     for i in range(warmup):
         launch(i)
     stream.synchronize()
-    # one rotation captured as a graph keeps the host out of the timed region; the remainder
-    # (steps mod n_buffers) is launched directly so exactly `steps` kernels run
-    stream.begin_capture()
-    for i in range(n_buffers):
-        launch(i)
-    graph = stream.end_capture()
-    graph.launch(stream)  # untimed: first replay uploads the graph
-    stream.synchronize()
+    # The launches are captured as graphs so that the host stays out of the timed region.  Starting a
+    # graph costs about 13 us on the device whatever it holds (measured with empty kernels: 14.4 us
+    # for a graph of one, 1.58 us per kernel in a graph of 256, 1.53 us per kernel launched
+    # directly), so a graph holds up to 16 rotations; exactly `steps` kernels run, all from graphs.
+    # A short run (fewer than 64 steps) is launched directly instead: the host issues a launch in
+    # about 4 us, less than one takes, and the graph's start would weigh on so few kernels.
+    graph_len = min(steps, 16 * n_buffers) if steps >= 64 else 0
+
+    def capture(count):
+        stream.begin_capture()
+        for i in range(count):
+            launch(i)
+        g = stream.end_capture()
+        g.launch(stream)  # untimed: the first replay uploads the graph
+        stream.synchronize()
+        return g
+
+    graph = capture(graph_len) if graph_len else None
+    rest = capture(steps % graph_len) if graph_len and steps % graph_len else None
     e0, e1 = hiprt.Event(), hiprt.Event()
     hiprt.device_synchronize()
     t0 = time.perf_counter()
     e0.record(stream)
-    for _ in range(steps // n_buffers):
-        graph.launch(stream)
-    for i in range(steps % n_buffers):
-        launch(i)
+    if graph is None:
+        for i in range(steps):
+            launch(i)
+    else:
+        for _ in range(steps // graph_len):
+            graph.launch(stream)
+        if rest is not None:
+            rest.launch(stream)
     e1.record(stream)
     stream.synchronize()
     hiprt.device_synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     event_ms = e0.elapsed_ms(e1)
-    graph.destroy()
+    for g in (graph, rest):
+        if g is not None:
+            g.destroy()
     result = y.numpy()
     assert np.all(np.isfinite(result))
     for w in weights:
@@ -191,7 +208,7 @@ def bench_prefill_gemm(ln, hiprt, only=None):
     return out
 
 
-def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=125):
+def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=8):
     """What the headline GEMV's time is made of, measured on the same card with the same rotation of
     weight buffers and the same graph replay (lib/liblitenn_hip_trace.so: the library with timeline
     stamps compiled into the streaming kernel, plus csrc/microbench.hip):
@@ -208,7 +225,7 @@ def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=125):
     tl.litenn_hip_last_error.restype = C.c_char_p
     vp, sz = C.c_void_p, C.c_size_t
     tl.litenn_hip_mul_mat_q.argtypes = [C.c_int, C.c_int, vp, sz, sz, vp, C.c_int, sz, vp, vp, C.c_uint, C.POINTER(Exec)]
-    tl.litenn_hip_mb_empty.argtypes = [vp]
+    tl.litenn_hip_mb_empty.argtypes = [C.c_int, C.c_int, sz, vp]
     tl.litenn_hip_mb_read.argtypes = [vp, sz, C.c_int, C.c_int, vp, vp]
     tl.litenn_hip_gemv_trace_read.argtypes = [vp, sz]
     tl.litenn_hip_gemv_trace_skip_arithmetic.argtypes = [C.c_int]
@@ -226,13 +243,15 @@ def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=125):
     stream = hiprt.Stream()
     opts = Exec(stream.handle, 0)
 
+    graph_len = 16 * n_buffers
+
     def per_launch_us(launch):
-        """One rotation captured as a graph, replayed; HIP events on the stream."""
+        """16 rotations captured as one graph, replayed; HIP events on the stream."""
         for i in range(n_buffers):
             launch(i)
         stream.synchronize()
         stream.begin_capture()
-        for i in range(n_buffers):
+        for i in range(graph_len):
             launch(i)
         graph = stream.end_capture()
         graph.launch(stream)
@@ -243,12 +262,15 @@ def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=125):
             graph.launch(stream)
         e1.record(stream)
         stream.synchronize()
-        us = e0.elapsed_ms(e1) * 1e3 / (replays * n_buffers)
+        us = e0.elapsed_ms(e1) * 1e3 / (replays * graph_len)
         graph.destroy()
         return us
 
-    out = {"rotation": f"{n_buffers} buffers x {w_bytes} B, graph of {n_buffers} launches replayed {replays} times"}
-    out["empty_kernel_us"] = round(per_launch_us(lambda i: ok(tl.litenn_hip_mb_empty(stream.handle))), 3)
+    out = {"rotation": f"{n_buffers} buffers x {w_bytes} B, graph of {graph_len} launches replayed {replays} times"}
+    out["empty_kernel_us"] = round(per_launch_us(lambda i: ok(tl.litenn_hip_mb_empty(256, 512, 90 * 1024,
+                                                                                      stream.handle))), 3)
+    out["empty_kernel_one_workgroup_us"] = round(per_launch_us(lambda i: ok(tl.litenn_hip_mb_empty(1, 64, 0,
+                                                                                                    stream.handle))), 3)
     reads = []
     for blocks in (256, 512, 1024, 2048):
         for depth in (2, 4, 8):
@@ -259,7 +281,8 @@ def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=125):
     best = min(reads, key=lambda r: r["us"])
     out["read_kernel_best"] = best
     out["read_kernel_all"] = reads
-    log(f"[bench] microbench: empty kernel {out['empty_kernel_us']} us/launch; read-only kernel best "
+    log(f"[bench] microbench: empty kernel {out['empty_kernel_us']} us/launch (one workgroup of 64 threads: "
+        f"{out['empty_kernel_one_workgroup_us']}); read-only kernel best "
         f"{best['us']} us = {best['gbps']} GB/s ({best['blocks']} workgroups, {best['loads_in_flight_per_lane']} loads/lane)")
 
     def gemv(i):

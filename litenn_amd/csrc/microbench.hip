@@ -51,11 +51,17 @@ namespace litenn_hip
 	} // namespace
 } // namespace litenn_hip
 
-// One launch of the kernel that does nothing (256 workgroups of 512 threads, like the GEMV).
-extern "C" int litenn_hip_mb_empty(void* stream)
+// One launch of the kernel that does nothing: `blocks` workgroups of `threads` threads (the GEMV
+// launches 256 of 512) that each reserve `lds_bytes` of LDS.
+extern "C" int litenn_hip_mb_empty(int blocks, int threads, size_t lds_bytes, void* stream)
 {
 	using namespace litenn_hip;
-	mb_empty_kernel<<<dim3(256), dim3(512), 0, static_cast<hipStream_t>(stream)>>>();
+	if (blocks < 1 || threads < 64 || threads > 512 || lds_bytes > 160 * 1024)
+	{
+		return fail("launch the empty kernel", "geometry out of range");
+	}
+	allow_dynamic_lds(reinterpret_cast<const void*>(&mb_empty_kernel), 160 * 1024);
+	mb_empty_kernel<<<dim3(blocks), dim3(threads), lds_bytes, static_cast<hipStream_t>(stream)>>>();
 	LITENN_HIP_TRY("launch the empty kernel", hipGetLastError());
 	return 0;
 }
