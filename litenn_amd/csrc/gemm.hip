@@ -1183,6 +1183,268 @@ namespace litenn_hip
 			}
 		}
 
+		// ---- the GEMM for few activation rows ------------------------------------------------------
+		// With 16 or 32 activation rows the product is a stream of the weights, like the single-row
+		// GEMV, and is built like it: one workgroup of eight wavefronts per CU, always a single round,
+		// each workgroup owning a run of consecutive weight rows.  The rows are walked in tiles of 16;
+		// wavefront w multiplies the tile's chunks [w CPW, (w + 1) CPW) of K, whose activation
+		// fragments (already fp16, in MFMA order) it holds in registers for the whole launch, and
+		// keeps PD tiles' worth of its slice of the raw blocks in flight towards its LDS slots with
+		// direct-to-LDS loads.  The eight partial products of a tile meet in LDS and are added in
+		// wavefront order, so the result does not depend on scheduling.  One launch, no second pass
+		// over y, every weight byte read once.
+		constexpr int kStreamWaves = 8;
+		constexpr int kStreamTilesInFlight = 2;
+
+		struct GemmStreamArgs
+		{
+			const uint8_t* w;
+			float* y;
+			const uint8_t* xf;
+			const float* unscale;
+			const float* residual;
+			int n, k, m, m_tiles;
+			size_t row_bytes;
+			int rows_per_block; // consecutive weight rows of a workgroup, a multiple of 4
+			int round_tiles;    // tiles whose partial products LDS holds before they are added and stored
+		};
+
+		template <typename F, int CPW>
+		constexpr int stream_slot_bytes()
+		{
+			return 16 * 16 * fetch::gemm_weight_pieces(CPW * F::kChunkBytes, F::kAligned16);
+		}
+
+		template <typename F, int MT, int CPW>
+		__global__ __launch_bounds__(64 * kStreamWaves) void gemm_stream_kernel(const GemmStreamArgs a)
+		{
+			constexpr int PD = kStreamTilesInFlight;
+			constexpr int kSliceBytes = CPW * F::kChunkBytes; // a wavefront's share of one row
+			constexpr int P = fetch::gemm_weight_pieces(kSliceBytes, F::kAligned16);
+			constexpr int kRowStride = 16 * P;
+			constexpr int kSlotBytes = 16 * kRowStride;
+			constexpr int kWLoads = (16 * P + 63) / 64;
+			static_assert(kSlotBytes == stream_slot_bytes<F, CPW>(), "slot size");
+			static_assert(PD * kWLoads <= 63, "vmcnt range");
+			extern __shared__ __attribute__((aligned(16))) uint8_t lds[]; // [waves][PD][slot] [round][waves][MT][1 KB]
+			const int lane = threadIdx.x & 63;
+			const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+			const int r = lane & 15, g = lane >> 4;
+			const int chunks = a.k / kChunk;
+			const int row0 = static_cast<int>(blockIdx.x) * a.rows_per_block;
+			const int block_rows = min(a.rows_per_block, a.n - row0);
+			const int last_row = row0 + block_rows - 1;
+			const int tiles = (block_rows + 15) >> 4;
+			const uint32_t lds_base =
+			    static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const uint8_t*)(lds)));
+			const uint32_t slots_lds = lds_base + wave * (PD * kSlotBytes);
+			const int part_base = kStreamWaves * PD * kSlotBytes;
+
+			// ---- weight requests: piece p = 64 i + lane of a slot is piece p % P of tile row p / P.
+			// Rows past the workgroup's run re-read its last row (same bytes as a neighbouring lane:
+			// no further traffic); their products are never stored.  The address arithmetic is the
+			// matrix-core GEMM's (fetch_model.hpp) with the wavefront's slice in the place of a chunk.
+			int w_row[kWLoads], w_piece[kWLoads];
+			bool w_issued[kWLoads];
+#pragma unroll
+			for (int i = 0; i < kWLoads; ++i)
+			{
+				const fetch::GemmWeightRequest rq = fetch::gemm_weight_request(i, lane, 1, P);
+				w_row[i] = rq.row;
+				w_piece[i] = rq.offset;
+				w_issued[i] = rq.issued;
+			}
+			const auto issue_tile = [&](int t, int slot) {
+#pragma unroll
+				for (int i = 0; i < kWLoads; ++i)
+				{
+					if (64 * (i + 1) <= 16 * P || w_issued[i])
+					{
+						const int row = fetch::gemm_weight_row(row0 + 16 * t, w_row[i], last_row + 1);
+						const uint8_t* row_start = a.w + static_cast<size_t>(row) * a.row_bytes;
+						const uint8_t* src = reinterpret_cast<const uint8_t*>(fetch::gemm_weight_piece(
+						    reinterpret_cast<uintptr_t>(row_start), wave, kSliceBytes, F::kAligned16, w_piece[i]));
+						const uint32_t dst = slots_lds + slot * kSlotBytes + i * 1024;
+						asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+						             :
+						             : "s"(dst), "v"(src)
+						             : "memory", "m0");
+					}
+				}
+			};
+#pragma unroll
+			for (int t = 0; t < PD; ++t)
+			{
+				if (t < tiles) // uniform
+				{
+					issue_tile(t, t);
+				}
+			}
+
+			// ---- this wavefront's activation fragments: chunks [wave CPW, (wave + 1) CPW), every step,
+			// MT tiles (a tile past the end repeats the last one; its products are not stored)
+			u32x4 b[CPW][8][MT];
+#pragma unroll
+			for (int ci = 0; ci < CPW; ++ci)
+			{
+#pragma unroll
+				for (int t = 0; t < MT; ++t)
+				{
+					const int mt = min(t, a.m_tiles - 1);
+					const uint8_t* tile = a.xf + (static_cast<size_t>(mt) * chunks + wave * CPW + ci) * kChunkTileBytes + lane * 16;
+#pragma unroll
+					for (int st = 0; st < 8; ++st)
+					{
+						b[ci][st][t] = *reinterpret_cast<const u32x4*>(tile + st * kFragBytes);
+					}
+				}
+			}
+
+			// the factor that undoes the pre-pass's scaling of this thread's activation row (the same row
+			// in every round: MT divides the number of wavefronts), fetched before the walk
+			const int my_mm = ((threadIdx.x >> 6) % MT) * 16 + (lane & 15);
+			float my_unscale = a.unscale[min(my_mm, 16 * a.m_tiles - 1)];
+			// The compiler's own wait for these loads must sit here, before the walk: inside the loop it
+			// would be repeated on every pass and wait for the tiles requested ahead as well.
+			asm volatile("" : "+v"(my_unscale));
+#pragma unroll
+			for (int ci = 0; ci < CPW; ++ci)
+			{
+#pragma unroll
+				for (int st = 0; st < 8; ++st)
+				{
+#pragma unroll
+					for (int t = 0; t < MT; ++t)
+					{
+						asm volatile("" : "+v"(b[ci][st][t]));
+					}
+				}
+			}
+			static_assert(kStreamWaves % MT == 0, "a thread keeps one activation row through the rounds");
+
+			const int round_tiles = a.round_tiles;
+			const bool vec_ok = (a.n & 3) == 0 && (reinterpret_cast<uintptr_t>(a.y) & 15) == 0 &&
+			                    (!a.residual || (reinterpret_cast<uintptr_t>(a.residual) & 15) == 0);
+			// adds the eight partial products of tiles [first, first + count) in wavefront order and stores them
+			const auto finish_round = [&](int first, int count) {
+				__syncthreads();
+				for (int idx = threadIdx.x; idx < count * MT * 64; idx += 64 * kStreamWaves)
+				{
+					const int ti = idx / (MT * 64), t = (idx >> 6) % MT, ln = idx & 63;
+					const uint8_t* src = lds + part_base + ((ti * kStreamWaves) * MT + t) * 1024 + ln * 16;
+					floatx4 sum = *reinterpret_cast<const floatx4*>(src);
+#pragma unroll
+					for (int wv = 1; wv < kStreamWaves; ++wv)
+					{
+						const floatx4 v = *reinterpret_cast<const floatx4*>(src + wv * MT * 1024);
+						sum.x += v.x, sum.y += v.y, sum.z += v.z, sum.w += v.w;
+					}
+					// D layout: lane holds activation row ln % 16 and weight rows 4 (ln / 16) + 0 .. 3
+					const int mm = t * 16 + (ln & 15);
+					const int n0 = row0 + 16 * (first + ti) + 4 * (ln >> 4);
+					if (mm < a.m && n0 <= last_row)
+					{
+						float* dst = a.y + static_cast<size_t>(mm) * a.n + n0;
+						const float* res = a.residual ? a.residual + static_cast<size_t>(mm) * a.n + n0 : nullptr;
+						const float us = my_unscale;
+						const float vals[4] = { sum.x * us, sum.y * us, sum.z * us, sum.w * us };
+						if (vec_ok && n0 + 3 <= last_row)
+						{
+							float4 out = { vals[0], vals[1], vals[2], vals[3] };
+							if (res)
+							{
+								const float4 rv = *reinterpret_cast<const float4*>(res);
+								out.x += rv.x, out.y += rv.y, out.z += rv.z, out.w += rv.w;
+							}
+							*reinterpret_cast<float4*>(dst) = out;
+						}
+						else
+						{
+#pragma unroll
+							for (int e = 0; e < 4; ++e)
+							{
+								if (n0 + e <= last_row)
+								{
+									dst[e] = res ? res[e] + vals[e] : vals[e];
+								}
+							}
+						}
+					}
+				}
+				__syncthreads();
+			};
+
+			int slot = 0, in_round = 0, round_first = 0;
+			for (int t = 0; t < tiles; ++t)
+			{
+				// tile t has landed once only the tiles requested after it are outstanding
+				if (t + PD - 1 < tiles)
+				{
+					vm_wait<(PD - 1) * kWLoads>();
+				}
+				else
+				{
+					vm_wait<0>();
+				}
+				const int row = fetch::gemm_weight_row(row0 + 16 * t, r, last_row + 1);
+				const int mis = fetch::gemm_weight_misalignment(
+				    reinterpret_cast<uintptr_t>(a.w + static_cast<size_t>(row) * a.row_bytes), wave, kSliceBytes, F::kAligned16);
+				lds_bytes_t mine = (lds_bytes_t)(lds) + wave * (PD * kSlotBytes) + slot * kSlotBytes + r * kRowStride + mis;
+				typename F::Raw raw[CPW];
+				typename F::Scale sc[CPW];
+#pragma unroll
+				for (int ci = 0; ci < CPW; ++ci)
+				{
+					raw[ci] = F::load(mine + ci * F::kChunkBytes, g);
+				}
+				// the slot is free once those reads have returned: refill it before the arithmetic
+				asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+				if (t + PD < tiles)
+				{
+					issue_tile(t + PD, slot);
+				}
+				floatx4 acc[MT];
+#pragma unroll
+				for (int mt = 0; mt < MT; ++mt)
+				{
+					acc[mt] = floatx4{ 0.0f, 0.0f, 0.0f, 0.0f };
+				}
+#pragma unroll
+				for (int ci = 0; ci < CPW; ++ci)
+				{
+					sc[ci] = F::prep(raw[ci], g);
+#pragma unroll
+					for (int st = 0; st < 8; ++st)
+					{
+						uint32_t pk[4];
+						F::frag(raw[ci], sc[ci], st, pk);
+						const u32x4 v = { pk[0], pk[1], pk[2], pk[3] };
+						const half8 av = __builtin_bit_cast(half8, v);
+#pragma unroll
+						for (int mt = 0; mt < MT; ++mt)
+						{
+							// D[i = weight row][j = activation row] += A[i][k] * B[k][j]
+							acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, __builtin_bit_cast(half8, b[ci][st][mt]), acc[mt],
+							                                                 0, 0, 0);
+						}
+					}
+				}
+#pragma unroll
+				for (int mt = 0; mt < MT; ++mt)
+				{
+					*reinterpret_cast<floatx4*>(lds + part_base + ((in_round * kStreamWaves + wave) * MT + mt) * 1024 + lane * 16) =
+					    acc[mt];
+				}
+				slot = slot + 1 == PD ? 0 : slot + 1;
+				if (++in_round == round_tiles || t + 1 == tiles)
+				{
+					finish_round(round_first, in_round);
+					round_first += in_round;
+					in_round = 0;
+				}
+			}
+		}
+
 #pragma clang diagnostic pop
 
 		struct GemmCall
@@ -1355,10 +1617,95 @@ namespace litenn_hip
 #undef LITENN_GEMM_CASE
 		}
 
+		// The streaming form takes a single matrix against at most 32 activation rows when K is a whole
+		// number of chunks per wavefront (2048 elements) whose fragments fit the registers and the slots
+		// fit LDS.  Returns false, launching nothing, otherwise.
+		template <typename F, int MT, int CPW>
+		bool launch_stream_variant(const GemmCall& c, int cus)
+		{
+			constexpr size_t slots = static_cast<size_t>(kStreamWaves) * kStreamTilesInFlight * stream_slot_bytes<F, CPW>();
+			constexpr size_t per_round_tile = static_cast<size_t>(kStreamWaves) * MT * 1024;
+			if constexpr (slots + per_round_tile > kLdsLimit)
+			{
+				return false;
+			}
+			else
+			{
+				GemmStreamArgs a{};
+				a.w = c.w[0];
+				a.y = c.y[0];
+				a.xf = c.xf;
+				a.unscale = c.unscale;
+				a.residual = c.residual;
+				a.n = c.n[0];
+				a.k = c.k;
+				a.m = c.m;
+				a.m_tiles = c.m_tiles;
+				a.row_bytes = c.row_bytes;
+				int rows = (c.n[0] + cus - 1) / cus;
+				rows = (rows + 3) / 4 * 4;
+				a.rows_per_block = rows;
+				const int blocks = (c.n[0] + rows - 1) / rows;
+				const int tiles = (rows + 15) / 16;
+				int round = static_cast<int>((kLdsLimit - slots) / per_round_tile);
+				round = std::max(1, std::min(std::min(round, tiles), 8));
+				a.round_tiles = round;
+				const size_t lds = slots + round * per_round_tile;
+				allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_stream_kernel<F, MT, CPW>), kLdsLimit);
+				gemm_stream_kernel<F, MT, CPW><<<dim3(blocks), dim3(64 * kStreamWaves), lds, c.stream>>>(a);
+				return true;
+			}
+		}
+
+		template <typename F>
+		bool launch_stream_form(const GemmCall& c, int cus)
+		{
+			static const int use_stream = env_int("LITENN_HIP_GEMM_STREAM", 1);
+			if (!use_stream || c.count != 1 || c.m_tiles > 2 || c.k % (kChunk * kStreamWaves) != 0)
+			{
+				return false;
+			}
+			const int cpw = c.k / (kChunk * kStreamWaves);
+			if (c.m_tiles == 1)
+			{
+				switch (cpw)
+				{
+				case 1: return launch_stream_variant<F, 1, 1>(c, cus);
+				case 2: return launch_stream_variant<F, 1, 2>(c, cus);
+				case 4: return launch_stream_variant<F, 1, 4>(c, cus);
+				default: return false;
+				}
+			}
+			switch (cpw)
+			{
+			case 1: return launch_stream_variant<F, 2, 1>(c, cus);
+			case 2: return launch_stream_variant<F, 2, 2>(c, cus);
+			default: return false;
+			}
+		}
+
 		template <typename F>
 		void launch_prepass_and_gemm(GemmCall& c, const float* x, const float* norm_w, double eps, const float* up,
 		                             uint8_t* xf, float* unscale, int m_pad, int cus)
 		{
+			if (c.m_tiles <= 2)
+			{
+				to_half_kernel<F><<<dim3(static_cast<unsigned>(m_pad)), dim3(256), 0, c.stream>>>(x, xf, unscale, c.m, c.k,
+				                                                                                 norm_w, eps, up);
+				if (launch_stream_form<F>(c, cus))
+				{
+					return;
+				}
+				choose_tile<F>(c, cus);
+				launch_format<F>(c);
+				if (c.k_splits > 1)
+				{
+					const size_t total = static_cast<size_t>(c.m) * c.n[0];
+					add_partial_kernel<<<dim3(static_cast<unsigned>((total / 4 + 255) / 256 + 1)), dim3(256), 0, c.stream>>>(
+					    c.y[0], c.partial, total, c.k_splits - 1);
+				}
+				return;
+			}
 			choose_tile<F>(c, cus);
 			to_half_kernel<F><<<dim3(static_cast<unsigned>(m_pad)), dim3(256), 0, c.stream>>>(x, xf, unscale, c.m, c.k,
 			                                                                                 norm_w, eps, up);

@@ -174,6 +174,107 @@ static void test_gemm_weight_pieces()
 	std::printf("Q2_K 512 x 512, page-exact: %ld pieces behind the tensor before the fix, %ld now\n", before, after);
 }
 
+// ---- streaming GEMM for few activation rows -----------------------------------------------------
+// A workgroup owns a run of consecutive rows and walks it in tiles of 16; wavefront w of eight fetches
+// the bytes of chunks [w cpw, (w + 1) cpw) of every row of a tile (its slice) with the matrix-core
+// GEMM's piece arithmetic, the slice in the place of a chunk.
+static void test_gemm_stream_pieces()
+{
+	long cases = 0;
+	for (const Format& f : kFormats)
+	{
+		for (int cpw : { 1, 2, 4 })
+		{
+			const int slice_bytes = cpw * f.chunk_bytes;
+			const size_t row_bytes = static_cast<size_t>(8) * slice_bytes;
+			const int pieces = fm::gemm_weight_pieces(slice_bytes, f.aligned16);
+			const int loads = (16 * pieces + 63) / 64;
+			for (int n : { 1, 15, 16, 17, 56, 57, 100, 300 })
+			{
+				for (int cus : { 256, 8, 1 })
+				{
+					const size_t bytes = static_cast<size_t>(n) * row_bytes;
+					std::vector<uintptr_t> bases;
+					for (int mis = 0; mis < 16; mis += f.base_align)
+					{
+						bases.push_back(64 * kPage + mis);
+					}
+					const uintptr_t ends_on_page = 4096 * kPage - bytes;
+					if (ends_on_page % f.base_align == 0)
+					{
+						bases.push_back(ends_on_page);
+					}
+					int rows = (n + cus - 1) / cus;
+					rows = (rows + 3) / 4 * 4;
+					const int blocks = (n + rows - 1) / rows;
+					for (uintptr_t base : bases)
+					{
+						const uintptr_t end = base + bytes;
+						std::vector<int> stored(n, 0);
+						for (int block = 0; block < blocks; ++block)
+						{
+							const int row0 = block * rows;
+							const int block_rows = rows < n - row0 ? rows : n - row0;
+							CHECK(block_rows > 0, "%s n %d: empty workgroup %d", f.name, n, block);
+							const int last_row = row0 + block_rows - 1;
+							for (int t = 0; t < (block_rows + 15) / 16; ++t)
+							{
+								for (int wave = 0; wave < 8; ++wave)
+								{
+									std::vector<uintptr_t> slot(static_cast<size_t>(loads) * 64, 0); // by 16-byte piece of the slot
+									for (int i = 0; i < loads; ++i)
+									{
+										for (int lane = 0; lane < 64; ++lane)
+										{
+											const fm::GemmWeightRequest rq = fm::gemm_weight_request(i, lane, 1, pieces);
+											if (!(64 * (i + 1) <= 16 * pieces || rq.issued))
+											{
+												continue;
+											}
+											const int row = fm::gemm_weight_row(row0 + 16 * t, rq.row, last_row + 1);
+											CHECK(row >= row0 && row <= last_row, "%s: row %d outside the run", f.name, row);
+											const uintptr_t row_start = base + static_cast<size_t>(row) * row_bytes;
+											const uintptr_t from = fm::gemm_weight_piece(row_start, wave, slice_bytes, f.aligned16, rq.offset);
+											CHECK(from % 16 == 0, "%s: piece not aligned", f.name);
+											CHECK(from < end && from + 16 > base, "%s cpw %d n %d base %#zx: piece outside the tensor", f.name, cpw,
+											      n, static_cast<size_t>(base));
+											slot[64 * i + lane] = from;
+										}
+									}
+									for (int r = 0; r < 16; ++r)
+									{
+										const int row = fm::gemm_weight_row(row0 + 16 * t, r, last_row + 1);
+										const uintptr_t row_start = base + static_cast<size_t>(row) * row_bytes;
+										const uintptr_t slice = row_start + static_cast<size_t>(wave) * slice_bytes;
+										const int mis = fm::gemm_weight_misalignment(row_start, wave, slice_bytes, f.aligned16);
+										for (int b = 0; b < slice_bytes; ++b)
+										{
+											const int at = r * 16 * pieces + mis + b;
+											const uintptr_t from = slot[at >> 4];
+											CHECK(from != 0 && from + (at & 15) == slice + b, "%s cpw %d n %d row %d byte %d", f.name,
+											      cpw, n, r, b);
+										}
+										if (wave == 0 && row0 + 16 * t + r <= last_row)
+										{
+											++stored[row0 + 16 * t + r];
+										}
+									}
+								}
+							}
+						}
+						for (int r = 0; r < n; ++r)
+						{
+							CHECK(stored[r] == 1, "%s n %d: row %d stored %d times", f.name, n, r, stored[r]);
+						}
+						++cases;
+					}
+				}
+			}
+		}
+	}
+	std::printf("streaming gemm: %ld launches walked\n", cases);
+}
+
 // ---- streaming GEMV ------------------------------------------------------------------------------
 static void test_stream_rows_and_pieces()
 {
@@ -341,6 +442,7 @@ static void test_attention_tiles()
 int main()
 {
 	test_gemm_weight_pieces();
+	test_gemm_stream_pieces();
 	test_stream_rows_and_pieces();
 	test_attention_tiles();
 	if (g_failures)

@@ -57,6 +57,25 @@ def test_gemm_residual_and_precise_flag(hip, oracle, fmt):
     assert run_case(hip, oracle, fmt, 48, 200, 512, seed=9, flags=MATMUL_PRECISE) <= 1e-5
 
 
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("m,n,k", [(16, 999, 2048),    # one chunk per wavefront, ragged rows
+                                   (23, 4100, 4096),   # two activation tiles, two chunks per wavefront
+                                   (32, 777, 2048),
+                                   (16, 260, 8192),    # four chunks per wavefront (where the slots fit LDS)
+                                   (17, 20000, 2048)])  # runs of 80 rows: the partial products meet in several rounds
+def test_streaming_form_for_few_activation_rows(hip, oracle, fmt, m, n, k):
+    """Up to 32 activation rows against a single matrix whose K is a multiple of 2048 take the streaming
+    form (one workgroup per CU, K cut over its eight wavefronts, partial products added in LDS);
+    where its slots do not fit LDS the tiled kernel takes the shape: same bar either way."""
+    rows = None
+    if n > 5000:
+        rows = np.sort(np.random.default_rng(n).choice(n, 640, replace=False))
+        rows[0], rows[-1] = 0, n - 1
+    err = run_case(hip, oracle, fmt, m, n, k, seed=m + n + k, rows=rows)
+    assert 1e-6 < err <= TOL, err
+    assert run_case(hip, oracle, fmt, m, n, k, seed=m + n + k + 1, residual=True, rows=rows) <= TOL
+
+
 @pytest.mark.parametrize("m", [16, 64, 512])
 def test_config3_q4_k_14336x4096(hip, oracle, m):
     """BASELINE config 3: K=4096, N=14336 Q4_K at full size (a 768-row sample of N is checked)."""
@@ -175,7 +194,8 @@ def test_prefill_through_the_matrix_cores(hip, oracle, fmt):
         assert rel_l2(dev.eval(toks[lo:hi], precise=False), ref.eval(toks[lo:hi])) < 5e-3
 
 
-@pytest.mark.parametrize("fmt,n,k", [(Q2_K, 512, 512), (Q3_K, 1024, 512), (Q6_K, 1024, 512), (Q2_K, 1024, 256)])
+@pytest.mark.parametrize("fmt,n,k", [(Q2_K, 512, 512), (Q3_K, 1024, 512), (Q6_K, 1024, 512), (Q2_K, 1024, 256),
+                                     (Q2_K, 128, 2048), (Q3_K, 256, 2048), (Q6_K, 256, 4096)])  # the streaming form's
 def test_weights_that_end_on_a_page_boundary(hip, oracle, fmt, n, k):
     """Blocks of 84, 110 and 210 bytes are fetched as 16-byte pieces from the boundary below them;
     no piece may lie wholly behind the tensor, where the next page need not be mapped (these
