@@ -129,8 +129,8 @@ int litenn_hip_permute(int dev, void* dst, int dtype, const size_t* src_shape, s
  * AddLinear produces after the lowering's dequantise + transpose
  * (tools/gguf/LLaMABuilder.cpp:144-150,225-230; src/LiteNN/Layer/Linear.h:67-95).
  * wq is the raw GGUF payload: n rows of k/block blocks.  x_dtype is F32; F16 and BF16
- * activations are accepted too and widened exactly into a Float32 copy first (the copy is
- * allocated and freed by the call, which therefore always synchronises).
+ * activations are accepted too and widened exactly into a Float32 copy first (the copy is taken
+ * from and returned to the device's memory pool in stream order, see below).
  * residual (f32 [m, n]) may be NULL; when given, y = residual + x.W
  * (the Add at tools/gguf/LLaMABuilder.cpp:652-653,661-663).  residual may alias y.
  * m == 1..15 runs the streaming GEMV.  m >= 16 (with k a multiple of 256) runs on the matrix
@@ -138,8 +138,12 @@ int litenn_hip_permute(int dev, void* dst, int dtype, const size_t* src_shape, s
  * by a power of two into the fp16 range), products accumulate in f32; relative L2 error about
  * 4e-4.  LITENN_HIP_MATMUL_PRECISE in `flags` keeps f32 operands (GEMV path) for any m.
  * The matrix-core path needs a device workspace of litenn_hip_mul_mat_q_workspace_bytes(m, k):
- * litenn_hip_mul_mat_q allocates and frees it itself (and therefore always synchronises for
- * m >= 16); litenn_hip_mul_mat_q_ws takes the caller's (16-byte aligned; NULL = as above).
+ * litenn_hip_mul_mat_q takes it from the device's memory pool in stream order (hipMallocAsync /
+ * hipFreeAsync on the call's stream: no wait for the stream, opts->synchronize is honoured; only
+ * where the device has no memory pools does the call fall back to hipMalloc and drain the stream);
+ * litenn_hip_mul_mat_q_ws takes the caller's (16-byte aligned; NULL = as above).
+ * m <= 32 against a single matrix whose k is a multiple of 2048 takes a streaming form of the
+ * matrix-core kernel (one launch, every weight byte read once).
  * A workspace larger than that (rounded up to 16) by 4*m*n bytes, or by three times as much,
  * also lets a launch that would leave the card short of work walk K in two, or four, parts at
  * once (k >= 8192 with 128 x 128 tiles on half the card; m <= 32 or so, where the launch is a

@@ -44,6 +44,7 @@ namespace litenn_hip
 	                                     size_t m, size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim,
 	                                     float* out, size_t splits, hipStream_t s);
 	void launch_silu_mul(const float* gate, const float* up, float* y, size_t n, hipStream_t s);
+	void launch_zero_ints(int* p, size_t n, hipStream_t s);
 	void launch_argmax(const float* x, size_t rows, size_t n, int32_t* out, hipStream_t s);
 
 	// ---- error state -----------------------------------------------------------------------
@@ -109,6 +110,105 @@ namespace litenn_hip
 	{
 		LITENN_HIP_TRY(action, hipGetLastError());
 		if (!opts || opts->synchronize)
+		{
+			LITENN_HIP_TRY(action, hipStreamSynchronize(stream_of(opts)));
+		}
+		return 0;
+	}
+
+	// Device memory a call needs beyond its operands, in stream order: hipMallocAsync takes it from the
+	// device's pool and hipFreeAsync returns it once the work queued before has run, so such a call
+	// neither waits for the stream nor stalls the device the way hipMalloc / hipFree do.  The pool keeps
+	// what was returned (release threshold: everything) for the next call.  Where the stream-ordered
+	// allocator is not available the memory comes from hipMalloc and the call drains the stream before
+	// freeing it; `blocking()` tells the caller which it was.
+	class StreamScratch
+	{
+	public:
+		explicit StreamScratch(hipStream_t s) : stream_(s) {}
+		StreamScratch(const StreamScratch&) = delete;
+		StreamScratch& operator=(const StreamScratch&) = delete;
+		~StreamScratch()
+		{
+			if (!ptr_)
+			{
+				return;
+			}
+			if (async_)
+			{
+				(void)hipFreeAsync(ptr_, stream_);
+			}
+			else
+			{
+				(void)hipStreamSynchronize(stream_);
+				(void)hipFree(ptr_);
+			}
+		}
+		hipError_t allocate(size_t bytes)
+		{
+			static const bool use_pool = env_int("LITENN_HIP_STREAM_ORDERED_SCRATCH", 1) != 0;
+			if (use_pool && pool_ready())
+			{
+				if (hipMallocAsync(&ptr_, bytes ? bytes : 1, stream_) == hipSuccess)
+				{
+					async_ = true;
+					return hipSuccess;
+				}
+				(void)hipGetLastError();
+				ptr_ = nullptr;
+			}
+			async_ = false;
+			return hipMalloc(&ptr_, bytes ? bytes : 1);
+		}
+		void* get() const { return ptr_; }
+		bool blocking() const { return ptr_ && !async_; }
+
+	private:
+		// once per device: the default pool keeps freed memory instead of handing it back at every
+		// synchronisation
+		static bool pool_ready()
+		{
+			static std::mutex mutex;
+			static std::set<int> ready, refused;
+			int dev = 0;
+			if (hipGetDevice(&dev) != hipSuccess)
+			{
+				return false;
+			}
+			std::lock_guard<std::mutex> lock(mutex);
+			if (ready.count(dev))
+			{
+				return true;
+			}
+			if (refused.count(dev))
+			{
+				return false;
+			}
+			int supported = 0;
+			hipMemPool_t pool = nullptr;
+			unsigned long long keep = ~0ull;
+			if (hipDeviceGetAttribute(&supported, hipDeviceAttributeMemoryPoolsSupported, dev) == hipSuccess && supported &&
+			    hipDeviceGetDefaultMemPool(&pool, dev) == hipSuccess &&
+			    hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep) == hipSuccess)
+			{
+				ready.insert(dev);
+				return true;
+			}
+			(void)hipGetLastError();
+			refused.insert(dev);
+			return false;
+		}
+		void* ptr_ = nullptr;
+		hipStream_t stream_ = nullptr;
+		bool async_ = false;
+	};
+
+	// like finish(), for a call that holds a StreamScratch: a scratch that came from hipMalloc is freed
+	// by draining the stream, so the launch error is collected first and the drain reported
+	int finish_with(const StreamScratch& scratch, const char* action, const litenn_hip_exec* opts)
+	{
+		LITENN_HIP_TRY(action, hipGetLastError());
+		if (scratch.blocking() || !opts || opts->synchronize)
 		{
 			LITENN_HIP_TRY(action, hipStreamSynchronize(stream_of(opts)));
 		}
@@ -586,31 +686,18 @@ extern "C" int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t 
 	}
 	GUARD(action, dev);
 	hipStream_t s = stream_of(opts);
-	// 16-bit activations are widened (exactly) into a Float32 copy that this call owns; the copy
-	// is released after the stream has drained, so such a call always blocks
-	struct Widened
-	{
-		void* p = nullptr;
-		hipStream_t s = nullptr;
-		~Widened()
-		{
-			if (p)
-			{
-				(void)hipStreamSynchronize(s);
-				(void)hipFree(p);
-			}
-		}
-	} widened;
+	// 16-bit activations are widened (exactly) into a Float32 copy that this call owns (stream-ordered
+	// scratch: returned to the pool once the work queued here has run)
+	StreamScratch widened(s);
 	const float* xf = static_cast<const float*>(x);
 	if (x_dtype != LITENN_F32)
 	{
-		widened.s = s;
-		LITENN_HIP_TRY(action, hipMalloc(&widened.p, sizeof(float) * m * k));
-		if (!launch_convert(x_dtype, x, m * k, LITENN_F32, widened.p, s))
+		LITENN_HIP_TRY(action, widened.allocate(sizeof(float) * m * k));
+		if (!launch_convert(x_dtype, x, m * k, LITENN_F32, widened.get(), s))
 		{
 			return fail(action, "activation dtype is not supported on the device");
 		}
-		xf = static_cast<const float*>(widened.p);
+		xf = static_cast<const float*>(widened.get());
 	}
 	float* yf = static_cast<float*>(y);
 	const float* rf = static_cast<const float*>(residual);
@@ -635,30 +722,32 @@ extern "C" int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t 
 			{
 				launch_gemv(fmt, wq, n, k, xf, m, yf, rf, s);
 			}
-			return finish(action, opts);
+			return finish_with(widened, action, opts);
 		}
-		// none given: this call owns one, and frees it after the stream has drained, whatever
-		// opts->synchronize says
-		void* scratch = nullptr;
+		// none given: this call takes one in stream order and returns it the same way
+		StreamScratch scratch(s);
 		const bool splits = (k >= 8192 && m >= 128) || m <= 64;
-		LITENN_HIP_TRY(action, hipMalloc(&scratch, splits ? with_partial : need));
-		float* partial = splits ? reinterpret_cast<float*>(static_cast<char*>(scratch) + need16) : nullptr;
-		if (!launch_gemm(fmt, wq, n, k, xf, m, yf, rf, scratch, partial, splits ? (with_partial - need16) / sizeof(float) : 0,
-		                 s))
+		LITENN_HIP_TRY(action, scratch.allocate(splits ? with_partial : need));
+		float* partial = splits ? reinterpret_cast<float*>(static_cast<char*>(scratch.get()) + need16) : nullptr;
+		if (!launch_gemm(fmt, wq, n, k, xf, m, yf, rf, scratch.get(), partial,
+		                 splits ? (with_partial - need16) / sizeof(float) : 0, s))
 		{
 			launch_gemv(fmt, wq, n, k, xf, m, yf, rf, s);
 		}
-		const hipError_t launched = hipGetLastError();
-		const hipError_t drained = hipStreamSynchronize(s);
-		(void)hipFree(scratch);
-		if (launched != hipSuccess || drained != hipSuccess)
+		if (scratch.blocking() || widened.blocking())
 		{
-			return fail_hip(action, launched != hipSuccess ? launched : drained);
+			const hipError_t launched = hipGetLastError();
+			const hipError_t drained = hipStreamSynchronize(s);
+			if (launched != hipSuccess || drained != hipSuccess)
+			{
+				return fail_hip(action, launched != hipSuccess ? launched : drained);
+			}
+			return 0;
 		}
-		return 0;
+		return finish(action, opts);
 	}
 	launch_gemv(fmt, wq, n, k, xf, m, yf, rf, s);
-	return finish(action, opts);
+	return finish_with(widened, action, opts);
 }
 
 extern "C" int litenn_hip_linear_group(int dev, int fmt, size_t count, const void* const* wq, const size_t* n, size_t k,
@@ -702,24 +791,15 @@ extern "C" int litenn_hip_linear_group(int dev, int fmt, size_t count, const voi
 	}
 	GUARD(action, dev);
 	hipStream_t s = stream_of(opts);
-	// scratch for the composed form; private to the call, so it always completes before returning
-	float* scratch = nullptr;
+	// scratch for the composed form, taken and returned in stream order
+	StreamScratch scratch_mem(s);
 	const size_t scratch_floats = k + 2 * n[0];
-	LITENN_HIP_TRY(action, hipMalloc(reinterpret_cast<void**>(&scratch), sizeof(float) * scratch_floats));
+	LITENN_HIP_TRY(action, scratch_mem.allocate(sizeof(float) * scratch_floats));
+	float* scratch = static_cast<float*>(scratch_mem.get());
 	launch_linear_group(fmt, static_cast<int>(count), wq, ys, n, k, static_cast<const float*>(x),
 	                    static_cast<const float*>(residual), static_cast<const float*>(norm_w), eps, silu, scratch,
 	                    scratch + k, scratch + k + n[0], s);
-	hipError_t e = hipGetLastError();
-	if (e == hipSuccess)
-	{
-		e = hipStreamSynchronize(s);
-	}
-	(void)hipFree(scratch);
-	if (e != hipSuccess)
-	{
-		return fail_hip(action, e);
-	}
-	return 0;
+	return finish_with(scratch_mem, action, opts);
 }
 
 extern "C" int litenn_hip_dequantize(int dev, int fmt, const void* wq, size_t rows, size_t k, void* dst,
@@ -952,37 +1032,23 @@ static int attn_rows_impl(int dev, const void* q, const void* kcache, const void
 	{
 		return finish(action, opts);
 	}
-	// a single row against a long cache is cut into chunks that meet in scratch memory, which
-	// this call owns: it is freed after the stream has drained, whatever opts->synchronize says
+	// a single row against a long cache is cut into chunks that meet in scratch memory, which this
+	// call takes and returns in stream order
 	const size_t splits = attn_splits(m, past + m, n_head);
+	StreamScratch scratch(stream_of(opts));
 	float* partial = nullptr;
 	int* counters = nullptr;
 	if (splits > 1)
 	{
 		const size_t bytes = sizeof(float) * attn_partial_floats(m, n_head, head_dim, splits);
-		LITENN_HIP_TRY(action, hipMalloc(reinterpret_cast<void**>(&partial), bytes + sizeof(int) * m * n_head));
+		LITENN_HIP_TRY(action, scratch.allocate(bytes + sizeof(int) * m * n_head));
+		partial = static_cast<float*>(scratch.get());
 		counters = reinterpret_cast<int*>(reinterpret_cast<char*>(partial) + bytes);
-		const hipError_t e = hipMemsetAsync(counters, 0, sizeof(int) * m * n_head, stream_of(opts));
-		if (e != hipSuccess)
-		{
-			(void)hipFree(partial);
-			return fail_hip(action, e);
-		}
+		launch_zero_ints(counters, m * n_head, stream_of(opts));
 	}
 	launch_attn_decode(static_cast<const float*>(q), kcache, vcache, cache_dtype, m, nullptr, past, n_head, n_kv_head,
 	                   head_dim, static_cast<float*>(out), splits, partial, counters, stream_of(opts));
-	if (partial)
-	{
-		const hipError_t launched = hipGetLastError();
-		const hipError_t drained = hipStreamSynchronize(stream_of(opts));
-		(void)hipFree(partial);
-		if (launched != hipSuccess || drained != hipSuccess)
-		{
-			return fail_hip(action, launched != hipSuccess ? launched : drained);
-		}
-		return 0;
-	}
-	return finish(action, opts);
+	return finish_with(scratch, action, opts);
 }
 
 extern "C" int litenn_hip_attn_decode(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype,

@@ -850,6 +850,15 @@ namespace litenn_hip
 	} // namespace
 
 	// ---- launchers used by the C ABI and by the decoder runtime ---------------------------
+	// clears n ints with a small kernel (a fill that a captured graph replays correctly)
+	void launch_zero_ints(int* p, size_t n, hipStream_t s)
+	{
+		if (n)
+		{
+			zero_ints_kernel<<<dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, s>>>(p, static_cast<int>(n));
+		}
+	}
+
 	void launch_rmsnorm(const float* x, const float* w, double eps, size_t m, size_t d, float* y, hipStream_t s)
 	{
 		rmsnorm_kernel<<<dim3(m), dim3(d >= 4096 ? 1024 : 256), 0, s>>>(x, w, eps, static_cast<int>(d), y);

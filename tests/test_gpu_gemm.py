@@ -208,3 +208,28 @@ def test_weights_that_end_on_a_page_boundary(hip, oracle, fmt, n, k):
         x = synth.activations(m, k, 9, m)
         y = hip.mul_mat_q(fmt, w, n, k, hip.Tensor.from_numpy(x)).numpy()
         assert rel_l2(y, oracle.mul_mat_q(fmt, wq, n, k, x)) <= 1e-3
+
+
+def test_calls_without_a_workspace_queue_on_their_stream(hip, oracle):
+    """Without a caller's workspace the matrix-core path takes its scratch from the device's memory
+    pool in stream order: a run of calls with synchronize = 0 on one stream (different shapes, 16-bit
+    activations among them, so that scratch of several sizes is taken and returned while earlier
+    work is still queued) gives the same results as blocking calls."""
+    from litenn_amd import hiprt
+    from litenn_amd.formats import DT_F16
+    stream = hiprt.Stream()
+    cases = []
+    for i, (fmt, m, n, k) in enumerate([(Q4_K, 16, 520, 2048), (Q6_K, 64, 300, 512), (Q4_0, 40, 1000, 1024),
+                                        (Q8_0, 16, 64, 4096), (Q4_K, 130, 700, 256)] * 3):
+        wq = synth.quant_weights(fmt, n, k, 70 + i, 1)
+        x = synth.activations(m, k, 70 + i, 2)
+        half = i % 4 == 1
+        xt = hip.Tensor.from_numpy(x.astype(np.float16) if half else x)
+        assert not half or xt.dtype == DT_F16
+        w = hip.Tensor.from_numpy(wq)
+        y = hip.mul_mat_q(fmt, w, n, k, xt, stream=stream.handle, synchronize=False)
+        cases.append((fmt, wq, n, k, x.astype(np.float16).astype(np.float32) if half else x, y, w, xt))
+    stream.synchronize()
+    for fmt, wq, n, k, x, y, _, _ in cases:
+        assert rel_l2(y.numpy(), oracle.mul_mat_q(fmt, wq, n, k, x)) <= TOL
+    stream.destroy()
