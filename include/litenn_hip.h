@@ -91,7 +91,9 @@ int litenn_hip_alloc(int dev, int dtype, size_t n, void** out);
 int litenn_hip_free(int dev, void* ptr, int dtype, size_t n);
 int litenn_hip_zero(int dev, void* ptr, int dtype, size_t n);
 /* CopyToCPU / CopyFromCPU / ConvertTo, src/LiteNN/Device.h:35-39, CUDA.cpp:1785-1892.
- * Synchronous on return unless opts says otherwise; dtype may change. */
+ * Synchronous on return unless opts says otherwise; dtype may change: every pair of the eleven
+ * element types converts as static_cast does on the CPU, Float16 / BFloat16 / Float8E4M3 /
+ * Float8E5M2 through LiteNN's own constructors (src/LiteNN/DType.h:58-229). */
 int litenn_hip_copy_to_host(int dev, int src_dtype, const void* src, size_t n, int dst_dtype, void* dst,
                             const litenn_hip_exec* opts);
 int litenn_hip_copy_from_host(int dev, int dst_dtype, void* dst, int src_dtype, const void* src, size_t n,

@@ -311,6 +311,78 @@ namespace litenn_hip
 	{
 		struct F16 { uint16_t bits; };
 		struct BF16 { uint16_t bits; };
+		// Float8E4M3 (4 exponent bits, bias 7) and Float8E5M2 (5, bias 15), both with the top
+		// exponent reserved for infinity and NaN as LiteNN defines them (DType.h:290-344)
+		template <int EBITS, int MBITS, int BIAS>
+		struct F8 { uint8_t bits; };
+		using F8E4M3 = F8<4, 3, 7>;
+		using F8E5M2 = F8<5, 2, 15>;
+
+		// Float8BitsToFloat32 (DType.h:203-229): every value is exact in Float32
+		template <int EBITS, int MBITS, int BIAS>
+		__device__ __forceinline__ float f8_bits_to_f32(uint8_t bits)
+		{
+			const uint32_t exp_mask = (1u << EBITS) - 1u;
+			const uint32_t e = (bits >> MBITS) & exp_mask, mant = bits & ((1u << MBITS) - 1u);
+			const float sign = (bits & 0x80u) ? -1.0f : 1.0f;
+			if (e == 0)
+			{
+				return sign * ldexpf(static_cast<float>(mant), 1 - BIAS - MBITS); // zero keeps its sign
+			}
+			if (e == exp_mask)
+			{
+				return mant == 0 ? sign * INFINITY : __uint_as_float(0x7fc00000u);
+			}
+			return sign * ldexpf(static_cast<float>((1u << MBITS) | mant), static_cast<int>(e) - BIAS - MBITS);
+		}
+
+		// Float32ToFloat8Bits (DType.h:148-201), step for step: the magnitude is brought into [1, 2)
+		// (exact), the mantissa is (uint32)(x * 2^MBITS + 0.5f) with the Float32 addition's own
+		// rounding, a mantissa that rounds up to 2^MBITS carries into the exponent, the top exponent is
+		// infinity (NaN goes there too, with its sign bit), stored exponents <= 0 are subnormal with the
+		// mantissa clamped to its field.
+		template <int EBITS, int MBITS, int BIAS>
+		__device__ __forceinline__ uint8_t f32_to_f8_bits(float value)
+		{
+			const uint32_t raw = __float_as_uint(value);
+			const uint32_t sign = (raw >> 24) & 0x80u;
+			const uint32_t mag = raw & 0x7fffffffu;
+			const uint32_t max_exp = (1u << EBITS) - 1u;
+			if (mag == 0)
+			{
+				return static_cast<uint8_t>(sign);
+			}
+			if (mag >= 0x7f800000u)
+			{
+				return static_cast<uint8_t>(sign | (max_exp << MBITS));
+			}
+			if (mag < 0x00800000u)
+			{
+				return static_cast<uint8_t>(sign); // a Float32 subnormal is far below half the smallest step
+			}
+			const int exponent = static_cast<int>(mag >> 23) - 127;
+			const float m = __uint_as_float((mag & 0x007fffffu) | 0x3f800000u); // in [1, 2)
+			const int stored = exponent + BIAS;
+			const float scale = static_cast<float>(1u << MBITS);
+			if (stored >= static_cast<int>(max_exp))
+			{
+				return static_cast<uint8_t>(sign | (max_exp << MBITS));
+			}
+			if (stored <= 0)
+			{
+				const float sub = ldexpf(m, stored - 1); // exact here: the product below is compared with 1/2
+				const uint32_t q = static_cast<uint32_t>(__fadd_rn(__fmul_rn(sub, scale), 0.5f));
+				return static_cast<uint8_t>(sign | min(q, (1u << MBITS) - 1u));
+			}
+			uint32_t q = static_cast<uint32_t>(__fadd_rn(__fmul_rn(__fsub_rn(m, 1.0f), scale), 0.5f));
+			uint32_t e = static_cast<uint32_t>(stored);
+			if (q == (1u << MBITS))
+			{
+				q = 0;
+				e = min(e + 1u, max_exp);
+			}
+			return static_cast<uint8_t>(sign | (e << MBITS) | q);
+		}
 
 		template <typename T>
 		__device__ __forceinline__ double load_as_double(const T* p, size_t i) { return static_cast<double>(p[i]); }
@@ -323,6 +395,17 @@ namespace litenn_hip
 		__device__ __forceinline__ double load_as_double<BF16>(const BF16* p, size_t i)
 		{
 			return static_cast<double>(__uint_as_float(static_cast<uint32_t>(p[i].bits) << 16));
+		}
+
+		template <>
+		__device__ __forceinline__ double load_as_double<F8E4M3>(const F8E4M3* p, size_t i)
+		{
+			return static_cast<double>(f8_bits_to_f32<4, 3, 7>(p[i].bits));
+		}
+		template <>
+		__device__ __forceinline__ double load_as_double<F8E5M2>(const F8E5M2* p, size_t i)
+		{
+			return static_cast<double>(f8_bits_to_f32<5, 2, 15>(p[i].bits));
 		}
 
 		template <typename S>
@@ -375,6 +458,12 @@ namespace litenn_hip
 			dst[i].bits = static_cast<uint16_t>((bits + 0x7fffu + lsb) >> 16);
 		}
 
+		template <typename S, int EBITS, int MBITS, int BIAS>
+		__device__ __forceinline__ void convert_one(const S* src, F8<EBITS, MBITS, BIAS>* dst, size_t i)
+		{
+			dst[i].bits = f32_to_f8_bits<EBITS, MBITS, BIAS>(load_as_float<S>(src, i));
+		}
+
 		template <typename S, typename D>
 		__global__ void convert_kernel(const S* __restrict__ src, D* __restrict__ dst, size_t n)
 		{
@@ -399,6 +488,8 @@ namespace litenn_hip
 			case LITENN_BOOL: convert_kernel<S, bool><<<grid, block, 0, s>>>(sp, static_cast<bool*>(dst), n); return true;
 			case LITENN_F16: convert_kernel<S, F16><<<grid, block, 0, s>>>(sp, static_cast<F16*>(dst), n); return true;
 			case LITENN_BF16: convert_kernel<S, BF16><<<grid, block, 0, s>>>(sp, static_cast<BF16*>(dst), n); return true;
+			case LITENN_F8E4M3: convert_kernel<S, F8E4M3><<<grid, block, 0, s>>>(sp, static_cast<F8E4M3*>(dst), n); return true;
+			case LITENN_F8E5M2: convert_kernel<S, F8E5M2><<<grid, block, 0, s>>>(sp, static_cast<F8E5M2*>(dst), n); return true;
 			case LITENN_I8: convert_kernel<S, int8_t><<<grid, block, 0, s>>>(sp, static_cast<int8_t*>(dst), n); return true;
 			case LITENN_U8: convert_kernel<S, uint8_t><<<grid, block, 0, s>>>(sp, static_cast<uint8_t*>(dst), n); return true;
 			default: return false;
@@ -422,6 +513,8 @@ namespace litenn_hip
 		case LITENN_BOOL: return convert_from<bool>(src, dst_dtype, dst, n, s);
 		case LITENN_F16: return convert_from<F16>(src, dst_dtype, dst, n, s);
 		case LITENN_BF16: return convert_from<BF16>(src, dst_dtype, dst, n, s);
+		case LITENN_F8E4M3: return convert_from<F8E4M3>(src, dst_dtype, dst, n, s);
+		case LITENN_F8E5M2: return convert_from<F8E5M2>(src, dst_dtype, dst, n, s);
 		case LITENN_I8: return convert_from<int8_t>(src, dst_dtype, dst, n, s);
 		case LITENN_U8: return convert_from<uint8_t>(src, dst_dtype, dst, n, s);
 		default: return false;

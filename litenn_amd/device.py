@@ -15,7 +15,8 @@ import numpy as np
 
 from . import _lib
 from ._lib import Exec, LiteNNHipError, check
-from .formats import (DT_BF16, DT_BOOL, DT_F16, DT_F32, DT_F64, DT_I8, DT_I32, DT_I64, DT_U8, DTYPE_SIZE, F32,
+from .formats import (DT_BF16, DT_BOOL, DT_F8E4M3, DT_F8E5M2, DT_F16, DT_F32, DT_F64, DT_I8, DT_I32, DT_I64, DT_U8,
+                      DTYPE_SIZE, F32,
                       row_bytes)
 
 _NP_TO_DT = {np.dtype(np.float32): DT_F32, np.dtype(np.float64): DT_F64, np.dtype(np.int32): DT_I32,
@@ -23,6 +24,8 @@ _NP_TO_DT = {np.dtype(np.float32): DT_F32, np.dtype(np.float64): DT_F64, np.dtyp
              np.dtype(np.int8): DT_I8, np.dtype(np.uint8): DT_U8}
 _DT_TO_NP = {v: k for k, v in _NP_TO_DT.items()}
 _DT_TO_NP[DT_BF16] = np.dtype(np.uint16)  # raw bits
+_DT_TO_NP[DT_F8E4M3] = np.dtype(np.uint8)  # raw bits
+_DT_TO_NP[DT_F8E5M2] = np.dtype(np.uint8)  # raw bits
 
 
 @dataclass(frozen=True)

@@ -159,3 +159,87 @@ def convert(x: np.ndarray, dtype) -> np.ndarray:
     float with the reference's own rounding is checked elsewhere; this covers the plain types)."""
     with np.errstate(all="ignore"):
         return x.astype(dtype)
+
+
+# ---- Float8E4M3 / Float8E5M2 (src/LiteNN/DType.h:148-229, 290-344) ---------------------------------
+F8_LAYOUTS = {"e4m3": (4, 3, 7), "e5m2": (5, 2, 15)}  # exponent bits, mantissa bits, bias
+
+
+def _ldexp_f32(value: np.float32, exponent: int) -> np.float32:
+    """Detail::Ldexp (DType.h:34-51): repeated multiplication by 2 or 0.5 in Float32."""
+    if value == 0:
+        return np.float32(0.0)
+    value = np.float32(value)
+    while exponent > 0:
+        value = np.float32(value * np.float32(2.0))
+        exponent -= 1
+    while exponent < 0:
+        value = np.float32(value * np.float32(0.5))
+        exponent += 1
+    return value
+
+
+def _round_to_uint(value: np.float32) -> int:
+    """Detail::RoundToUInt (DType.h:53-56): static_cast<uint32>(value + 0.5F), the sum in Float32."""
+    return int(np.float32(np.float32(value) + np.float32(0.5)))
+
+
+def f8_bits_to_f32(bits, kind: str) -> np.ndarray:
+    """Float8BitsToFloat32 (DType.h:203-229), element by element."""
+    ebits, mbits, bias = F8_LAYOUTS[kind]
+    flat = np.asarray(bits, np.uint8).reshape(-1)
+    out = np.empty(flat.shape, np.float32)
+    exp_mask = (1 << ebits) - 1
+    scale = np.float32(1 << mbits)
+    for i, b in enumerate(flat.tolist()):
+        sign = np.float32(-1.0 if b & 0x80 else 1.0)
+        e = (b >> mbits) & exp_mask
+        mant = b & ((1 << mbits) - 1)
+        if e == 0:
+            out[i] = sign * np.float32(0.0) if mant == 0 else sign * _ldexp_f32(np.float32(mant) / scale, 1 - bias)
+        elif e == exp_mask:
+            out[i] = sign * np.float32(np.inf) if mant == 0 else np.float32(np.nan)
+        else:
+            out[i] = sign * _ldexp_f32(np.float32(1.0) + np.float32(mant) / scale, e - bias)
+    return out.reshape(np.shape(bits))
+
+
+def f32_to_f8_bits(values, kind: str) -> np.ndarray:
+    """Float32ToFloat8Bits (DType.h:148-201), element by element, every step in Float32."""
+    ebits, mbits, bias = F8_LAYOUTS[kind]
+    flat = np.asarray(values, np.float32).reshape(-1)
+    out = np.empty(flat.shape, np.uint8)
+    max_exp = (1 << ebits) - 1
+    scale = np.float32(1 << mbits)
+    with np.errstate(all="ignore"):
+        for i, v in enumerate(flat):
+            sign = 0x80 if np.signbit(v) else 0
+            mag = np.float32(-v) if v < 0 else np.float32(v)
+            if mag == 0:
+                out[i] = sign
+                continue
+            if not np.isfinite(mag):
+                out[i] = sign | (max_exp << mbits)
+                continue
+            exponent = 0
+            while mag >= 2:
+                mag = np.float32(mag * np.float32(0.5))
+                exponent += 1
+            while mag < 1:
+                mag = np.float32(mag * np.float32(2.0))
+                exponent -= 1
+            stored = exponent + bias
+            if stored >= max_exp:
+                out[i] = sign | (max_exp << mbits)
+                continue
+            if stored <= 0:
+                sub = _ldexp_f32(mag, exponent + bias - 1)
+                out[i] = sign | min(_round_to_uint(np.float32(sub * scale)), (1 << mbits) - 1)
+                continue
+            mant = _round_to_uint(np.float32(np.float32(mag - np.float32(1.0)) * scale))
+            e = stored
+            if mant == (1 << mbits):
+                mant = 0
+                e = min(e + 1, max_exp)
+            out[i] = sign | (e << mbits) | mant
+    return out.reshape(np.shape(values))

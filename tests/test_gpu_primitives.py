@@ -8,7 +8,8 @@ import pytest
 
 from litenn_amd import LiteNNHipError
 from litenn_amd.device import HIP, DeviceTraits, _NP_TO_DT
-from litenn_amd.formats import DT_BF16, DT_BOOL, DT_F16, DT_F32, DT_F64, DT_I8, DT_I32, DT_I64, DT_U8
+from litenn_amd.formats import (DT_BF16, DT_BOOL, DT_F8E4M3, DT_F8E5M2, DT_F16, DT_F32, DT_F64, DT_I8, DT_I32, DT_I64,
+                                DT_U8)
 from oracle import primitives as P
 
 pytestmark = pytest.mark.gpu
@@ -276,3 +277,56 @@ def test_low_precision_conversions(hip, oracle):
     assert np.array_equal(bf.numpy(), want)
     DeviceTraits.ConvertTo(DEV, DT_BF16, bf.ptr, bf.size, DT_F32, back.ptr)
     assert np.array_equal(back.numpy().view(np.uint32), want.astype(np.uint32) << 16)
+
+
+@pytest.mark.parametrize("kind,dtype", [("e4m3", DT_F8E4M3), ("e5m2", DT_F8E5M2)])
+def test_float8_conversions(hip, kind, dtype):
+    """ConvertTo with Float8E4M3 / Float8E5M2 on either side (src/LiteNN/Device.h:372-391 through the
+    constructors and conversion operators of src/LiteNN/DType.h:148-229, 290-344), bit for bit
+    against the checker's restatement: every code decoded, Float32 inputs that land on values,
+    midpoints, both sides of midpoints, the subnormal range, overflow, infinities and NaN, and the
+    other element types through their conversion to float."""
+    from litenn_amd.formats import DT_BF16, DT_F16, DT_F64, DT_I32
+
+    def as_tensor(raw_bits):
+        t = hip.Tensor(raw_bits.shape, dtype)
+        DeviceTraits.CopyFromCPU(DEV, dtype, t.ptr, dtype, np.ascontiguousarray(raw_bits, np.uint8), t.size)
+        return t
+
+    def convert(src, dst_dtype):
+        dst = hip.Tensor(src.shape, dst_dtype)
+        DeviceTraits.ConvertTo(DEV, src.dtype, src.ptr, src.size, dst_dtype, dst.ptr)
+        return dst.numpy()
+
+    codes = np.arange(256, dtype=np.uint8)
+    table = P.f8_bits_to_f32(codes, kind)
+    got = convert(as_tensor(codes), DT_F32)
+    assert np.array_equal(got.view(np.uint32)[~np.isnan(table)], table.view(np.uint32)[~np.isnan(table)])
+    assert np.all(np.isnan(got[np.isnan(table)]))
+    finite = np.isfinite(table)
+    assert np.array_equal(convert(as_tensor(codes[finite]), DT_F64), table[finite].astype(np.float64))
+    assert np.array_equal(convert(as_tensor(codes[finite]), DT_I32), table[finite].astype(np.int32))
+    assert np.array_equal(convert(as_tensor(codes[finite]), DT_F16).view(np.uint16),
+                          table[finite].astype(np.float16).view(np.uint16))  # every value is exact in a half
+    # Float32 -> Float8
+    rng = np.random.default_rng(23)
+    pos = np.sort(table[np.isfinite(table) & ~np.signbit(table)]).astype(np.float64)
+    mids = (pos[1:] + pos[:-1]) / 2
+    x = np.concatenate([pos, mids, np.nextafter(mids.astype(np.float32), np.float32(0)),
+                        np.nextafter(mids.astype(np.float32), np.float32(np.inf)),
+                        [pos[-1] * 1.03, pos[-1] * 1.07, pos[-1] * 2, 1e30, 1e-30, 1e-40, np.inf, np.nan, 0.0],
+                        rng.standard_normal(3000) * 3, rng.standard_normal(1000) * pos[-1] / 2,
+                        rng.standard_normal(1000) * pos[2]]).astype(np.float32)
+    x = np.concatenate([x, -x])
+    want = P.f32_to_f8_bits(x, kind)
+    assert np.array_equal(convert(hip.Tensor.from_numpy(x), dtype), want)
+    # other sources reach Float8 through their conversion to float
+    xd = np.concatenate([mids, pos, rng.standard_normal(500)]).astype(np.float64)
+    assert np.array_equal(convert(hip.Tensor.from_numpy(xd), dtype), P.f32_to_f8_bits(xd.astype(np.float32), kind))
+    xi = rng.integers(-300, 300, 500).astype(np.int32)
+    assert np.array_equal(convert(hip.Tensor.from_numpy(xi), dtype), P.f32_to_f8_bits(xi.astype(np.float32), kind))
+    xh = (rng.standard_normal(500) * 4).astype(np.float16)
+    assert np.array_equal(convert(hip.Tensor.from_numpy(xh), dtype), P.f32_to_f8_bits(xh.astype(np.float32), kind))
+    # and a host copy with a type change takes the same route
+    t = hip.Tensor.from_numpy(x[:64])
+    assert np.array_equal(t.numpy(dtype), want[:64])

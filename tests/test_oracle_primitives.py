@@ -94,3 +94,50 @@ def test_matmul_is_k_ascending_with_separate_rounding():
     a = np.array([[1e8, 1.0, -1e8]], np.float32)
     b = np.ones((3, 1), np.float32)
     assert P.binary(P.BIN_MATMUL, a, b)[0, 0] == 0.0
+
+
+@pytest.mark.parametrize("kind", ["e4m3", "e5m2"])
+def test_float8_restatement_against_what_the_format_fixes(kind):
+    """The checker's Float8 conversions (DType.h:148-229) against facts that do not come from its own
+    formula: the value of every code written out from the format's definition, codes surviving a
+    round trip, and, for inputs with few mantissa bits, the code chosen being the nearest value in
+    the table of all codes with ties going to the larger magnitude (the reference adds one half
+    and truncates)."""
+    ebits, mbits, bias = P.F8_LAYOUTS[kind]
+    codes = np.arange(256, dtype=np.uint8)
+    table = P.f8_bits_to_f32(codes, kind)
+    top = (1 << ebits) - 1
+    for c in range(256):
+        e, m = (c >> mbits) & top, c & ((1 << mbits) - 1)
+        sign = -1.0 if c & 0x80 else 1.0
+        if e == top:
+            assert (np.isinf(table[c]) and np.sign(table[c]) == sign) if m == 0 else np.isnan(table[c])
+        elif e == 0:
+            assert table[c] == np.float32(sign * m * 2.0 ** (1 - bias - mbits)) and np.signbit(table[c]) == (sign < 0)
+        else:
+            assert table[c] == np.float32(sign * (1 + m / 2.0 ** mbits) * 2.0 ** (e - bias))
+    finite = np.isfinite(table) | np.isinf(table)
+    assert np.array_equal(P.f32_to_f8_bits(table[finite], kind), codes[finite])
+    # landmarks
+    one = P.f32_to_f8_bits(np.float32(1.0), kind)
+    assert int(one) == (bias << mbits)
+    largest = table[(top << mbits) - 1]
+    step = largest - table[(top << mbits) - 2]
+    got = P.f32_to_f8_bits(np.array([largest, largest + step / 2 * 0.999, largest + step / 2, np.nan, -np.inf,
+                                     -0.0, table[1] / 2, table[1] / 2 * 0.99], np.float32), kind)
+    assert got.tolist() == [(top << mbits) - 1, (top << mbits) - 1, top << mbits, top << mbits,
+                            0x80 | (top << mbits), 0x80, 1, 0]
+    # nearest-value property by brute force over the table
+    rng = np.random.default_rng(5)
+    pos = table[:top << mbits].astype(np.float64)  # the non-negative finite values, ascending
+    assert np.all(np.diff(pos) > 0)
+    x = (rng.integers(0, 1 << 14, 4000) * 2.0 ** -14 * rng.choice(2.0 ** np.arange(-bias - mbits, top - bias), 4000))
+    x = x[x <= largest].astype(np.float32)
+    got = P.f32_to_f8_bits(x, kind)
+    for xv, c in zip(x.astype(np.float64), got.tolist()):
+        dist = np.abs(pos - xv)
+        best = np.flatnonzero(dist == dist.min()).max()  # a tie goes to the larger value
+        if xv < pos[1 << mbits] and best == (1 << mbits):
+            best -= 1  # below the smallest normal the mantissa is clamped to its field (DType.h:184-185)
+        assert c == best, (xv, c, best)
+    assert np.array_equal(P.f32_to_f8_bits(-x, kind), got | 0x80)
