@@ -15,6 +15,9 @@ LIB_PATH = os.path.join(LIB_DIR, "liblitenn_hip.so")
 TRACE_LIB_PATH = os.path.join(LIB_DIR, "liblitenn_hip_trace.so")
 
 SOURCES = ["api.hip", "gemv.hip", "gemm.hip", "glue.hip", "attn_tile.hip", "primitives.hip", "llama.hip", "gguf.hip"]
+# gemv.hip: the dispatcher hands the first six kernel arguments over in registers (the streaming
+# kernel's activation pointer, K and first-row addressing), see gemv_stream_kernel
+SOURCE_FLAGS = {"gemv.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=6"]}
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -42,7 +45,7 @@ def build(verbose: bool = True, jobs: int = 6) -> str:
         obj = os.path.join(obj_dir, obj_name)
         if not extra and src in SOURCES:
             objs.append(obj)
-        cmd = [hipcc(), *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc(), *HIPCC_FLAGS, *SOURCE_FLAGS.get(src, []), *extra, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

@@ -1137,11 +1137,27 @@ namespace litenn_hip
 		};
 
 		// The statements live in gemv_stream_body.inc and are compiled into both forms below.
+		// The first six arguments repeat fields of the argument block: the dispatcher hands the leading
+		// kernel arguments over in registers (this file is compiled with kernel-argument preloading for
+		// six of them), so the activation loads and the first row requests do not wait for the block to
+		// be read from memory; on a card whose firmware does not preload, the kernel's compatibility
+		// prologue loads them like any other argument.
 		template <typename U, int XP, bool WHOLE>
-		__global__ __launch_bounds__(512) void gemv_stream_kernel(const GemvArgs a)
+		__global__ __launch_bounds__(512) void gemv_stream_kernel(const float* x_first, int k_first,
+		                                                           const uint8_t* w0_first, uint32_t row_bytes_first,
+		                                                           int rows_per_group_first, int n_total_first,
+		                                                           const GemvArgs block_args)
 		{
+			GemvArgs a = block_args;
+			a.x = x_first;
+			a.k = k_first;
+			a.w[0] = w0_first;
+			a.row_bytes = row_bytes_first;
+			a.rows_per_group = rows_per_group_first;
+			a.n_total = n_total_first;
 			const int block = static_cast<int>(blockIdx.x);
 			constexpr bool kWholeSlices = WHOLE;
+			constexpr bool kEarlyActivations = true;
 #include "gemv_stream_body.inc"
 		}
 
@@ -1149,6 +1165,7 @@ namespace litenn_hip
 		__device__ __forceinline__ void gemv_stream_part(const GemvArgs a, const int block)
 		{
 			constexpr bool kWholeSlices = false;
+			constexpr bool kEarlyActivations = false;
 #include "gemv_stream_body.inc"
 		}
 
@@ -1507,12 +1524,20 @@ namespace litenn_hip
 				if (XP == 2 && launch.part[0].k == 4096)
 				{
 					allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, 2, true>), kStreamLdsLimit);
-					gemv_stream_kernel<U0, 2, true><<<dim3(blocks), dim3(threads), lds, stream>>>(launch.part[0]);
+					{
+						const GemvArgs& g = launch.part[0];
+						gemv_stream_kernel<U0, 2, true><<<dim3(blocks), dim3(threads), lds, stream>>>(g.x, g.k, g.w[0], g.row_bytes,
+						                                                                         g.rows_per_group, g.n_total, g);
+					}
 				}
 				else
 				{
 					allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, XP, false>), kStreamLdsLimit);
-					gemv_stream_kernel<U0, XP, false><<<dim3(blocks), dim3(threads), lds, stream>>>(launch.part[0]);
+					{
+						const GemvArgs& g = launch.part[0];
+						gemv_stream_kernel<U0, XP, false><<<dim3(blocks), dim3(threads), lds, stream>>>(g.x, g.k, g.w[0], g.row_bytes,
+						                                                                         g.rows_per_group, g.n_total, g);
+					}
 				}
 			}
 			else
