@@ -478,8 +478,10 @@ def main() -> int:
     ap.add_argument("--no-configs", action="store_true", help="skip the other single-row GEMV configurations")
     ap.add_argument("--decode-prompt", type=int, default=128, help="prompt length of the decode run")
     ap.add_argument("--decode-new", type=int, default=256, help="tokens generated by the decode run")
-    ap.add_argument("--decode-model", choices=["7b", "8b"], default="7b",
-                    help="7b: 7B-shape Q4_0 (the headline decode); 8b: 8B GQA shape, Q4_K + Q6_K")
+    ap.add_argument("--decode-model", choices=["7b", "8b", "both"], default="both",
+                    help="7b: 7B-shape Q4_0 at --decode-prompt / --decode-new; 8b: 8B GQA shape, Q4_K + Q6_K, at the "
+                         "same lengths; both (default): the 7B shape at those lengths and the 8B shape at prompt 512 "
+                         "+ 512 tokens")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill (batched matmul) measurements")
     ap.add_argument("--gemm-case", default=None, help="run only this prefill case, e.g. Q4_K:512")
@@ -576,9 +578,11 @@ def main() -> int:
                                           cpu_steps=cpu_steps)
             log(f"[bench] decode: {line['decode']['tokens_per_s']} tok/s"
                 + (f" (CPU checker: {line['decode']['cpu_tokens_per_s']} tok/s)" if cpu_steps else ""))
-            line["decode_8b"] = bench_decode(ln, 512, 512, model_name="8b")
-        log(f"[bench] decode 8B shape: {line['decode_8b']['tokens_per_s']} tok/s, prompt pass "
-            f"{line['decode_8b']['prefill_ms']} ms")
+            if args.decode_model == "both":
+                line["decode_8b"] = bench_decode(ln, 512, 512, model_name="8b")
+        if "decode_8b" in line:
+            log(f"[bench] decode 8B shape: {line['decode_8b']['tokens_per_s']} tok/s, prompt pass "
+                f"{line['decode_8b']['prefill_ms']} ms")
     print(json.dumps(line), flush=True)
     return 0
 

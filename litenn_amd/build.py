@@ -17,7 +17,9 @@ TRACE_LIB_PATH = os.path.join(LIB_DIR, "liblitenn_hip_trace.so")
 SOURCES = ["api.hip", "gemv.hip", "gemm.hip", "glue.hip", "attn_tile.hip", "primitives.hip", "llama.hip", "gguf.hip"]
 # gemv.hip: the dispatcher hands the first six kernel arguments over in registers (the streaming
 # kernel's activation pointer, K and first-row addressing), see gemv_stream_kernel
-SOURCE_FLAGS = {"gemv.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=6"]}
+# glue.hip: the attention step's pointers, among them the device-resident position it loads first
+SOURCE_FLAGS = {"gemv.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=6"],
+                "glue.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=6"]}
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
