@@ -927,6 +927,11 @@ namespace litenn_hip
 		{
 			return 1;
 		}
+		static const int forced = env_int("LITENN_HIP_ATTN_SPLITS", 0);
+		if (forced > 0)
+		{
+			return std::min<size_t>(kMaxAttnSplits, static_cast<size_t>(forced));
+		}
 		const size_t by_len = (max_len + 63) / 64;
 		const size_t by_heads = (1024 + n_head - 1) / n_head;
 		return std::max<size_t>(1, std::min<size_t>({ kMaxAttnSplits, by_len, by_heads }));
