@@ -1,0 +1,52 @@
+"""Randomised differential test of litenn_hip_mul_mat_q against the CPU checker: formats, ragged row
+counts, every number of activation rows around the thresholds between its kernels (single-row GEMV,
+row-by-row GEMV below 16 rows, streaming and tiled matrix-core forms), K from one chunk to 8192,
+residual on or off, 16-bit activations now and then.  Seeds are fixed, so a failure names its case;
+the address arithmetic of every fetch pattern these shapes reach is walked on the host for whole
+launches by tests/cpp/fetch_bounds_test.cpp, which is where an over-fetch would be found first."""
+import numpy as np
+import pytest
+
+from conftest import rel_l2
+from litenn_amd import synth
+from litenn_amd.formats import Q2_K, Q3_K, Q4_0, Q4_1, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0, block_layout, row_bytes
+from litenn_amd.llama import MATMUL_PRECISE
+
+pytestmark = pytest.mark.gpu
+FORMATS = [Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K]
+
+
+def draw_case(seed):
+    rng = np.random.default_rng(1000 + seed)
+    fmt = FORMATS[seed % len(FORMATS)]
+    k = int(rng.choice([256, 512, 768, 1024, 2048, 2304, 4096, 6144, 8192]))
+    m = int(rng.choice([1, 2, 3, 7, 15, 16, 17, 24, 31, 32, 33, 40, 64, 100]))
+    n = int(rng.choice([1, 5, 16, 31, 100, 257, 1000, 2051, 4100]))
+    if k >= 4096 and m >= 33:
+        n = min(n, 1000)  # bounds the checker's time
+    return fmt, m, n, k, bool(rng.integers(2)), bool(rng.integers(4) == 0), bool(rng.integers(5) == 0)
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_matmul_matches_checker(hip, oracle, seed):
+    fmt, m, n, k, residual, half_x, precise = draw_case(seed)
+    what = f"seed {seed}: format {fmt} m {m} n {n} k {k} residual {residual} half {half_x} precise {precise}"
+    print(what, flush=True)
+    assert k % block_layout(fmt)[0] == 0 and row_bytes(fmt, k) > 0
+    wq = synth.quant_weights(fmt, n, k, seed, 1)
+    x = synth.activations(m, k, seed, 2)
+    if half_x:
+        x = x.astype(np.float16).astype(np.float32)
+    res = synth.activations(m, n, seed, 3) if residual else None
+    xt = hip.Tensor.from_numpy(x.astype(np.float16) if half_x else x)
+    y = hip.mul_mat_q(fmt, hip.Tensor.from_numpy(wq), n, k, xt,
+                      residual=hip.Tensor.from_numpy(res) if residual else None,
+                      flags=MATMUL_PRECISE if precise else 0).numpy()
+    want = oracle.mul_mat_q(fmt, wq, n, k, x)
+    if residual:
+        want = res + want
+    err = rel_l2(y, want)
+    print("  rel-L2 %.2e" % err, flush=True)
+    # f32 operands (single rows, fewer than 16 rows, or the flag): summation order only; matrix cores:
+    # the stated bar for Float16 operands
+    assert err <= (1e-5 if (m < 16 or precise) else 1e-3), what
