@@ -55,7 +55,7 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def bench_gemv(ln, hiprt, fmt, n, k, steps, warmup, n_buffers, seed=1):
+def bench_gemv(ln, hiprt, fmt, n, k, steps, warmup, n_buffers, seed=1, graph_rotations=16):
     """Times `steps` launches of the GEMV rotating over `n_buffers` weight buffers.
     Returns (ms_per_step from HIP events on the launch stream, wall ms per step)."""
     from litenn_amd import synth
@@ -86,7 +86,7 @@ def bench_gemv(ln, hiprt, fmt, n, k, steps, warmup, n_buffers, seed=1):
     # directly), so a graph holds up to 16 rotations; exactly `steps` kernels run, all from graphs.
     # A short run (fewer than 64 steps) is launched directly instead: the host issues a launch in
     # about 4 us, less than one takes, and the graph's start would weigh on so few kernels.
-    graph_len = min(steps, 16 * n_buffers) if steps >= 64 else 0
+    graph_len = min(steps, graph_rotations * n_buffers) if steps >= 64 else 0
 
     def capture(count):
         stream.begin_capture()
@@ -474,6 +474,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=4000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--buffers", type=int, default=16)
+    ap.add_argument("--graph-rotations", type=int, default=16,
+                    help="rotations of the weight buffers one replayed graph holds (the profiler slows long graphs "
+                         "down a great deal: its runs use 1)")
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="skip the other single-row GEMV configurations")
     ap.add_argument("--decode-prompt", type=int, default=128, help="prompt length of the decode run")
@@ -509,7 +512,8 @@ def main() -> int:
 
     n, k = 14336, 4096
     algo_bytes = n * row_bytes(Q4_K, k) + 4 * k + 4 * n
-    ms_event, ms_wall = bench_gemv(ln, hiprt, Q4_K, n, k, args.steps, args.warmup, args.buffers)
+    ms_event, ms_wall = bench_gemv(ln, hiprt, Q4_K, n, k, args.steps, args.warmup, args.buffers,
+                                   graph_rotations=max(1, args.graph_rotations))
     gbps = algo_bytes / (ms_event * 1e-3) / 1e9
     log(f"[bench] Q4_K GEMV {n}x{k}: {ms_event * 1e3:.2f} us/launch (events), {ms_wall * 1e3:.2f} us (wall), "
         f"{gbps:.0f} GB/s = {100 * gbps / HBM_PEAK_GBPS:.1f}% of HBM peak")
