@@ -1185,15 +1185,14 @@ namespace litenn_hip
 
 		// ---- the GEMM for few activation rows ------------------------------------------------------
 		// With 16 or 32 activation rows the product is a stream of the weights, like the single-row
-		// GEMV, and is built like it: one workgroup of eight wavefronts per CU, always a single round,
+		// GEMV, and is built like it: one workgroup of eight or sixteen wavefronts per CU, always a single round,
 		// each workgroup owning a run of consecutive weight rows.  The rows are walked in tiles of 16;
 		// wavefront w multiplies the tile's chunks [w CPW, (w + 1) CPW) of K, whose activation
 		// fragments (already fp16, in MFMA order) it holds in registers for the whole launch, and
 		// keeps PD tiles' worth of its slice of the raw blocks in flight towards its LDS slots with
-		// direct-to-LDS loads.  The eight partial products of a tile meet in LDS and are added in
+		// direct-to-LDS loads.  The wavefronts' partial products of a tile meet in LDS and are added in
 		// wavefront order, so the result does not depend on scheduling.  One launch, no second pass
 		// over y, every weight byte read once.
-		constexpr int kStreamWaves = 8;
 		constexpr int kStreamTilesInFlight = 2;
 
 		struct GemmStreamArgs
@@ -1215,7 +1214,7 @@ namespace litenn_hip
 			return 16 * 16 * fetch::gemm_weight_pieces(CPW * F::kChunkBytes, F::kAligned16);
 		}
 
-		template <typename F, int MT, int CPW>
+		template <typename F, int MT, int CPW, int kStreamWaves>
 		__global__ __launch_bounds__(64 * kStreamWaves) void gemm_stream_kernel(const GemmStreamArgs a)
 		{
 			constexpr int PD = kStreamTilesInFlight;
@@ -1325,7 +1324,7 @@ namespace litenn_hip
 			const int round_tiles = a.round_tiles;
 			const bool vec_ok = (a.n & 3) == 0 && (reinterpret_cast<uintptr_t>(a.y) & 15) == 0 &&
 			                    (!a.residual || (reinterpret_cast<uintptr_t>(a.residual) & 15) == 0);
-			// adds the eight partial products of tiles [first, first + count) in wavefront order and stores them
+			// adds the wavefronts' partial products of tiles [first, first + count) in wavefront order and stores them
 			const auto finish_round = [&](int first, int count) {
 				__syncthreads();
 				for (int idx = threadIdx.x; idx < count * MT * 64; idx += 64 * kStreamWaves)
@@ -1620,7 +1619,7 @@ namespace litenn_hip
 		// The streaming form takes a single matrix against at most 32 activation rows when K is a whole
 		// number of chunks per wavefront (2048 elements) whose fragments fit the registers and the slots
 		// fit LDS.  Returns false, launching nothing, otherwise.
-		template <typename F, int MT, int CPW>
+		template <typename F, int MT, int CPW, int kStreamWaves>
 		bool launch_stream_variant(const GemmCall& c, int cus)
 		{
 			constexpr size_t slots = static_cast<size_t>(kStreamWaves) * kStreamTilesInFlight * stream_slot_bytes<F, CPW>();
@@ -1651,8 +1650,8 @@ namespace litenn_hip
 				round = std::max(1, std::min(std::min(round, tiles), 8));
 				a.round_tiles = round;
 				const size_t lds = slots + round * per_round_tile;
-				allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_stream_kernel<F, MT, CPW>), kLdsLimit);
-				gemm_stream_kernel<F, MT, CPW><<<dim3(blocks), dim3(64 * kStreamWaves), lds, c.stream>>>(a);
+				allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_stream_kernel<F, MT, CPW, kStreamWaves>), kLdsLimit);
+				gemm_stream_kernel<F, MT, CPW, kStreamWaves><<<dim3(blocks), dim3(64 * kStreamWaves), lds, c.stream>>>(a);
 				return true;
 			}
 		}
@@ -1661,25 +1660,44 @@ namespace litenn_hip
 		bool launch_stream_form(const GemmCall& c, int cus)
 		{
 			static const int use_stream = env_int("LITENN_HIP_GEMM_STREAM", 1);
-			if (!use_stream || c.count != 1 || c.m_tiles > 2 || c.k % (kChunk * kStreamWaves) != 0)
+			if (!use_stream || c.count != 1 || c.m_tiles > 2 || c.k % (kChunk * 8) != 0)
 			{
 				return false;
 			}
-			const int cpw = c.k / (kChunk * kStreamWaves);
+			// Sixteen wavefronts (K cut sixteen ways) where a workgroup's run holds two tiles and more:
+			// with four wavefronts per SIMD more of the fragment decode hides behind the row stream
+			// (Q4_K 14336 x 4096: 15.2 us against 16.7 with eight).  A run of a single tile is faster
+			// with eight (Q6_K 4096 x 4096: 11.1 us against 11.8).
+			const int rows = ((c.n[0] + cus - 1) / cus + 3) / 4 * 4;
+			const bool wide = rows > 16 && c.k % (kChunk * 16) == 0;
+			const int cpw = c.k / (kChunk * (wide ? 16 : 8));
 			if (c.m_tiles == 1)
 			{
+				if (wide)
+				{
+					switch (cpw)
+					{
+					case 1: return launch_stream_variant<F, 1, 1, 16>(c, cus);
+					case 2: return launch_stream_variant<F, 1, 2, 16>(c, cus);
+					default: return false;
+					}
+				}
 				switch (cpw)
 				{
-				case 1: return launch_stream_variant<F, 1, 1>(c, cus);
-				case 2: return launch_stream_variant<F, 1, 2>(c, cus);
-				case 4: return launch_stream_variant<F, 1, 4>(c, cus);
+				case 1: return launch_stream_variant<F, 1, 1, 8>(c, cus);
+				case 2: return launch_stream_variant<F, 1, 2, 8>(c, cus);
+				case 4: return launch_stream_variant<F, 1, 4, 8>(c, cus);
 				default: return false;
 				}
 			}
-			switch (cpw)
+			if (wide && cpw == 1)
 			{
-			case 1: return launch_stream_variant<F, 2, 1>(c, cus);
-			case 2: return launch_stream_variant<F, 2, 2>(c, cus);
+				return launch_stream_variant<F, 2, 1, 16>(c, cus);
+			}
+			switch (c.k / (kChunk * 8))
+			{
+			case 1: return launch_stream_variant<F, 2, 1, 8>(c, cus);
+			case 2: return launch_stream_variant<F, 2, 2, 8>(c, cus);
 			default: return false;
 			}
 		}

@@ -175,7 +175,7 @@ static void test_gemm_weight_pieces()
 }
 
 // ---- streaming GEMM for few activation rows -----------------------------------------------------
-// A workgroup owns a run of consecutive rows and walks it in tiles of 16; wavefront w of eight fetches
+// A workgroup owns a run of consecutive rows and walks it in tiles of 16; wavefront w of eight or sixteen fetches
 // the bytes of chunks [w cpw, (w + 1) cpw) of every row of a tile (its slice) with the matrix-core
 // GEMM's piece arithmetic, the slice in the place of a chunk.
 static void test_gemm_stream_pieces()
@@ -183,10 +183,11 @@ static void test_gemm_stream_pieces()
 	long cases = 0;
 	for (const Format& f : kFormats)
 	{
-		for (int cpw : { 1, 2, 4 })
+		for (int geometry : { 801, 802, 804, 1601, 1602 }) // wavefronts x 100 + chunks per wavefront
 		{
+			const int waves = geometry / 100, cpw = geometry % 100;
 			const int slice_bytes = cpw * f.chunk_bytes;
-			const size_t row_bytes = static_cast<size_t>(8) * slice_bytes;
+			const size_t row_bytes = static_cast<size_t>(waves) * slice_bytes;
 			const int pieces = fm::gemm_weight_pieces(slice_bytes, f.aligned16);
 			const int loads = (16 * pieces + 63) / 64;
 			for (int n : { 1, 15, 16, 17, 56, 57, 100, 300 })
@@ -219,7 +220,7 @@ static void test_gemm_stream_pieces()
 							const int last_row = row0 + block_rows - 1;
 							for (int t = 0; t < (block_rows + 15) / 16; ++t)
 							{
-								for (int wave = 0; wave < 8; ++wave)
+								for (int wave = 0; wave < waves; ++wave)
 								{
 									std::vector<uintptr_t> slot(static_cast<size_t>(loads) * 64, 0); // by 16-byte piece of the slot
 									for (int i = 0; i < loads; ++i)
