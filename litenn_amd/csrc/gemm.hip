@@ -1669,30 +1669,34 @@ namespace litenn_hip
 			// (Q4_K 14336 x 4096: 15.2 us against 16.7 with eight).  A run of a single tile is faster
 			// with eight (Q6_K 4096 x 4096: 11.1 us against 11.8).
 			const int rows = ((c.n[0] + cus - 1) / cus + 3) / 4 * 4;
-			const bool wide = rows > 16 && c.k % (kChunk * 16) == 0;
-			const int cpw = c.k / (kChunk * (wide ? 16 : 8));
 			if (c.m_tiles == 1)
 			{
-				if (wide)
+				// (only where the sixteen-wavefront instance keeps its registers: one chunk per wavefront,
+				// one activation tile, and not the formats whose decoders need the most of them)
+				constexpr bool wide_fits = !std::is_same<F, Q3_KFrag>::value && !std::is_same<F, Q6_KFrag>::value &&
+				                           !std::is_same<F, Q8_0Frag>::value;
+				if constexpr (wide_fits)
 				{
-					switch (cpw)
+					if (rows > 16 && c.k == kChunk * 16)
 					{
-					case 1: return launch_stream_variant<F, 1, 1, 16>(c, cus);
-					case 2: return launch_stream_variant<F, 1, 2, 16>(c, cus);
-					default: return false;
+						return launch_stream_variant<F, 1, 1, 16>(c, cus);
 					}
 				}
-				switch (cpw)
+				switch (c.k / (kChunk * 8))
 				{
 				case 1: return launch_stream_variant<F, 1, 1, 8>(c, cus);
 				case 2: return launch_stream_variant<F, 1, 2, 8>(c, cus);
-				case 4: return launch_stream_variant<F, 1, 4, 8>(c, cus);
+				case 4:
+					if constexpr (std::is_same<F, Q3_KFrag>::value)
+					{
+						return false; // its decoder and 128 registers of fragments do not fit: the tiled kernel takes it
+					}
+					else
+					{
+						return launch_stream_variant<F, 1, 4, 8>(c, cus);
+					}
 				default: return false;
 				}
-			}
-			if (wide && cpw == 1)
-			{
-				return launch_stream_variant<F, 2, 1, 16>(c, cus);
 			}
 			switch (c.k / (kChunk * 8))
 			{
