@@ -209,9 +209,10 @@ int litenn_hip_attn_decode(int dev, const void* q, const void* kcache, const voi
  * GPU, held until the process ends) instead of memory allocated and freed by the call.  No
  * counterpart in the reference.  The call allocates nothing, records no memset node, and honours
  * opts->synchronize like every other entry point.  It refuses a launch whose chunks do not fit:
- * a single row (m == 1) is cut into c = min(16, ceil(keys / 64), ceil(1024 / n_head)) chunks and
- * needs n_head * c * (head_dim + 2) <= 262144 floats, which holds for every head_dim <= 128 and
- * e.g. for 48 heads of 256 features but not for 64.  Every call on one GPU shares that GPU's array:
+ * a single row (m == 1) is cut into c = min(16, ceil(keys / 64), round(2.2 * sqrt(keys / 64)),
+ * ceil(1024 / n_head)) chunks and needs n_head * c * (head_dim + 2) <= 262144 floats, which holds
+ * for every head_dim <= 128 and, at the 16 chunks of a long cache, e.g. for 48 heads of 256
+ * features but not for 64.  Every call on one GPU shares that GPU's array:
  * calls that overlap on one GPU (two streams, two threads) race and must be serialised by the
  * caller. */
 int litenn_hip_attn_decode_noalloc(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype,

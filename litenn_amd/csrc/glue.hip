@@ -313,6 +313,23 @@ namespace litenn_hip
 
 		constexpr int kMaxAttnSplits = 16;
 
+		// Key chunks a single row's attention over `len` cached keys is cut into: the nearest integer
+		// to 2.2 sqrt(len / 64), within 1 .. 16 (3 at 128 keys, 6 at 512, 9 at 1024, 16 from 3400 on).
+		// More chunks shorten a chunk's key loop and lengthen nothing but the merge, whose cost hardly
+		// depends on their number; measured in the decoder, 8B shape at 512 .. 1024 keys: 2 chunks
+		// 574, 4: 602, 6: 608, 8: 606, 12: 602, 16: 600 tok/s; 7B shape at 128 .. 384 keys flat within
+		// 2 % from 3 to 8.  Integer arithmetic, so the host (which sizes the grid) and the kernel
+		// (which reads the length on the device) agree: c + 1 chunks from (2c + 1)^2 * 400 <= 121 len.
+		__host__ __device__ inline int attn_live_chunks(long long len)
+		{
+			int c = 1;
+			while (c < kMaxAttnSplits && static_cast<long long>(2 * c + 1) * (2 * c + 1) * 400 <= 121 * len)
+			{
+				++c;
+			}
+			return c;
+		}
+
 		__device__ __forceinline__ void device_store(float* p, float v)
 		{
 			__hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -437,12 +454,19 @@ namespace litenn_hip
 			__shared__ float s_o[16][256 + 4];
 			__shared__ int s_last;
 			const int h = blockIdx.x;
-			const int split = blockIdx.y, splits = gridDim.y;
+			const int split = blockIdx.y;
 			const int row = blockIdx.z;
 			const int tid = threadIdx.x;
 			const int past = past_dev ? *past_dev : past_host;
 			const int pos = past + row;
 			const int len = FUSED ? pos : pos + 1; // keys read from the cache
+			// The grid holds the chunks of the longest cache the launch may meet (a captured launch is
+			// replayed while the cache fills); the chunks this length does not need leave at once.
+			const int splits = min(static_cast<int>(gridDim.y), attn_live_chunks(len));
+			if (split >= splits)
+			{
+				return;
+			}
 			const int kvh = h / (n_head / n_kv_head);
 			const size_t kvw = static_cast<size_t>(n_kv_head) * head_dim;
 			const float* qr = q + (static_cast<size_t>(row) * n_head + h) * head_dim;
@@ -918,23 +942,24 @@ namespace litenn_hip
 		}
 	}
 
-	// Number of key chunks one query row is cut into.  Only a single row is ever split (several
-	// rows already give the machine enough workgroups); the count depends on the upper bound of
-	// the key length alone, so a captured launch stays valid while the cache fills.
+	// Upper bound of the key chunks one query row is cut into, which is the grid's second extent and
+	// sizes the scratch.  Only a single row is ever split (several rows already give the machine
+	// enough workgroups).  It depends on the upper bound of the key length alone, so a captured
+	// launch stays valid while the cache fills; the kernel itself uses as many of the grid's chunks
+	// as the length it finds on the device asks for.
 	size_t attn_splits(size_t m, size_t max_len, size_t n_head)
 	{
 		if (m != 1)
 		{
 			return 1;
 		}
+		// the kernel cuts a row into min(grid, attn_live_chunks(keys)) chunks; the grid is capped so that
+		// a launch stays near a thousand workgroups, and by LITENN_HIP_ATTN_SPLITS for experiments
 		static const int forced = env_int("LITENN_HIP_ATTN_SPLITS", 0);
-		if (forced > 0)
-		{
-			return std::min<size_t>(kMaxAttnSplits, static_cast<size_t>(forced));
-		}
-		const size_t by_len = (max_len + 63) / 64;
+		const size_t cap = forced > 0 ? std::min<size_t>(kMaxAttnSplits, static_cast<size_t>(forced)) : kMaxAttnSplits;
+		const size_t by_len = static_cast<size_t>(attn_live_chunks(static_cast<long long>(max_len)));
 		const size_t by_heads = (1024 + n_head - 1) / n_head;
-		return std::max<size_t>(1, std::min<size_t>({ kMaxAttnSplits, by_len, by_heads }));
+		return std::max<size_t>(1, std::min<size_t>({ cap, by_len, by_heads }));
 	}
 
 	// floats of `partial` a launch with that many splits needs (and m * n_head zeroed ints of counters)

@@ -272,8 +272,8 @@ def test_linear_rope_scaling_and_partial_rotation(hip, oracle, tmp_path):
 def test_a_context_of_forty_thousand_positions(hip, oracle):
     """Nothing in the runtime holds per-key storage, so the context is bounded by the caches' memory
     only: a model declared with 40000 positions (beyond what an earlier score buffer held) is created,
-    evaluates a prompt and single steps like any other, and its attention is cut into key chunks
-    sized for the declared context from the first token on."""
+    evaluates a prompt and single steps like any other (the key chunks of a single row's attention
+    follow the cache's current length, not the declared context)."""
     cfg = synth.tiny_llama(Q4_0, block_count=2, d_model=256, heads=4, kv_heads=2, ff=512, vocab=300,
                            context_length=40000)
     toks = synth.prompt_tokens(cfg, 24, 12)
@@ -284,4 +284,28 @@ def test_a_context_of_forty_thousand_positions(hip, oracle):
     dev.reset()
     ref.reset()
     assert dev.generate(toks[:5], 10)[0].tolist() == ref.generate(toks[:5], 10)[0].tolist()
+    dev.close()
+
+
+def test_generation_across_a_doubling_of_the_cache_length(hip, oracle):
+    """The number of key chunks a single row's attention is cut into follows the cache length the
+    kernel finds on the device, so it changes several times under one captured step: a run that
+    starts at 250 rows and ends above 512 must give the checker's tokens, the same tokens as
+    evaluation one token at a time (whose launches are sized on the host), and the same cache."""
+    cfg = synth.tiny_llama(Q4_0, block_count=2, d_model=256, heads=4, kv_heads=2, ff=512, vocab=300,
+                           context_length=2048)
+    prompt = synth.prompt_tokens(cfg, 250, 21)
+    dev, ref = hip_model(hip, cfg, 6, kv_dtype=DT_F32), oracle_model(oracle, cfg, 6, kv_f16=False)
+    got, _, _ = dev.generate(prompt, 280)
+    assert dev.past == 250 + 279
+    want, _ = ref.generate(prompt, 280)
+    assert got.tolist() == want.tolist(), np.nonzero(got != want)[0][:4]
+    kv = dev.get_kv(1)
+    dev.reset()
+    logits = dev.eval(prompt, all_logits=False)
+    for step in range(279):
+        assert int(np.argmax(logits)) == int(got[step]), step
+        logits = dev.eval([int(got[step])], all_logits=False)
+    for a, b in zip(dev.get_kv(1), kv):
+        assert np.array_equal(a, b)
     dev.close()

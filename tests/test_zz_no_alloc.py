@@ -80,12 +80,12 @@ def test_repeated_calls_reuse_the_scratch(hip):
 
 
 def test_sizes_beyond_the_scratch_are_refused(hip):
-    """64 heads of 256 features cut into 16 chunks need 64 * 16 * 258 floats, more than the fixed
-    array holds: an error return with a clear message, no launch.  The allocating entry point takes
-    the same shape."""
+    """64 heads of 256 features cut into 16 chunks (a cache of 4096 rows) need 64 * 16 * 258 floats,
+    more than the fixed array holds: an error return with a clear message, no launch.  The
+    allocating entry point takes such heads."""
     lib = _lib.load()
     one = ctypes.c_void_p(256)  # never dereferenced: the call fails in validation
-    assert lib.litenn_hip_attn_decode_noalloc(0, one, one, one, DT_F16, 1, 1023, 64, 8, 256, one, None) != 0
+    assert lib.litenn_hip_attn_decode_noalloc(0, one, one, one, DT_F16, 1, 4095, 64, 8, 256, one, None) != 0
     assert b"static scratch" in lib.litenn_hip_last_error()
     rng = np.random.default_rng(79)
     q, k, v, qd, kc, vc = _case(hip, rng, 1, 1023, 64, 8, 256, DT_F16)
