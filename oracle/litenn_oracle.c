@@ -905,6 +905,146 @@ void oracle_attention_head(const float* q, size_t mq, const float* k, const floa
 	free(s);
 }
 
+/* Detail::ComputeALiBiSlope, FlashAttnExt.h:69-96: 1 when maxBias <= 0 */
+double oracle_alibi_slope(size_t head_index, size_t head_count, double max_bias)
+{
+	if (max_bias <= 0.0)
+	{
+		return 1.0;
+	}
+	size_t head_log2 = 1;
+	while ((head_log2 << 1) <= head_count)
+	{
+		head_log2 <<= 1;
+	}
+	const double m0 = pow(2.0, -max_bias / (double)head_log2);
+	const double m1 = pow(2.0, -(max_bias / 2.0) / (double)head_log2);
+	if (head_index < head_log2)
+	{
+		return pow(m0, (double)(head_index + 1));
+	}
+	return pow(m1, (double)(2 * (head_index - head_log2) + 1));
+}
+
+/* One head of AddFlashAttnExt with every option, node by node in f32 (FlashAttnExt.h:126-228):
+ * MatMul, scalar multiply by scale (or scale / softcap), AddTanh as (exp(2x) - 1) / (exp(2x) + 1)
+ * (Activation.h:34-50) and multiply by softcap, + mask (times the ALiBi slope when maxBias > 0),
+ * + causal mask (CausalMask.h:16-34), row max (joined with the sink), exp, sequential sum (+ the
+ * sink's term), divide, MatMul.  A scalar multiply by exactly 1 is not emitted (:57-67). */
+void oracle_flash_attn_ext(const float* q, size_t mq, const float* k, const float* v, size_t l, size_t d, size_t dv,
+                           double scale, double logit_softcap, const float* mask, double mask_slope,
+                           const float* sink, int causal, size_t key_pos_offset, size_t query_pos_offset, float* out)
+{
+	float* s = (float*)malloc(sizeof(float) * (l ? l : 1));
+	const double score_scale = logit_softcap != 0.0 ? scale / logit_softcap : scale;
+	const float score_scale_f = (float)score_scale; /* MakeScalarTensor(f32, .) */
+	const float softcap_f = (float)logit_softcap;
+	const float slope_f = (float)mask_slope;
+	const float masked = (float)-1.0e9;
+	for (size_t row = 0; row < mq; ++row)
+	{
+		for (size_t col = 0; col < l; ++col)
+		{
+			s[col] = 0.0f;
+		}
+		for (size_t kk = 0; kk < d; ++kk)
+		{
+			const float lhs = q[row * d + kk];
+			for (size_t col = 0; col < l; ++col)
+			{
+				s[col] += lhs * k[col * d + kk];
+			}
+		}
+		if ((scale != 1.0 || logit_softcap != 0.0) && score_scale != 1.0)
+		{
+			for (size_t col = 0; col < l; ++col)
+			{
+				s[col] = s[col] * score_scale_f;
+			}
+		}
+		if (logit_softcap != 0.0)
+		{
+			for (size_t col = 0; col < l; ++col)
+			{
+				const float scaled = s[col] * 2.0f;
+				const float e = expf(scaled);
+				const float numerator = e - 1.0f;
+				const float denominator = e + 1.0f;
+				s[col] = numerator / denominator;
+			}
+			if (logit_softcap != 1.0)
+			{
+				for (size_t col = 0; col < l; ++col)
+				{
+					s[col] = s[col] * softcap_f;
+				}
+			}
+		}
+		if (mask)
+		{
+			for (size_t col = 0; col < l; ++col)
+			{
+				float mv = mask[row * l + col];
+				if (mask_slope != 1.0)
+				{
+					mv = mv * slope_f;
+				}
+				s[col] = s[col] + mv;
+			}
+		}
+		if (causal)
+		{
+			for (size_t col = 0; col < l; ++col)
+			{
+				const float cm = (key_pos_offset + col > query_pos_offset + row) ? masked : 0.0f;
+				s[col] = s[col] + cm;
+			}
+		}
+		float mx = s[0];
+		for (size_t col = 1; col < l; ++col)
+		{
+			if (s[col] > mx)
+			{
+				mx = s[col];
+			}
+		}
+		if (sink && *sink > mx) /* BinaryOp::Max(maxScores, sink) */
+		{
+			mx = *sink;
+		}
+		for (size_t col = 0; col < l; ++col)
+		{
+			s[col] = expf(s[col] - mx);
+		}
+		float denom = s[0];
+		for (size_t col = 1; col < l; ++col)
+		{
+			denom += s[col];
+		}
+		if (sink)
+		{
+			denom = denom + expf(*sink - mx);
+		}
+		for (size_t col = 0; col < l; ++col)
+		{
+			s[col] = s[col] / denom;
+		}
+		for (size_t c = 0; c < dv; ++c)
+		{
+			out[row * dv + c] = 0.0f;
+		}
+		for (size_t col = 0; col < l; ++col)
+		{
+			const float p = s[col];
+			for (size_t c = 0; c < dv; ++c)
+			{
+				out[row * dv + c] += p * v[col * dv + c];
+			}
+		}
+	}
+	free(s);
+}
+
 /* Activation.h:22-35,56-63 */
 void oracle_silu(const float* x, float* y, size_t n)
 {

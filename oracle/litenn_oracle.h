@@ -109,6 +109,16 @@ void oracle_rope(const float* x, float* y, size_t m, size_t d, size_t rope_dims,
 void oracle_attention_head(const float* q, size_t mq, const float* k, const float* v, size_t l, size_t d, size_t dv,
                            double scale, int causal, size_t key_pos_offset, size_t query_pos_offset, float* out);
 
+/* Detail::ComputeALiBiSlope, src/LiteNN/Layer/FlashAttnExt.h:69-96 */
+double oracle_alibi_slope(size_t head_index, size_t head_count, double max_bias);
+/* One head of AddFlashAttnExt with every option (src/LiteNN/Layer/FlashAttnExt.h:17-29,126-228):
+ * logit softcap (tanh composed as in Activation.h:34-50), additive mask [mq, l] times mask_slope
+ * (oracle_alibi_slope, 1 when maxBias is off; NULL = no mask), scalar sink (NULL = none), causal
+ * mask with position offsets. */
+void oracle_flash_attn_ext(const float* q, size_t mq, const float* k, const float* v, size_t l, size_t d, size_t dv,
+                           double scale, double logit_softcap, const float* mask, double mask_slope,
+                           const float* sink, int causal, size_t key_pos_offset, size_t query_pos_offset, float* out);
+
 /* AddSiLU / AddSigmoid, src/LiteNN/Layer/Activation.h:22-63 */
 void oracle_silu(const float* x, float* y, size_t n);
 /* gated = silu(gate) * up, src/LiteNN/Layer/SwiGLU.h:59-69 */

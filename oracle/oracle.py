@@ -60,6 +60,9 @@ def lib() -> C.CDLL:
         L.oracle_rmsnorm.argtypes = [vp, vp, f64, sz, sz, vp]
         L.oracle_rope.argtypes = [vp, vp, sz, sz, sz, f64, f64, sz]
         L.oracle_attention_head.argtypes = [vp, sz, vp, vp, sz, sz, sz, f64, i32, sz, sz, vp]
+        L.oracle_alibi_slope.argtypes = [sz, sz, f64]
+        L.oracle_alibi_slope.restype = f64
+        L.oracle_flash_attn_ext.argtypes = [vp, sz, vp, vp, sz, sz, sz, f64, f64, vp, f64, vp, i32, sz, sz, vp]
         L.oracle_silu.argtypes = [vp, vp, sz]
         L.oracle_silu_mul.argtypes = [vp, vp, vp, sz]
         L.oracle_get_rows.argtypes = [vp, sz, sz, vp, sz, vp]
@@ -195,6 +198,31 @@ def attention_head(q, k, v, scale: float = 1.0, causal: bool = False, key_pos_of
     out = np.empty((mq, dv), np.float32)
     lib().oracle_attention_head(_p(q), mq, _p(k), _p(v), l, d, dv, scale, int(causal), key_pos_offset,
                                 query_pos_offset, _p(out))
+    return out
+
+
+def alibi_slope(head_index: int, head_count: int, max_bias: float) -> float:
+    return float(lib().oracle_alibi_slope(head_index, head_count, max_bias))
+
+
+def flash_attn_ext(q, k, v, scale: float = 1.0, softcap: float = 0.0, mask=None, max_bias: float = 0.0,
+                   head_index: int = 0, head_count: int = 1, sink=None, causal: bool = False,
+                   key_pos_offset: int = 0, query_pos_offset: int = 0) -> np.ndarray:
+    """One head of the reference's AddFlashAttnExt with its options (FlashAttnExt.h:17-29,100-228)."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    mq, d = q.shape
+    l, dv = v.shape
+    assert k.shape == (l, d)
+    if max_bias > 0.0 and mask is None:
+        raise ValueError("FlashAttnExt maxBias requires an explicit additive mask")
+    m_arr = None if mask is None else _f32(mask)
+    assert m_arr is None or m_arr.shape == (mq, l)
+    s_arr = None if sink is None else np.array([sink], np.float32)
+    out = np.empty((mq, dv), np.float32)
+    lib().oracle_flash_attn_ext(_p(q), mq, _p(k), _p(v), l, d, dv, scale, softcap,
+                                None if m_arr is None else _p(m_arr), alibi_slope(head_index, head_count, max_bias),
+                                None if s_arr is None else _p(s_arr), int(causal), key_pos_offset, query_pos_offset,
+                                _p(out))
     return out
 
 

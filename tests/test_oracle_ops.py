@@ -29,6 +29,45 @@ def attention_expected_f64(q, k, v, scale, causal, key_off, query_off):
     return out
 
 
+def alibi_slope_f64(head_index, head_count, max_bias):
+    """ComputeALiBiSlope of the reference's test (tests/LayerTest.cpp:89-111), in Python floats."""
+    if max_bias <= 0.0:
+        return 1.0
+    head_log2 = 1
+    while head_log2 * 2 <= head_count:
+        head_log2 *= 2
+    m0 = 2.0 ** (-max_bias / head_log2)
+    m1 = 2.0 ** (-(max_bias / 2.0) / head_log2)
+    if head_index < head_log2:
+        return m0 ** (head_index + 1)
+    return m1 ** (2 * (head_index - head_log2) + 1)
+
+
+def attention_ext_expected_f64(q, k, v, scale=1.0, softcap=0.0, mask=None, slope=1.0, sink=None, causal=False,
+                               key_off=0, query_off=0):
+    """ComputeFlashAttnExpected (tests/LayerTest.cpp:112-183) with every option: scores in double,
+    softcap * tanh(score / softcap) with the library tanh (not the f32 exp composition the layer
+    lowers to), slope * mask, causal offset mask, the sink joins the maximum and the denominator."""
+    q, k, v = (np.asarray(a, np.float64) for a in (q, k, v))
+    out = np.zeros((q.shape[0], v.shape[1]), np.float32)
+    cols = np.arange(k.shape[0])
+    for row in range(q.shape[0]):
+        scores = (k @ q[row]) * float(np.float32(scale))
+        if softcap != 0.0:
+            cap = float(np.float32(softcap))
+            scores = cap * np.tanh(scores / cap)
+        if mask is not None:
+            scores = scores + slope * np.asarray(mask, np.float32).astype(np.float64)[row]
+        if causal:
+            scores = scores + np.where(key_off + cols > query_off + row, -1.0e9, 0.0)
+        top = scores.max() if sink is None else max(scores.max(), float(np.float32(sink)))
+        p = np.exp(scores - top)
+        denom = p.sum() + (0.0 if sink is None else math.exp(float(np.float32(sink)) - top))
+        for col in range(k.shape[0]):
+            out[row] += (p[col] / denom * v[col]).astype(np.float32)
+    return out
+
+
 def test_matmul_reference_vectors(oracle, golden):
     for case in golden["matmul"]:
         y = oracle.matmul_ikj(case["a"], case["b"])
@@ -170,6 +209,63 @@ def test_attention_properties(oracle):
     # constant values => output is that constant (softmax rows sum to one)
     const = oracle.attention_head(q, k, np.full((9, 3), 2.5, np.float32), scale, False)
     assert np.allclose(const, 2.5, atol=1e-6)
+
+
+def test_attention_options_reference_vector(oracle, golden):
+    """The reference's mask + softcap + sinks case (ALiBi slope of head 1 of 4 at maxBias 4), held to
+    its own double-precision checker at its own tolerance."""
+    c = golden["attention_ext"][0]
+    slope = alibi_slope_f64(c["head_index"], c["head_count"], c["max_bias"])
+    assert slope == 0.25  # 2^(-4/4) squared
+    assert oracle.alibi_slope(c["head_index"], c["head_count"], c["max_bias"]) == slope
+    got = oracle.flash_attn_ext(c["q"], c["k"], c["v"], c["scale"], c["logit_softcap"], c["mask"], c["max_bias"],
+                                c["head_index"], c["head_count"], c["sink"])
+    want = attention_ext_expected_f64(c["q"], c["k"], c["v"], c["scale"], c["logit_softcap"], c["mask"], slope, c["sink"])
+    assert np.allclose(got, want, atol=c["tol"])
+    # every option matters in this case: dropping one moves the result by far more than the tolerance
+    for drop in ("logit_softcap", "mask", "sink", "max_bias"):
+        o = dict(c)
+        o[drop] = {"logit_softcap": 0.0, "mask": None, "sink": None, "max_bias": 0.0}[drop]
+        if o["mask"] is None:
+            o["max_bias"] = 0.0
+        other = oracle.flash_attn_ext(o["q"], o["k"], o["v"], o["scale"], o["logit_softcap"], o["mask"], o["max_bias"],
+                                      o["head_index"], o["head_count"], o["sink"])
+        assert np.abs(other - want).max() > 1e-3, drop
+
+
+def test_attention_options_against_f64_checker(oracle):
+    rng = np.random.default_rng(29)
+    for case in range(24):
+        mq, l, d, dv = int(rng.integers(1, 6)), int(rng.integers(1, 40)), int(rng.choice([2, 16, 64, 128])), int(rng.integers(1, 9))
+        q = rng.standard_normal((mq, d)).astype(np.float32)
+        k = rng.standard_normal((l, d)).astype(np.float32)
+        v = rng.standard_normal((l, dv)).astype(np.float32)
+        scale = float(rng.choice([1.0, 1.0 / math.sqrt(d), 1.25]))
+        softcap = float(rng.choice([0.0, 0.75, 1.0, 30.0]))
+        mask = rng.standard_normal((mq, l)).astype(np.float32) if rng.random() < 0.6 else None
+        heads = int(rng.choice([1, 4, 6, 12]))
+        head = int(rng.integers(0, heads))
+        max_bias = float(rng.choice([0.0, 4.0, 8.0])) if mask is not None else 0.0
+        sink = float(rng.standard_normal()) if rng.random() < 0.5 else None
+        causal = bool(rng.random() < 0.5)
+        key_off = int(rng.integers(0, 3))
+        query_off = key_off + int(rng.integers(0, l + 2))  # the first row always sees key 0
+        slope = alibi_slope_f64(head, heads, max_bias)
+        assert abs(oracle.alibi_slope(head, heads, max_bias) - slope) <= 1e-15 * slope
+        got = oracle.flash_attn_ext(q, k, v, scale, softcap, mask, max_bias, head, heads, sink, causal, key_off, query_off)
+        want = attention_ext_expected_f64(q, k, v, scale, softcap, mask, slope, sink, causal, key_off, query_off)
+        assert np.allclose(got, want, atol=2e-5, rtol=1e-5), case
+    # with every option off it is the plain head, bit for bit
+    q = rng.standard_normal((3, 64)).astype(np.float32)
+    k = rng.standard_normal((17, 64)).astype(np.float32)
+    v = rng.standard_normal((17, 64)).astype(np.float32)
+    assert np.array_equal(oracle.flash_attn_ext(q, k, v, 0.125, causal=True, query_pos_offset=14),
+                          oracle.attention_head(q, k, v, 0.125, True, 0, 14))
+    # non-power-of-two head counts: heads past the largest power of two take the interleaved slopes
+    assert oracle.alibi_slope(4, 6, 8.0) == 2.0 ** (-(8.0 / 2) / 4)
+    assert oracle.alibi_slope(5, 6, 8.0) == (2.0 ** (-(8.0 / 2) / 4)) ** 3
+    with pytest.raises(ValueError, match="maxBias requires"):
+        oracle.flash_attn_ext(q, k, v, max_bias=4.0)
 
 
 def test_silu_and_swiglu_reference_vectors(oracle, golden):
