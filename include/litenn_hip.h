@@ -229,6 +229,32 @@ int litenn_hip_attn_decode_noalloc(int dev, const void* q, const void* kcache, c
 int litenn_hip_attn_rows(int dev, const void* q, const void* kcache, const void* vcache, int cache_dtype, size_t m,
                          size_t past, size_t n_head, size_t n_kv_head, size_t head_dim, void* out, unsigned flags,
                          const litenn_hip_exec* opts);
+/* The options of the reference's attention layer (FlashAttnExtOptions,
+ * src/LiteNN/Layer/FlashAttnExt.h:17-29) for all heads of one call; headIndex / headCount are the
+ * head's index and n_head. */
+typedef struct litenn_hip_attn_ext_opts
+{
+	double scale;         /* multiplies q.k; 1 = none */
+	double max_bias;      /* > 0: the mask is multiplied by the head's ALiBi slope; needs a mask */
+	double logit_softcap; /* != 0: scores become softcap * tanh(scale * q.k / softcap) */
+	const void* mask;     /* additive F32 [m, keys] on the device, shared by the heads, or NULL */
+	const void* sinks;    /* F32 [n_head] on the device, one scalar sink per head, or NULL */
+	int causal;           /* adds -1e9 where key_position_offset + key > query_position_offset + row */
+	size_t key_position_offset;
+	size_t query_position_offset;
+} litenn_hip_attn_ext_opts;
+/* AddFlashAttnExt with its options for every head at once
+ * (src/LiteNN/Layer/FlashAttnExt.h:100-228; causal mask src/LiteNN/Layer/CausalMask.h:16-34; tanh
+ * as the layer composes it, src/LiteNN/Layer/Activation.h:34-50): q [m, n_head, head_dim] F32,
+ * k / v [keys, n_kv_head, head_dim] F16 or F32, out [m, n_head, head_dim] F32; query head h reads kv
+ * head h / (n_head / n_kv_head).  o == NULL means no option (scale 1, no mask).  The LLaMA lowering
+ * uses none of the options and goes through litenn_hip_attn_decode / litenn_hip_attn_rows; this
+ * entry point is a plain f32 row kernel.  The tanh is (exp(2x) - 1) / (exp(2x) + 1) in f32 as in the
+ * reference, NaN once 2x exceeds 88.  Refused: max_bias without a mask (the reference's text), a
+ * causal mask that hides every key from the first row. */
+int litenn_hip_flash_attn_ext(int dev, const void* q, const void* k, const void* v, int kv_dtype, size_t m, size_t keys,
+                              size_t n_head, size_t n_kv_head, size_t head_dim, const litenn_hip_attn_ext_opts* o,
+                              void* out, const litenn_hip_exec* opts);
 /* y = silu(gate) * up (src/LiteNN/Layer/SwiGLU.h:59-69, Activation.h:22-63) */
 int litenn_hip_silu_mul(int dev, const void* gate, const void* up, void* y, size_t n, const litenn_hip_exec* opts);
 /* out_index[row] (I32) = first maximal index of x[row, :] (f32); ties pick the lowest index

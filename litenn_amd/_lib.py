@@ -27,6 +27,15 @@ class LlamaParams(C.Structure):
     ]
 
 
+class AttnExtOpts(C.Structure):
+    """litenn_hip_attn_ext_opts: the reference layer's FlashAttnExtOptions for all heads of one call."""
+    _fields_ = [
+        ("scale", C.c_double), ("max_bias", C.c_double), ("logit_softcap", C.c_double), ("mask", C.c_void_p),
+        ("sinks", C.c_void_p), ("causal", C.c_int), ("key_position_offset", C.c_size_t),
+        ("query_position_offset", C.c_size_t),
+    ]
+
+
 class GgufTensor(C.Structure):
     _fields_ = [
         ("name", C.c_char_p), ("ggml_type", C.c_int), ("fmt", C.c_int), ("dtype", C.c_int), ("quantized", C.c_int),
@@ -69,6 +78,7 @@ SIGNATURES = {
     "litenn_hip_attn_decode": [_i, _vp, _vp, _vp, _i, _sz, _sz, _sz, _sz, _sz, _vp, _ex],
     "litenn_hip_attn_decode_noalloc": [_i, _vp, _vp, _vp, _i, _sz, _sz, _sz, _sz, _sz, _vp, _ex],
     "litenn_hip_attn_rows": [_i, _vp, _vp, _vp, _i, _sz, _sz, _sz, _sz, _sz, _vp, _u, _ex],
+    "litenn_hip_flash_attn_ext": [_i, _vp, _vp, _vp, _i, _sz, _sz, _sz, _sz, _sz, C.POINTER(AttnExtOpts), _vp, _ex],
     "litenn_hip_silu_mul": [_i, _vp, _vp, _vp, _sz, _ex],
     "litenn_hip_argmax": [_i, _vp, _sz, _sz, _vp, _ex],
     "litenn_hip_llama_create": [_i, C.POINTER(LlamaParams), C.POINTER(_vp)],

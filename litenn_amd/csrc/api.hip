@@ -43,6 +43,10 @@ namespace litenn_hip
 	hipError_t launch_attn_decode_static(const float* q, const void* kcache, const void* vcache, int cache_dtype,
 	                                     size_t m, size_t past_host, size_t n_head, size_t n_kv_head, size_t head_dim,
 	                                     float* out, size_t splits, hipStream_t s);
+	void launch_attn_ext(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m, size_t keys,
+	                     size_t n_head, size_t n_kv_head, size_t head_dim, double scale, double max_bias,
+	                     double logit_softcap, const float* mask, const float* sinks, bool causal, size_t key_offset,
+	                     size_t query_offset, float* out, hipStream_t s);
 	void launch_silu_mul(const float* gate, const float* up, float* y, size_t n, hipStream_t s);
 	void launch_zero_ints(int* p, size_t n, hipStream_t s);
 	void launch_argmax(const float* x, size_t rows, size_t n, int32_t* out, hipStream_t s);
@@ -1180,6 +1184,54 @@ extern "C" int litenn_hip_attn_rows(int dev, const void* q, const void* kcache, 
 {
 	return attn_rows_impl(dev, q, kcache, vcache, cache_dtype, m, past, n_head, n_kv_head, head_dim, out,
 	                      !(flags & LITENN_HIP_MATMUL_PRECISE), opts);
+}
+
+extern "C" int litenn_hip_flash_attn_ext(int dev, const void* q, const void* k, const void* v, int kv_dtype, size_t m,
+                                        size_t keys, size_t n_head, size_t n_kv_head, size_t head_dim,
+                                        const litenn_hip_attn_ext_opts* o, void* out, const litenn_hip_exec* opts)
+{
+	const char* action = "HIP FlashAttnExt";
+	static const litenn_hip_attn_ext_opts plain = { 1.0, 0.0, 0.0, nullptr, nullptr, 0, 0, 0 };
+	if (!o)
+	{
+		o = &plain;
+	}
+	if (keys == 0)
+	{
+		return fail(action, "no keys");
+	}
+	if (const int rc = attn_check(action, q, k, v, kv_dtype, m, 0, n_head, n_kv_head, head_dim, out))
+	{
+		return rc < 0 ? 0 : rc;
+	}
+	if (keys > (size_t{ 1 } << 30))
+	{
+		return fail(action, "key length exceeds 2^30 positions");
+	}
+	if (o->max_bias > 0.0 && !o->mask)
+	{
+		// the reference's text (src/LiteNN/Layer/FlashAttnExt.h:163-166)
+		return fail(action, "FlashAttnExt maxBias requires an explicit additive mask");
+	}
+	if (!(o->scale == o->scale) || !(o->logit_softcap == o->logit_softcap) || !(o->max_bias == o->max_bias))
+	{
+		return fail(action, "scale, logit softcap and max bias must be numbers");
+	}
+	if (o->key_position_offset > (size_t{ 1 } << 40) || o->query_position_offset > (size_t{ 1 } << 40))
+	{
+		return fail(action, "position offsets exceed 2^40");
+	}
+	if (o->causal && o->key_position_offset > o->query_position_offset)
+	{
+		// such a row would take its weights from masked scores alone; the lowering never asks for it
+		return fail(action, "the causal mask hides every key from the first query row");
+	}
+	GUARD(action, dev);
+	launch_attn_ext(static_cast<const float*>(q), k, v, kv_dtype, m, keys, n_head, n_kv_head, head_dim, o->scale,
+	                o->max_bias, o->logit_softcap, static_cast<const float*>(o->mask), static_cast<const float*>(o->sinks),
+	                o->causal != 0, o->key_position_offset, o->query_position_offset, static_cast<float*>(out),
+	                stream_of(opts));
+	return finish(action, opts);
 }
 
 extern "C" int litenn_hip_silu_mul(int dev, const void* gate, const void* up, void* y, size_t n,

@@ -727,6 +727,169 @@ namespace litenn_hip
 			}
 		}
 
+		// ---------------- attention with the reference layer's options -----------------------
+		// AddFlashAttnExt with mask, ALiBi slope, logit softcap, sinks and an offset causal mask
+		// (src/LiteNN/Layer/FlashAttnExt.h:17-29,100-228), every head of a call at once.  The
+		// LLaMA lowering uses none of these options, so this kernel is plain: grid (n_head, m), 256
+		// threads, sixteen lanes per key as in the row kernel above, one pass with an online softmax.
+		struct AttnExt
+		{
+			const float* mask;  // additive [m, keys], or null
+			const float* sinks; // [n_head], or null
+			float score_scale;  // scale, or scale / softcap
+			float softcap;      // 0: none
+			int apply_scale;    // the reference emits no multiply by exactly 1 (FlashAttnExt.h:57-67)
+			int apply_cap;      // softcap != 1
+			double max_bias;    // > 0: the mask is multiplied by the head's ALiBi slope
+			int causal;
+			long long key_offset, query_offset;
+			int keys;
+		};
+
+		// Detail::ComputeALiBiSlope (FlashAttnExt.h:69-96), in double like the reference
+		__device__ inline double alibi_slope(int head, int heads, double max_bias)
+		{
+			int head_log2 = 1;
+			while ((head_log2 << 1) <= heads)
+			{
+				head_log2 <<= 1;
+			}
+			const double m0 = pow(2.0, -max_bias / static_cast<double>(head_log2));
+			const double m1 = pow(2.0, -(max_bias / 2.0) / static_cast<double>(head_log2));
+			return head < head_log2 ? pow(m0, static_cast<double>(head + 1))
+			                        : pow(m1, static_cast<double>(2 * (head - head_log2) + 1));
+		}
+
+		template <typename KV>
+		__global__ __launch_bounds__(256) void attn_ext_kernel(const float* __restrict__ q, const KV* __restrict__ kcache,
+		                                                       const KV* __restrict__ vcache, float* __restrict__ out,
+		                                                       int n_head, int n_kv_head, int head_dim, AttnExt x)
+		{
+			using Load = AttnLoad<KV, false>;
+			using LoadF = AttnLoad<float, false>;
+			constexpr int E = Load::E;
+			__shared__ float s_m[16], s_l[16];
+			__shared__ float s_o[16][256 + 4];
+			const int h = blockIdx.x, row = blockIdx.y, tid = threadIdx.x;
+			const int sub = tid & 15, grp = tid >> 4;
+			const int per = (head_dim + 15) >> 4;
+			const int first = sub * per;
+			const int kvh = h / (n_head / n_kv_head);
+			const size_t kvw = static_cast<size_t>(n_kv_head) * head_dim;
+			const KV* kbase = kcache + static_cast<size_t>(kvh) * head_dim;
+			const KV* vbase = vcache + static_cast<size_t>(kvh) * head_dim;
+			float qv[E];
+			LoadF::unpack(LoadF::load(q + (static_cast<size_t>(row) * n_head + h) * head_dim, first, per, head_dim), qv);
+			float slope = 1.0f;
+			bool apply_slope = false;
+			if (x.mask && x.max_bias > 0.0)
+			{
+				const double sl = alibi_slope(h, n_head, x.max_bias);
+				slope = static_cast<float>(sl);
+				apply_slope = sl != 1.0;
+			}
+			// keys the causal mask leaves visible; a masked key's weight is exp(-1e9 - max) = 0 exactly
+			// in the reference, so it is not visited (the host has checked that every row sees one)
+			int len = x.keys;
+			if (x.causal)
+			{
+				const long long visible = x.query_offset + row - x.key_offset + 1;
+				len = static_cast<int>(visible < len ? visible : len);
+			}
+			float run_m = -INFINITY, run_l = 0.0f;
+			float o[E];
+#pragma unroll
+			for (int e = 0; e < E; ++e)
+			{
+				o[e] = 0.0f;
+			}
+			for (int t = grp; t < len; t += 16)
+			{
+				float kf[E], vf[E];
+				Load::unpack(Load::load(kbase + static_cast<size_t>(t) * kvw, first, per, head_dim), kf);
+				Load::unpack(Load::load(vbase + static_cast<size_t>(t) * kvw, first, per, head_dim), vf);
+				float acc = 0.0f;
+#pragma unroll
+				for (int e = 0; e < E; ++e)
+				{
+					acc = fmaf(qv[e], kf[e], acc);
+				}
+				float sc = row16_sum(acc);
+				if (x.apply_scale)
+				{
+					sc = __fmul_rn(sc, x.score_scale);
+				}
+				if (x.softcap != 0.0f)
+				{
+					// AddTanh as the layer lowers it (Activation.h:34-50): (exp(2x) - 1) / (exp(2x) + 1)
+					const float ex = expf(__fmul_rn(sc, 2.0f));
+					sc = __fdiv_rn(__fsub_rn(ex, 1.0f), __fadd_rn(ex, 1.0f));
+					if (x.apply_cap)
+					{
+						sc = __fmul_rn(sc, x.softcap);
+					}
+				}
+				if (x.mask)
+				{
+					float mv = x.mask[static_cast<size_t>(row) * x.keys + t];
+					if (apply_slope)
+					{
+						mv = __fmul_rn(mv, slope);
+					}
+					sc = __fadd_rn(sc, mv);
+				}
+				const float new_m = fmaxf(run_m, sc);
+				const float corr = softmax_weight(run_m, new_m);
+				const float pw = expf(sc - new_m);
+				run_l = fmaf(run_l, corr, pw);
+#pragma unroll
+				for (int e = 0; e < E; ++e)
+				{
+					o[e] = fmaf(pw, vf[e], o[e] * corr);
+				}
+				run_m = new_m;
+			}
+			if (sub == 0)
+			{
+				s_m[grp] = run_m;
+				s_l[grp] = run_l;
+			}
+#pragma unroll
+			for (int e = 0; e < E; ++e)
+			{
+				if (e < per && first + e < head_dim)
+				{
+					s_o[grp][first + e] = o[e];
+				}
+			}
+			__syncthreads();
+			if (tid < head_dim)
+			{
+				float m_all = -INFINITY;
+#pragma unroll
+				for (int g = 0; g < 16; ++g)
+				{
+					m_all = fmaxf(m_all, s_m[g]);
+				}
+				float l_all = 0.0f, o_all = 0.0f;
+				if (x.sinks)
+				{
+					// the sink joins the row maximum and the denominator, not the values (FlashAttnExt.h:184-212)
+					const float sink = x.sinks[h];
+					m_all = fmaxf(m_all, sink);
+					l_all = expf(sink - m_all);
+				}
+#pragma unroll
+				for (int g = 0; g < 16; ++g)
+				{
+					const float w = softmax_weight(s_m[g], m_all);
+					l_all = fmaf(s_l[g], w, l_all);
+					o_all = fmaf(s_o[g][tid], w, o_all);
+				}
+				out[(static_cast<size_t>(row) * n_head + h) * head_dim + tid] = o_all / l_all;
+			}
+		}
+
 		// ---------------- SiLU(gate) * up (Activation.h:22-35,56-63; SwiGLU.h:63-66) ---------
 		__global__ void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
 		                                float* __restrict__ y, size_t n)
@@ -1104,6 +1267,43 @@ namespace litenn_hip
 		const AttnStep step{ k, v, cos_t, sin_t, static_cast<int>(rope_dims) };
 		launch_attn_any(q, kcache, vcache, cache_dtype, 1, past_dev, 0, n_head, n_kv_head, head_dim, out, splits,
 		                partial, counters, &step, s);
+	}
+
+	// Attention of m rows over `keys` cached rows with the reference layer's options; operands as in
+	// launch_attn_decode, mask [m, keys] and sinks [n_head] in f32 on the device or null.
+	void launch_attn_ext(const float* q, const void* kcache, const void* vcache, int cache_dtype, size_t m, size_t keys,
+	                     size_t n_head, size_t n_kv_head, size_t head_dim, double scale, double max_bias,
+	                     double logit_softcap, const float* mask, const float* sinks, bool causal, size_t key_offset,
+	                     size_t query_offset, float* out, hipStream_t s)
+	{
+		AttnExt x;
+		const double score_scale = logit_softcap != 0.0 ? scale / logit_softcap : scale;
+		x.mask = mask;
+		x.sinks = sinks;
+		x.score_scale = static_cast<float>(score_scale);
+		x.softcap = static_cast<float>(logit_softcap);
+		x.apply_scale = (scale != 1.0 || logit_softcap != 0.0) && score_scale != 1.0;
+		x.apply_cap = logit_softcap != 1.0;
+		x.max_bias = max_bias;
+		x.causal = causal;
+		x.key_offset = static_cast<long long>(key_offset);
+		x.query_offset = static_cast<long long>(query_offset);
+		x.keys = static_cast<int>(keys);
+		const dim3 grid(n_head, m), block(256);
+		if (cache_dtype == LITENN_F16)
+		{
+			attn_ext_kernel<uint16_t><<<grid, block, 0, s>>>(q, static_cast<const uint16_t*>(kcache),
+			                                                 static_cast<const uint16_t*>(vcache), out,
+			                                                 static_cast<int>(n_head), static_cast<int>(n_kv_head),
+			                                                 static_cast<int>(head_dim), x);
+		}
+		else
+		{
+			attn_ext_kernel<float><<<grid, block, 0, s>>>(q, static_cast<const float*>(kcache),
+			                                              static_cast<const float*>(vcache), out,
+			                                              static_cast<int>(n_head), static_cast<int>(n_kv_head),
+			                                              static_cast<int>(head_dim), x);
+		}
 	}
 
 	void launch_silu_mul(const float* gate, const float* up, float* y, size_t n, hipStream_t s)

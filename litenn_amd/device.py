@@ -285,6 +285,21 @@ def attn_rows(q: Tensor, kcache: Tensor, vcache: Tensor, m: int, past: int, n_he
     return out
 
 
+def flash_attn_ext(q: Tensor, k: Tensor, v: Tensor, m: int, keys: int, n_head: int, n_kv_head: int, head_dim: int,
+                   scale: float = 1.0, max_bias: float = 0.0, logit_softcap: float = 0.0, mask: Tensor | None = None,
+                   sinks: Tensor | None = None, causal: bool = False, key_position_offset: int = 0,
+                   query_position_offset: int = 0) -> Tensor:
+    """The reference's AddFlashAttnExt with its options, every head at once: q [m, n_head * head_dim],
+    k / v [keys, n_kv_head * head_dim] (Float16 or Float32), mask [m, keys] and sinks [n_head] Float32."""
+    out = Tensor((m, n_head * head_dim), DT_F32, q.device)
+    o = _lib.AttnExtOpts(scale, max_bias, logit_softcap, mask.ptr if mask is not None else None,
+                         sinks.ptr if sinks is not None else None, int(causal), key_position_offset,
+                         query_position_offset)
+    check(_lib.load().litenn_hip_flash_attn_ext(q.device.deviceIndex, q.ptr, k.ptr, v.ptr, k.dtype, m, keys, n_head,
+                                                n_kv_head, head_dim, o, out.ptr, None))
+    return out
+
+
 def silu_mul(gate: Tensor, up: Tensor) -> Tensor:
     y = Tensor(gate.shape, DT_F32, gate.device)
     check(_lib.load().litenn_hip_silu_mul(gate.device.deviceIndex, gate.ptr, up.ptr, y.ptr, gate.size, None))
@@ -300,5 +315,5 @@ def argmax(x: Tensor) -> Tensor:
 
 __all__ = ["HIP", "HIPDeviceCount", "IsHIPDeviceAvailable", "DeviceTraits", "Tensor", "mul_mat_q", "linear_group",
            "dequantize",
-           "get_rows_q", "rmsnorm", "rope_interleaved", "kv_append", "attn_decode", "attn_decode_noalloc", "silu_mul", "argmax",
+           "get_rows_q", "rmsnorm", "rope_interleaved", "kv_append", "attn_decode", "attn_decode_noalloc", "flash_attn_ext", "silu_mul", "argmax",
            "MATMUL_PRECISE", "LiteNNHipError", "F32"]
