@@ -108,6 +108,31 @@ def test_attention_decode(hip, oracle, cache_dtype):
         assert rel_l2(got, want) < 1e-5, (m, past, H, KH, hd)
 
 
+@pytest.mark.parametrize("cache_dtype", [DT_F32, DT_F16])
+def test_attention_with_large_scores(hip, oracle, cache_dtype):
+    """Scores of order 1e3 (a query fifty times unit scale), one key that dominates, keys that all
+    tie, and cache entries near the top of Float16's range: the running maximum keeps every
+    exponent in range, on one row cut into key chunks and on several rows."""
+    rng = np.random.default_rng(41)
+    for m, past, H, KH, hd in [(1, 700, 8, 2, 128), (5, 90, 4, 4, 64), (1, 2000, 4, 1, 128)]:
+        L = past + m
+        q = (rng.standard_normal((m, H * hd)) * 50).astype(np.float32)
+        k = rng.standard_normal((L, KH * hd)).astype(np.float32)
+        v = np.clip(rng.standard_normal((L, KH * hd)) * 2.0e4, -6.5e4, 6.5e4).astype(np.float32)
+        k[L // 3] = q[0, :KH * hd] / 50 * 4       # aligned with the first query heads: dominates their rows
+        k[5:9] = k[5]                               # exact ties
+        if cache_dtype == DT_F16:
+            k = oracle.f16_to_f32(oracle.f32_to_f16_bits(k))
+            v = oracle.f16_to_f32(oracle.f32_to_f16_bits(v))
+            kc, vc = T(hip, k, np.float16), T(hip, v, np.float16)
+        else:
+            kc, vc = T(hip, k), T(hip, v)
+        got = hip.attn_decode(T(hip, q), kc, vc, m, past, H, KH, hd).numpy()
+        want = _attention_want(oracle, q, k, v, past, H, KH, hd)
+        assert np.all(np.isfinite(got))
+        assert rel_l2(got, want) < 1e-5, (m, past, H, KH, hd)
+
+
 def _attention_want(oracle, q, k, v, past, H, KH, hd):
     want = np.empty_like(q)
     for h in range(H):
