@@ -1271,17 +1271,15 @@ namespace litenn_hip
 					}
 				}
 			};
-#pragma unroll
-			for (int t = 0; t < PD; ++t)
-			{
-				if (t < tiles) // uniform
-				{
-					issue_tile(t, t);
-				}
-			}
-
 			// ---- this wavefront's activation fragments: chunks [wave CPW, (wave + 1) CPW), every step,
-			// MT tiles (a tile past the end repeats the last one; its products are not stored)
+			// MT tiles (a tile past the end repeats the last one; its products are not stored), and the
+			// factor that undoes the pre-pass's scaling of this thread's activation row (the same row in
+			// every round: MT divides the number of wavefronts).  They are requested before the first
+			// weight tiles: a wavefront's loads return in order, the fragments come from the L2 the
+			// pre-pass left them in, and behind the tiles they would arrive a memory latency later
+			// than they could.  The loads are issued from assembly like the tiles' so that the wait
+			// below can let the tiles stay in flight; a wait of the compiler's own would cover
+			// everything outstanding.
 			u32x4 b[CPW][8][MT];
 #pragma unroll
 			for (int ci = 0; ci < CPW; ++ci)
@@ -1294,17 +1292,30 @@ namespace litenn_hip
 #pragma unroll
 					for (int st = 0; st < 8; ++st)
 					{
-						b[ci][st][t] = *reinterpret_cast<const u32x4*>(tile + st * kFragBytes);
+						asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(b[ci][st][t]) : "v"(tile + st * kFragBytes) : "memory");
 					}
 				}
 			}
-
-			// the factor that undoes the pre-pass's scaling of this thread's activation row (the same row
-			// in every round: MT divides the number of wavefronts), fetched before the walk
 			const int my_mm = ((threadIdx.x >> 6) % MT) * 16 + (lane & 15);
-			float my_unscale = a.unscale[min(my_mm, 16 * a.m_tiles - 1)];
-			// The compiler's own wait for these loads must sit here, before the walk: inside the loop it
-			// would be repeated on every pass and wait for the tiles requested ahead as well.
+			float my_unscale;
+			asm volatile("global_load_dword %0, %1, off" : "=v"(my_unscale) : "v"(a.unscale + min(my_mm, 16 * a.m_tiles - 1)) : "memory");
+#pragma unroll
+			for (int t = 0; t < PD; ++t)
+			{
+				if (t < tiles) // uniform
+				{
+					issue_tile(t, t);
+				}
+			}
+			// fragments and factor have landed once only the tiles requested after them are outstanding
+			if (tiles >= PD)
+			{
+				vm_wait<PD * kWLoads>();
+			}
+			else
+			{
+				vm_wait<0>();
+			}
 			asm volatile("" : "+v"(my_unscale));
 #pragma unroll
 			for (int ci = 0; ci < CPW; ++ci)
