@@ -309,3 +309,29 @@ def test_generation_across_a_doubling_of_the_cache_length(hip, oracle):
     for a, b in zip(dev.get_kv(1), kv):
         assert np.array_equal(a, b)
     dev.close()
+
+
+@pytest.mark.timeout(300)
+def test_generation_through_every_chunk_count(hip, oracle):
+    """From 30 cached rows to 3700 under one captured step: the single-row attention goes from one key
+    chunk to sixteen on the way.  The device loop must give the checker's tokens and the tokens of
+    evaluation one token at a time, and leave the same cache."""
+    cfg = synth.tiny_llama(Q4_0, block_count=2, d_model=256, heads=4, kv_heads=2, ff=512, vocab=300,
+                           context_length=4096)
+    prompt = synth.prompt_tokens(cfg, 30, 22)
+    n_new = 3670
+    dev, ref = hip_model(hip, cfg, 8, kv_dtype=DT_F32), oracle_model(oracle, cfg, 8, kv_f16=False)
+    got, _, _ = dev.generate(prompt, n_new)
+    assert dev.past == 30 + n_new - 1
+    want, _ = ref.generate(prompt, n_new)
+    first_bad = np.nonzero(got != want)[0]
+    assert first_bad.size == 0, first_bad[:4]
+    kv = dev.get_kv(1)
+    dev.reset()
+    logits = dev.eval(prompt, all_logits=False)
+    for step in range(n_new - 1):
+        assert int(np.argmax(logits)) == int(got[step]), step
+        logits = dev.eval([int(got[step])], all_logits=False)
+    for a, b in zip(dev.get_kv(1), kv):
+        assert np.array_equal(a, b)
+    dev.close()
