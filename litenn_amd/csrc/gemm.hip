@@ -1563,8 +1563,12 @@ namespace litenn_hip
 				{
 					pick = 828;
 				}
-				else if (m_tiles >= 8 && 5 * blocks(8, 128) >= 4 * cus)
+				else if (m_tiles >= 8 && 8 * blocks(8, 128) >= 5 * cus)
 				{
+					// from 5/8 of the CUs on the 128-row tile beats the 64-row one, which decodes every
+					// weight twice as often (gate/up 22016 x 4096 at M = 128, 172 workgroups: 45.4 against
+					// 50.3 us; q/k 5120 x 4096 at M = 512, 160 workgroups: 47.4 against 53.3 us); at half
+					// the CUs it loses (4096 x 4096 at M = 512, 128 workgroups: 45.9 against 38.5 us)
 					pick = 818;
 				}
 				else if (split_ok && c.partial && c.partial_floats >= static_cast<size_t>(c.m) * c.n[0] && m_tiles >= 8 &&
