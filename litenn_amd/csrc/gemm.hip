@@ -1559,7 +1559,10 @@ namespace litenn_hip
 				// cuts K in two when the caller lends a buffer for the second product: each weight is
 				// then decoded four times instead of eight, and one pass adds the two products.
 				const int m_tiles = c.m_tiles;
-				if (m_tiles >= 8 && F::kWideTile && 5 * blocks(8, 256) >= 4 * cus)
+				// (the wide tile, too, from 5/8 of the CUs on: 22016 x 4096 at M = 256, 172 workgroups,
+				// 74.9 against 84.7 us; 12288 x 4096 at M = 512, 192: 78.9 against 86.2; 5120 x 4096 at
+				// M = 1024, 160: 77.7 against 87.9; at half the CUs and below the narrower tiles win)
+				if (m_tiles >= 8 && F::kWideTile && 8 * blocks(8, 256) >= 5 * cus)
 				{
 					pick = 828;
 				}
