@@ -330,6 +330,26 @@ def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=8):
         + " ".join(f"{v:.2f}" for v in by_wave))
     out["gemv_timeline_note"] = ("us after the launch's first wavefront entered the kernel, averaged over 8 launches x "
                                  "2048 wavefronts; earliest / latest are the per-launch extremes, averaged")
+    # The matrix-core GEMM's instruction mix without its memory traffic: cycles per MFMA and SIMD
+    tl.litenn_hip_mb_mix.argtypes = [C.c_int] * 4 + [vp, C.c_int, C.c_int, C.c_int, vp]
+    cyc = ln.Tensor((2 * 4608,))  # 4608 counters of 8 bytes
+    steps, blocks = 2000, 256
+    mix = []
+    for threads in (256, 512):
+        for (mfma, reads, valu) in ((1, 0, 0), (1, 1, 0), (1, 0, 5), (1, 1, 3), (1, 1, 5), (1, 1, 8)):
+            ok(tl.litenn_hip_mb_mix(mfma, reads, valu, 1, cyc.ptr, blocks, threads, steps, stream.handle))
+            stream.synchronize()
+            raw = cyc.numpy().view(np.uint64)[: blocks * 8].reshape(blocks, 8)[:, : threads // 64].astype(np.float64)
+            per_simd = threads // 256                      # wavefronts that share a SIMD
+            per_mfma = float(raw.max(axis=1).mean()) / (steps * 16 * per_simd)
+            mix.append({"wavefronts_per_simd": per_simd, "lds_reads_per_2_mfma": reads, "valu_per_2_mfma": valu,
+                        "cycles_per_mfma_per_simd": round(per_mfma, 2)})
+            log(f"[bench] microbench: mix of 2 MFMA + {reads} ds_read_b128 + {valu} VALU, {per_simd} wavefront(s) per SIMD, "
+                f"barrier every 64 MFMAs: {per_mfma:.1f} cycles per MFMA and SIMD")
+    out["mfma_mix"] = mix
+    out["mfma_mix_note"] = ("v_mfma_f32_16x16x32_f16 from registers, fragment reads from LDS, independent f32 multiply-adds; "
+                            "256 workgroups, shader-clock cycles of the slowest wavefront of a workgroup")
+    cyc.free()
     for w in weights:
         w.free()
     for tns in (x, y, sink):
