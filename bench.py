@@ -36,6 +36,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "gemv_q4_k_14336x4096_hbm_traffic.txt")
+CONFIG_TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "gemv_configs_hbm_traffic.txt")
 
 
 def measured_traffic_bytes():
@@ -49,6 +50,20 @@ def measured_traffic_bytes():
         return int(m.group(1)) if m else None
     except OSError:
         return None
+
+
+def measured_config_traffic():
+    """{(format name, n, k): HBM bytes per launch} of the other single-row configurations, from their
+    committed profiler summary (same method as the headline's); empty when the summary is not there."""
+    import re
+    out = {}
+    try:
+        with open(CONFIG_TRAFFIC_SUMMARY) as f:
+            for m in re.finditer(r"^(Q\w+) GEMV (\d+)x(\d+) traffic per launch:.*= (\d+) bytes", f.read(), re.M):
+                out[(m.group(1), int(m.group(2)), int(m.group(3)))] = int(m.group(4))
+    except OSError:
+        pass
+    return out
 
 
 def log(*a):
@@ -472,6 +487,7 @@ def bench_gemv_configs(ln, hiprt, steps=1600, warmup=64):
     with its own roofline object (rotating buffers of more than 512 MB in total)."""
     from litenn_amd.formats import Q4_0, Q4_K, Q8_0, row_bytes
     out = []
+    traffic = measured_config_traffic()
     for name, fmt, n, k in (("Q8_0", Q8_0, 4096, 4096), ("Q4_0", Q4_0, 11008, 4096), ("Q4_0", Q4_0, 4096, 11008),
                             ("Q4_K", Q4_K, 11008, 4096), ("Q4_K", Q4_K, 4096, 11008)):
         w_bytes = n * row_bytes(fmt, k)
@@ -482,7 +498,7 @@ def bench_gemv_configs(ln, hiprt, steps=1600, warmup=64):
         out.append({"format": name, "n": n, "k": k, "batch": 1, "us": round(ms * 1e3, 3), "buffers": buffers,
                     "algorithmic_bytes": algo,
                     "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                                 "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None}})
+                                 "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": traffic.get((name, n, k))}})
         log(f"[bench] {name} GEMV {n}x{k}: {ms * 1e3:.2f} us/launch, {gbps:.0f} GB/s = "
             f"{100 * gbps / HBM_PEAK_GBPS:.1f}% of HBM peak")
     return out
@@ -499,6 +515,7 @@ def main() -> int:
                          "down a great deal: its runs use 1)")
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="skip the other single-row GEMV configurations")
+    ap.add_argument("--config-steps", type=int, default=1600, help="launches timed per other GEMV configuration")
     ap.add_argument("--decode-prompt", type=int, default=128, help="prompt length of the decode run")
     ap.add_argument("--decode-new", type=int, default=256, help="tokens generated by the decode run")
     ap.add_argument("--decode-model", choices=["7b", "8b", "both"], default="both",
@@ -590,7 +607,7 @@ def main() -> int:
             f"{c['s_with_copy'] * 1e3:.1f} ms with the weight copy, dequantisation once {c['dequant_s'] * 1e3:.0f} ms, "
             f"{c['s_omp'] * 1e3:.1f} ms/call on {c['omp_threads']} threads (not the reference)")
     if not args.no_configs:
-        line["gemv_configs"] = bench_gemv_configs(ln, hiprt)
+        line["gemv_configs"] = bench_gemv_configs(ln, hiprt, steps=args.config_steps)
     if not args.no_gemm:
         line["prefill_gemm"] = bench_prefill_gemm(ln, hiprt, args.gemm_case)
     if not args.no_decode:
