@@ -1140,13 +1140,16 @@ namespace litenn_hip
 			// D layout: lane holds activation row j = lane % 16 and weight rows 4 (lane / 16) + 0..3
 			const bool vec_ok = (n & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 &&
 			                    (!residual || (reinterpret_cast<uintptr_t>(residual) & 15) == 0);
+			// tile by tile, the weight groups of a tile back to back: a lane's 16 bytes, its three
+			// neighbours' and the next group's make one 128-byte line of an output row, and stores that
+			// follow each other closely are combined before they leave the L2
 #pragma unroll
-			for (int q = 0; q < NG; ++q)
+			for (int t = 0; t < MT; ++t)
 			{
-				const int n0 = n_base + 16 * q + 4 * g;
 #pragma unroll
-				for (int t = 0; t < MT; ++t)
+				for (int q = 0; q < NG; ++q)
 				{
+					const int n0 = n_base + 16 * q + 4 * g;
 					const int mm = (mt_base + t) * 16 + r;
 					if (mm < m)
 					{
