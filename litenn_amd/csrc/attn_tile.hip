@@ -70,7 +70,10 @@ namespace litenn_hip
 			const int wave = tid >> 6;
 			const int j = lane & 15; // query (B operand / result column), key or dimension row (A operand)
 			const int g = lane >> 4;
-			const int h = blockIdx.x;
+			// heads are dealt to the XCDs in runs (XCD x: heads [x n_head / 8, (x + 1) n_head / 8)), so that
+			// the query heads of one KV head read its keys and values through one L2
+			const int h = (n_head & 7) == 0 ? static_cast<int>(blockIdx.x & 7) * (n_head >> 3) + static_cast<int>(blockIdx.x >> 3)
+			                                : static_cast<int>(blockIdx.x);
 			const int q_tiles = gridDim.y;
 			const int tile = q_tiles - 1 - static_cast<int>(blockIdx.y); // the longest key runs start first
 			const int past = past_dev ? *past_dev : past_host;

@@ -453,7 +453,13 @@ namespace litenn_hip
 			__shared__ float s_m[16], s_l[16];
 			__shared__ float s_o[16][256 + 4];
 			__shared__ int s_last;
-			const int h = blockIdx.x;
+			// Workgroups go to the eight XCDs (each with its own L2) round-robin in the order of
+			// blockIdx.x: with a head count that is a multiple of 8, XCD x is given the heads
+			// [x n_head / 8, (x + 1) n_head / 8), so that the query heads that share a KV head read
+			// its keys and values through one L2 (8B shape, 32 heads over 8 KV heads: 8.4 MB fetched
+			// per launch for 2.1 MB of cache otherwise).
+			const int h = (n_head & 7) == 0 ? static_cast<int>(blockIdx.x & 7) * (n_head >> 3) + static_cast<int>(blockIdx.x >> 3)
+			                                : static_cast<int>(blockIdx.x);
 			const int split = blockIdx.y;
 			const int row = blockIdx.z;
 			const int tid = threadIdx.x;
