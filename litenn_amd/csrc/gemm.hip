@@ -653,14 +653,23 @@ namespace litenn_hip
 		constexpr int kHeldItems = 8; // 8-element items per thread held in registers: rows up to 16384 wide
 
 		template <typename F>
-		__global__ __launch_bounds__(256) void to_half_kernel(const float* __restrict__ x, uint8_t* __restrict__ xf,
-		                                                       float* __restrict__ unscale, int m, int k,
-		                                                       const float* __restrict__ norm_w, double eps,
-		                                                       const float* __restrict__ up)
+		__device__ __forceinline__ void to_half_body(const float* __restrict__ x, uint8_t* __restrict__ xf,
+		                                             float* __restrict__ unscale, int m, int k,
+		                                             const float* __restrict__ norm_w, double eps,
+		                                             const float* __restrict__ up, float (&red)[4], double (&red64)[4])
 		{
-			__shared__ float red[4];
-			__shared__ double red64[4];
-			const int row = blockIdx.x;
+			// Eight consecutive rows of a tile share every 128-byte line of the fragment layout (16 bytes
+			// each).  Workgroups go to the eight XCDs round-robin in the order of blockIdx.x and the L2s
+			// are not coherent with each other, so with one row per workgroup in that order every line
+			// would be put together in memory from eight partial writes; with a row count that is a
+			// multiple of 64, XCD x takes the row octets x, x + 8, ... instead, eight workgroups that
+			// follow each other on that XCD per octet, and its L2 writes whole lines.
+			int row = blockIdx.x;
+			if ((gridDim.x & 63) == 0)
+			{
+				const int xcd = row & 7, nth = row >> 3;
+				row = (((nth >> 3) << 3) + xcd) * 8 + (nth & 7);
+			}
 
 			const int chunks = k / kChunk;
 			const int mt = row >> 4, r = row & 15;
@@ -804,6 +813,37 @@ namespace litenn_hip
 			}
 		}
 
+		template <typename F>
+		__global__ __launch_bounds__(256) void to_half_kernel(const float* __restrict__ x, uint8_t* __restrict__ xf,
+		                                                       float* __restrict__ unscale, int m, int k,
+		                                                       const float* __restrict__ norm_w, double eps,
+		                                                       const float* __restrict__ up)
+		{
+			__shared__ float red[4];
+			__shared__ double red64[4];
+			to_half_body<F>(x, xf, unscale, m, k, norm_w, eps, up, red, red64);
+		}
+
+		// The same rows in the fragment orders of two formats (matrices of two formats that share their
+		// activations and one GEMM launch): grid y picks the format, each with its own destination.
+		template <typename F0, typename F1>
+		__global__ __launch_bounds__(256) void to_half_pair_kernel(const float* __restrict__ x, uint8_t* __restrict__ xf0,
+		                                                            uint8_t* __restrict__ xf1, float* __restrict__ unscale0,
+		                                                            float* __restrict__ unscale1, int m, int k,
+		                                                            const float* __restrict__ norm_w, double eps)
+		{
+			__shared__ float red[4];
+			__shared__ double red64[4];
+			if (blockIdx.y == 0)
+			{
+				to_half_body<F0>(x, xf0, unscale0, m, k, norm_w, eps, nullptr, red, red64);
+			}
+			else
+			{
+				to_half_body<F1>(x, xf1, unscale1, m, k, norm_w, eps, nullptr, red, red64);
+			}
+		}
+
 		// ---- the GEMM ---------------------------------------------------------------------------
 		// grid (ceil(N / (16 WAVES NG)), ceil(M_tiles / MT)); block 64 WAVES; MT 16-row activation
 		// tiles and NG 16-row weight groups per wavefront.
@@ -858,11 +898,8 @@ namespace litenn_hip
 			float* partial;     // [grid z - 1][M, n[0]]: products of the later K ranges of a split walk (single matrix)
 		};
 
-		template <typename F, int MT, int NG, int WAVES>
-		__global__ __launch_bounds__(64 * WAVES) void gemm_q_kernel(const GemmMats mats, const uint8_t* __restrict__ xf,
-		                                                             const float* __restrict__ unscale,
-		                                                             const float* __restrict__ residual, int k, int m,
-		                                                             int m_tiles, size_t row_bytes)
+		// Workgroup numbering of the tiled GEMM
+		__device__ __forceinline__ void gemm_grid_position(int& grid_x, int& grid_y)
 		{
 			// Workgroups are dispatched in the order x + gridDim.x * y and dealt out to the eight XCDs
 			// (each with its own L2) round-robin.  The workgroups that share a strip of weight rows (one
@@ -871,7 +908,7 @@ namespace litenn_hip
 			// they sit on one XCD too when gridDim.x is a multiple of 8, but a launch of more workgroups
 			// than CUs reaches a strip's later row blocks only in its second round and fetches the strip
 			// again (8B-shape gate/up at 512 rows: 166 MB fetched for 66 MB of weights).
-			int grid_x = blockIdx.x, grid_y = blockIdx.y;
+			grid_x = blockIdx.x, grid_y = blockIdx.y;
 			if (gridDim.y > 1)
 			{
 				const int gx = gridDim.x, gy = gridDim.y;
@@ -889,11 +926,24 @@ namespace litenn_hip
 					grid_y = l2 / rem;
 				}
 			}
-			const int which = (grid_x >= mats.first_block[1]) + (grid_x >= mats.first_block[2]);
-			const uint8_t* __restrict__ w = which == 0 ? mats.w[0] : (which == 1 ? mats.w[1] : mats.w[2]);
-			float* __restrict__ y = which == 0 ? mats.y[0] : (which == 1 ? mats.y[1] : mats.y[2]);
-			const int n = which == 0 ? mats.n[0] : (which == 1 ? mats.n[1] : mats.n[2]);
-			const int block_x = grid_x - (which == 0 ? 0 : (which == 1 ? mats.first_block[1] : mats.first_block[2]));
+		}
+
+		// The matrix strip grid_x of a launch belongs to (selects, so that the argument block stays where it is)
+#define LITENN_GEMM_PICK_MATRIX(mats, grid_x)                                                                         \
+	const int which = ((grid_x) >= (mats).first_block[1]) + ((grid_x) >= (mats).first_block[2]);                       \
+	const uint8_t* w = which == 0 ? (mats).w[0] : (which == 1 ? (mats).w[1] : (mats).w[2]);                            \
+	float* y = which == 0 ? (mats).y[0] : (which == 1 ? (mats).y[1] : (mats).y[2]);                                    \
+	const int n = which == 0 ? (mats).n[0] : (which == 1 ? (mats).n[1] : (mats).n[2]);                                 \
+	const int block_x = (grid_x) - (which == 0 ? 0 : (which == 1 ? (mats).first_block[1] : (mats).first_block[2]))
+
+		// One workgroup's tile: strip block_x of the n-row matrix w against row block grid_y.
+		template <typename F, int MT, int NG, int WAVES>
+		__device__ __forceinline__ void gemm_q_body(const uint8_t* w, float* y, int n, int block_x, float* partial,
+		                                            const uint8_t* __restrict__ xf,
+		                                            const float* __restrict__ unscale,
+		                                            const float* __restrict__ residual, int k, int m, int m_tiles,
+		                                            size_t row_bytes, int grid_y)
+		{
 			constexpr int kHalfBytes = MT * 4 * kFragBytes; // one activation buffer: four steps of MT tiles
 			constexpr int kXLoads = MT * 4 / WAVES;         // 1 KB pieces a wavefront moves per half
 			static_assert(kXLoads >= 1 && kXLoads * WAVES == MT * 4, "activation pieces / wavefront split");
@@ -1178,7 +1228,7 @@ namespace litenn_hip
 					if (mm < m)
 					{
 						// the second K range of a split walk leaves its product beside y (no residual)
-						float* dst = (blockIdx.z == 0 ? y : mats.partial + (blockIdx.z - 1) * (static_cast<size_t>(m) * n)) +
+						float* dst = (blockIdx.z == 0 ? y : partial + (blockIdx.z - 1) * (static_cast<size_t>(m) * n)) +
 						             static_cast<size_t>(mm) * n + n0;
 						const float* res =
 						    residual && blockIdx.z == 0 ? residual + static_cast<size_t>(mm) * n + n0 : nullptr;
@@ -1207,6 +1257,49 @@ namespace litenn_hip
 						}
 					}
 				}
+			}
+		}
+
+		template <typename F, int MT, int NG, int WAVES>
+		__global__ __launch_bounds__(64 * WAVES) void gemm_q_kernel(const GemmMats mats, const uint8_t* __restrict__ xf,
+		                                                             const float* __restrict__ unscale,
+		                                                             const float* __restrict__ residual, int k, int m,
+		                                                             int m_tiles, size_t row_bytes)
+		{
+			int grid_x, grid_y;
+			gemm_grid_position(grid_x, grid_y);
+			LITENN_GEMM_PICK_MATRIX(mats, grid_x);
+			gemm_q_body<F, MT, NG, WAVES>(w, y, n, block_x, mats.partial, xf, unscale, residual, k, m, m_tiles, row_bytes,
+			                              grid_y);
+		}
+
+		// Matrices of two formats that share their activations (q and k in one, v in another): the
+		// strips from `second_block` on belong to the second format, which reads its own copy of the
+		// activations (its decoder's fragment order) and its own row size.  A workgroup runs one of the
+		// two bodies; the branch is uniform.
+		template <typename F0, typename F1, int MT, int NG, int WAVES>
+		__global__ __launch_bounds__(64 * WAVES) void gemm_q_pair_kernel(const GemmMats mats, int second_block,
+		                                                                  const uint8_t* __restrict__ xf0,
+		                                                                  const uint8_t* __restrict__ xf1,
+		                                                                  const float* __restrict__ unscale0,
+		                                                                  const float* __restrict__ unscale1, int k,
+		                                                                  int m, int m_tiles, size_t row_bytes0,
+		                                                                  size_t row_bytes1)
+		{
+			int grid_x, grid_y;
+			gemm_grid_position(grid_x, grid_y);
+			LITENN_GEMM_PICK_MATRIX(mats, grid_x);
+			// (grid z is 1 here and mats.partial unused; a literal null in its place makes this
+			// compiler's inliner fall over)
+			if (grid_x < second_block)
+			{
+				gemm_q_body<F0, MT, NG, WAVES>(w, y, n, block_x, mats.partial, xf0, unscale0, nullptr, k, m, m_tiles, row_bytes0,
+				                               grid_y);
+			}
+			else
+			{
+				gemm_q_body<F1, MT, NG, WAVES>(w, y, n, block_x, mats.partial, xf1, unscale1, nullptr, k, m, m_tiles, row_bytes1,
+				                               grid_y);
 			}
 		}
 
@@ -1525,6 +1618,31 @@ namespace litenn_hip
 			                                                                          c.k, c.m, c.m_tiles, c.row_bytes);
 		}
 
+		// Two formats in one launch: matrices [0, second) in F0, [second, count) in F1, single-group tiles.
+		template <typename F0, typename F1, int MT, int WAVES>
+		void launch_pair_variant(const GemmCall& c, int second, const uint8_t* xf1, const float* unscale1,
+		                         size_t row_bytes1)
+		{
+			constexpr size_t lds = std::max(gemm_lds_bytes<F0, MT, 1, WAVES>(), gemm_lds_bytes<F1, MT, 1, WAVES>());
+			static_assert(lds <= kLdsLimit, "LDS budget");
+			allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_q_pair_kernel<F0, F1, MT, 1, WAVES>), lds);
+			constexpr int bn = 16 * WAVES;
+			GemmMats mats;
+			mats.partial = nullptr;
+			int blocks = 0;
+			for (int i = 0; i < 3; ++i)
+			{
+				mats.w[i] = i < c.count ? c.w[i] : nullptr;
+				mats.y[i] = i < c.count ? c.y[i] : nullptr;
+				mats.n[i] = i < c.count ? c.n[i] : 0;
+				mats.first_block[i] = i < c.count ? blocks : 0x7fffffff;
+				blocks += i < c.count ? (c.n[i] + bn - 1) / bn : 0;
+			}
+			const dim3 grid(blocks, (c.m_tiles + MT - 1) / MT, 1);
+			gemm_q_pair_kernel<F0, F1, MT, 1, WAVES><<<grid, dim3(64 * WAVES), lds, c.stream>>>(
+			    mats, mats.first_block[second], c.xf, xf1, c.unscale, unscale1, c.k, c.m, c.m_tiles, c.row_bytes, row_bytes1);
+		}
+
 		// Tile choice: MT activation tiles per workgroup so that a weight is decoded as few times as
 		// possible; two weight groups per wavefront (each activation fragment read from LDS feeds two
 		// MFMAs) when that still nearly fills the card.
@@ -1784,6 +1902,28 @@ namespace litenn_hip
 				    c.y[0], c.partial, total, c.k_splits - 1);
 			}
 		}
+		template <typename F0, typename F1>
+		void launch_pair(GemmCall& c, int second, const float* x, const float* norm_w, double eps, uint8_t* xf0,
+		                 uint8_t* xf1, float* unscale0, float* unscale1, size_t row_bytes1, int m_pad, int cus)
+		{
+			choose_tile<F1>(c, cus); // (F1 has no wide tile, and without a partial buffer K is not split)
+			to_half_pair_kernel<F0, F1><<<dim3(static_cast<unsigned>(m_pad), 2), dim3(256), 0, c.stream>>>(
+			    x, xf0, xf1, unscale0, unscale1, c.m, c.k, norm_w, eps);
+			switch (c.tile)
+			{
+			case 828: case 818: launch_pair_variant<F0, F1, 8, 8>(c, second, xf1, unscale1, row_bytes1); break;
+			case 414: launch_pair_variant<F0, F1, 4, 4>(c, second, xf1, unscale1, row_bytes1); break;
+			case 214: launch_pair_variant<F0, F1, 2, 4>(c, second, xf1, unscale1, row_bytes1); break;
+			default: launch_pair_variant<F0, F1, 1, 4>(c, second, xf1, unscale1, row_bytes1); break;
+			}
+		}
+
+		// alignment the tiled kernel needs of a format's rows: Q6_K (210-byte) and Q3_K (110-byte) blocks
+		// are fetched from the 16-byte boundary below them; the other formats' chunks must start on one
+		uintptr_t weight_alignment(int fmt)
+		{
+			return fmt == LITENN_FMT_Q6_K || fmt == LITENN_FMT_Q3_K ? 2 : (fmt == LITENN_FMT_Q2_K ? 4 : 16);
+		}
 	} // namespace
 
 	// halves of scratch launch_gemm needs for an m-row batch of width k
@@ -1820,9 +1960,7 @@ namespace litenn_hip
 		{
 			return false;
 		}
-		// Q6_K blocks (210 bytes) are fetched from the 16-byte boundary below them; the other formats'
-		// chunks must start on one
-		const uintptr_t w_align = fmt == LITENN_FMT_Q6_K || fmt == LITENN_FMT_Q3_K ? 2 : (fmt == LITENN_FMT_Q2_K ? 4 : 16);
+		const uintptr_t w_align = weight_alignment(fmt);
 		for (int i = 0; i < count; ++i)
 		{
 			if (reinterpret_cast<uintptr_t>(wq[i]) % w_align != 0 || n[i] == 0 || n[i] > 0x7fffffffu)
@@ -1881,6 +2019,103 @@ namespace litenn_hip
 		case LITENN_FMT_Q4_K: launch_prepass_and_gemm<Q4_KFrag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
 		case LITENN_FMT_Q5_K: launch_prepass_and_gemm<Q5_KFrag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
 		default: launch_prepass_and_gemm<Q6_KFrag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
+		}
+		return true;
+	}
+
+	// Two or three matrices in two formats that share the activations (q and k in Q4_K or Q5_K beside
+	// a Q6_K v): y_i[M, n_i] = X'[M, K] . deq(W_i)^T with X' = x or RMSNorm(x) * norm_w, one pre-pass
+	// launch (the rows in both decoders' fragment orders) and one GEMM launch.  The formats must be a
+	// run of the first followed by a run of the second.  scratch_halves holds `scratch_capacity`
+	// halves and must have room for two batches (2 * gemm_scratch_halves(m, k)).  Returns false,
+	// launching nothing, for anything else; the caller then goes format by format.
+	bool launch_gemm_group_mixed(const int* fmts, int count, const void* const* wq, const size_t* n, size_t k,
+	                             const float* x, size_t m, float* const* y, const float* norm_w, double eps,
+	                             void* scratch_halves, size_t scratch_capacity, hipStream_t stream)
+	{
+		if (count < 2 || count > 3)
+		{
+			return false;
+		}
+		int second = 1;
+		while (second < count && fmts[second] == fmts[0])
+		{
+			++second;
+		}
+		if (second == count)
+		{
+			return false;
+		}
+		for (int i = second; i < count; ++i)
+		{
+			if (fmts[i] != fmts[second])
+			{
+				return false;
+			}
+		}
+		const int f0 = fmts[0], f1 = fmts[second];
+		if ((f0 != LITENN_FMT_Q4_K && f0 != LITENN_FMT_Q5_K) || f1 != LITENN_FMT_Q6_K)
+		{
+			return false;
+		}
+		const size_t rb0 = row_bytes(f0, k), rb1 = row_bytes(f1, k);
+		for (int i = 0; i < count; ++i)
+		{
+			const uintptr_t align = weight_alignment(i < second ? f0 : f1);
+			if (reinterpret_cast<uintptr_t>(wq[i]) % align != 0 || n[i] == 0 || n[i] > 0x7fffffffu)
+			{
+				return false;
+			}
+		}
+		const size_t m_pad = (m + 15) / 16 * 16;
+		const size_t one = gemm_scratch_halves(m, k);
+		if (k % kChunk != 0 || rb0 == 0 || rb1 == 0 || rb0 % weight_alignment(f0) != 0 || rb1 % weight_alignment(f1) != 0 ||
+		    reinterpret_cast<uintptr_t>(x) % 16 != 0 || !scratch_halves ||
+		    reinterpret_cast<uintptr_t>(scratch_halves) % 16 != 0 || (one & 7) != 0 || 2 * one > scratch_capacity ||
+		    2 * m_pad * k >= (size_t{ 1 } << 32) || k > static_cast<size_t>(kHeldItems) * 256 * 8 ||
+		    (norm_w && reinterpret_cast<uintptr_t>(norm_w) % 16 != 0))
+		{
+			return false;
+		}
+		static const int cus = [] {
+			int dev = 0;
+			hipDeviceProp_t prop;
+			if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+			{
+				return 256;
+			}
+			return prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+		}();
+		uint8_t* xf0 = static_cast<uint8_t*>(scratch_halves);
+		float* unscale0 = reinterpret_cast<float*>(xf0 + 2 * m_pad * k);
+		uint8_t* xf1 = xf0 + 2 * one;
+		float* unscale1 = reinterpret_cast<float*>(xf1 + 2 * m_pad * k);
+		GemmCall c{};
+		c.count = count;
+		for (int i = 0; i < count; ++i)
+		{
+			c.w[i] = static_cast<const uint8_t*>(wq[i]);
+			c.y[i] = y[i];
+			c.n[i] = static_cast<int>(n[i]);
+		}
+		c.xf = xf0;
+		c.unscale = unscale0;
+		c.residual = nullptr;
+		c.k = static_cast<int>(k);
+		c.m = static_cast<int>(m);
+		c.m_tiles = static_cast<int>(m_pad / 16);
+		c.row_bytes = rb0;
+		c.partial = nullptr;
+		c.partial_floats = 0;
+		c.stream = stream;
+		const int mp = static_cast<int>(m_pad);
+		if (f0 == LITENN_FMT_Q4_K)
+		{
+			launch_pair<Q4_KFrag, Q6_KFrag>(c, second, x, norm_w, eps, xf0, xf1, unscale0, unscale1, rb1, mp, cus);
+		}
+		else
+		{
+			launch_pair<Q5_KFrag, Q6_KFrag>(c, second, x, norm_w, eps, xf0, xf1, unscale0, unscale1, rb1, mp, cus);
 		}
 		return true;
 	}

@@ -24,6 +24,9 @@ namespace litenn_hip
 	                       size_t m, float* const* y, const float* residual, const float* norm_w, double eps,
 	                       const float* up, void* scratch_halves, float* partial, size_t partial_floats,
 	                       hipStream_t stream);
+	bool launch_gemm_group_mixed(const int* fmts, int count, const void* const* wq, const size_t* n, size_t k,
+	                             const float* x, size_t m, float* const* y, const float* norm_w, double eps,
+	                             void* scratch_halves, size_t scratch_capacity, hipStream_t stream);
 	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
 	                 const float* residual, void* scratch_halves, float* partial, size_t partial_floats,
 	                 hipStream_t stream);
@@ -104,6 +107,7 @@ struct litenn_hip_llama
 	float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *gate = nullptr,
 	      *gate2 = nullptr, *up = nullptr, *logits = nullptr;
 	void* xh = nullptr; // fp16 copy of a matmul's activations (multi-row path), 16-row padded
+	size_t xh_halves = 0; // its size: room for the widest matmul, and for two copies of the embedding width
 	void* argmax_scratch = nullptr; // per-chunk (value, index) pairs of the vocabulary arg-max
 	std::vector<void*> owned; // device buffers freed with the model (tensors uploaded by the GGUF loader)
 	int32_t* d_tokens = nullptr;
@@ -181,7 +185,9 @@ namespace
 				LITENN_HIP_TRY(kAction, hipMalloc(reinterpret_cast<void**>(b.p), sizeof(float) * rows * b.n));
 			}
 			LITENN_HIP_TRY(kAction, hipMalloc(reinterpret_cast<void**>(&m->d_tokens), sizeof(int32_t) * rows));
-			LITENN_HIP_TRY(kAction, hipMalloc(&m->xh, 2 * gemm_scratch_halves(rows, std::max({ d, qw, ff }))));
+			// (q/k/v projections in two formats share a launch that wants the rows in both fragment orders)
+			m->xh_halves = std::max(gemm_scratch_halves(rows, std::max({ d, qw, ff })), 2 * gemm_scratch_halves(rows, d));
+			LITENN_HIP_TRY(kAction, hipMalloc(&m->xh, 2 * m->xh_halves));
 			m->cap_rows = rows;
 		}
 		if (logit_rows > m->cap_logit_rows)
@@ -393,8 +399,17 @@ namespace
 		{
 			const Weight* qkv[3] = { &L.wq, &L.wk, &L.wv };
 			float* qkv_out[3] = { m->q, m->k, m->v };
-			// consecutive projections of one format share a launch (and its fused norm)
-			for (int i = 0; i < 3;)
+			// consecutive projections of one format share a launch (and its fused norm), and so do q and
+			// k in Q4_K or Q5_K beside a Q6_K v
+			const int qkv_fmt[3] = { L.wq.fmt, L.wk.fmt, L.wv.fmt };
+			const void* qkv_w[3] = { L.wq.data, L.wk.data, L.wv.data };
+			const size_t qkv_n[3] = { L.wq.n, L.wk.n, L.wv.n };
+			const bool mixed = L.wq.fmt != L.wk.fmt || L.wk.fmt != L.wv.fmt;
+			const bool one_launch = mixed && rows >= kGemmMinRows && !(flags & LITENN_HIP_MATMUL_PRECISE) &&
+			                        L.wq.k == L.wk.k && L.wk.k == L.wv.k &&
+			                        launch_gemm_group_mixed(qkv_fmt, 3, qkv_w, qkv_n, L.wq.k, m->x, rows, qkv_out, L.attn_norm,
+			                                                m->p.rms_norm_epsilon, m->xh, m->xh_halves, s);
+			for (int i = 0; i < 3 && !one_launch;)
 			{
 				int j = i + 1;
 				while (j < 3 && qkv[j]->fmt == qkv[i]->fmt && qkv[j]->k == qkv[i]->k)

@@ -121,6 +121,28 @@ def test_single_token_steps_with_a_q6_k_value_projection(hip, oracle, main_fmt, 
     assert got.tolist() == ref.generate(toks[:4], 12)[0].tolist()
 
 
+@pytest.mark.parametrize("main_fmt,d_model,rows", [(Q4_K, 512, 5), (Q5_K, 512, 40), (Q5_K, 1024, 352), (Q4_K, 1024, 704)])
+def test_prompt_pass_with_a_q6_k_value_projection(hip, oracle, main_fmt, d_model, rows):
+    """A prompt's q and k (Q4_K / Q5_K) and v (Q6_K) projections share one matrix-core launch, each
+    format's workgroups reading the rows in their decoder's fragment order.  The row counts reach
+    the launch's tiles of 16, 32 and 64 rows (the 128-row tile is reached by the 8B shape in
+    tests/test_gpu_config5.py).  The Float32 cache holds the k and v projections as the launch left
+    them (k after its rotation): they and the logits against the checker."""
+    cfg = synth.tiny_llama(main_fmt, block_count=1, d_model=d_model, heads=d_model // 128 * 2, kv_heads=2, ff=512,
+                           vocab=333, context_length=rows + 4,
+                           formats={"default": main_fmt, "attn_v": Q6_K, "ffn_down": Q6_K, "output": Q6_K})
+    toks = synth.prompt_tokens(cfg, rows, 12)
+    dev, ref = hip_model(hip, cfg, 6, kv_dtype=DT_F32), oracle_model(oracle, cfg, 6, kv_f16=False)
+    got, want = dev.eval(toks, all_logits=False), ref.eval(toks, all_logits=False)
+    for got_c, want_c in zip(dev.get_kv(0), ref.get_kv(0)):
+        assert got_c.shape == want_c.shape and rel_l2(got_c, want_c) < 1e-3
+    assert rel_l2(got, want) < 3e-3
+    # and the same rows through the Float32 path
+    dev.reset()
+    assert rel_l2(dev.eval(toks, all_logits=False, precise=True), want) < 1e-4
+    dev.close()
+
+
 def test_error_paths(hip):
     cfg = synth.tiny_llama(Q4_0, context_length=8)
     m = hip_model(hip, cfg, 1)
