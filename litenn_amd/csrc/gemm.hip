@@ -937,9 +937,12 @@ namespace litenn_hip
 	const int block_x = (grid_x) - (which == 0 ? 0 : (which == 1 ? (mats).first_block[1] : (mats).first_block[2]))
 
 		// One workgroup's tile: strip block_x of the n-row matrix w against row block grid_y.
-		template <typename F, int MT, int NG, int WAVES>
-		__device__ __forceinline__ void gemm_q_body(const uint8_t* w, float* y, int n, int block_x, float* partial,
-		                                            const uint8_t* __restrict__ xf,
+		// GATED (two weight groups per wavefront): the second group holds the same rows of a second
+		// matrix w_up, and what is stored is silu(x . w^T) * (x . w_up^T), SwiGLU's product with its
+		// separately rounded steps (Activation.h:22-35,56-63; SwiGLU.h:63-66), to the single output y.
+		template <typename F, int MT, int NG, int WAVES, bool GATED = false>
+		__device__ __forceinline__ void gemm_q_body(const uint8_t* w, const uint8_t* w_up, float* y, int n, int block_x,
+		                                            float* partial, const uint8_t* __restrict__ xf,
 		                                            const float* __restrict__ unscale,
 		                                            const float* __restrict__ residual, int k, int m, int m_tiles,
 		                                            size_t row_bytes, int grid_y)
@@ -955,7 +958,8 @@ namespace litenn_hip
 			const int lane = threadIdx.x & 63;
 			const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 			const int r = lane & 15, g = lane >> 4;
-			const int n_base = (block_x * WAVES + wave) * 16 * NG;
+			static_assert(!GATED || NG == 2, "the gated form pairs the two weight groups of a wavefront");
+			const int n_base = (block_x * WAVES + wave) * 16 * (GATED ? 1 : NG);
 			const int mt_base = grid_y * MT;
 			const int chunks = k / kChunk;
 			// grid z splits the K walk: this workgroup multiplies chunks [c_begin, c_end)
@@ -1006,7 +1010,9 @@ namespace litenn_hip
 				const fetch::GemmWeightRequest rq = fetch::gemm_weight_request(i, lane, NG, P);
 				w_piece[i] = rq.offset;
 				w_issued[i] = rq.issued;
-				w_src[i] = w + static_cast<size_t>(fetch::gemm_weight_row(n_base, rq.row, n)) * row_bytes;
+				// (gated: slot rows 16 .. 31 are rows 0 .. 15 of the second matrix)
+				w_src[i] = (GATED && rq.row >= 16 ? w_up : w) +
+				           static_cast<size_t>(fetch::gemm_weight_row(n_base, GATED ? (rq.row & 15) : rq.row, n)) * row_bytes;
 			}
 			const auto issue_w = [&](int c) {
 #pragma unroll
@@ -1035,7 +1041,8 @@ namespace litenn_hip
 #pragma unroll
 			for (int q = 0; q < NG; ++q)
 			{
-				lane_rows[q] = w + static_cast<size_t>(fetch::gemm_weight_row(n_base, 16 * q + r, n)) * row_bytes;
+				lane_rows[q] = (GATED && q == 1 ? w_up : w) +
+				               static_cast<size_t>(fetch::gemm_weight_row(n_base, GATED ? r : 16 * q + r, n)) * row_bytes;
 			}
 
 			floatx4 acc[NG][MT];
@@ -1217,6 +1224,45 @@ namespace litenn_hip
 			// tile by tile, the weight groups of a tile back to back: a lane's 16 bytes, its three
 			// neighbours' and the next group's make one 128-byte line of an output row, and stores that
 			// follow each other closely are combined before they leave the L2
+			if constexpr (GATED)
+			{
+#pragma unroll
+				for (int t = 0; t < MT; ++t)
+				{
+					const int n0 = n_base + 4 * g;
+					const int mm = (mt_base + t) * 16 + r;
+					if (mm < m)
+					{
+						float* dst = y + static_cast<size_t>(mm) * n + n0;
+						const float us = unscale[mm];
+						const float gate[4] = { acc[0][t].x * us, acc[0][t].y * us, acc[0][t].z * us, acc[0][t].w * us };
+						const float upv[4] = { acc[1][t].x * us, acc[1][t].y * us, acc[1][t].z * us, acc[1][t].w * us };
+						float vals[4];
+#pragma unroll
+						for (int e = 0; e < 4; ++e)
+						{
+							const float sig = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf(-gate[e])));
+							vals[e] = __fmul_rn(__fmul_rn(gate[e], sig), upv[e]);
+						}
+						if (vec_ok && n0 + 3 < n)
+						{
+							*reinterpret_cast<float4*>(dst) = float4{ vals[0], vals[1], vals[2], vals[3] };
+						}
+						else
+						{
+#pragma unroll
+							for (int e = 0; e < 4; ++e)
+							{
+								if (n0 + e < n)
+								{
+									dst[e] = vals[e];
+								}
+							}
+						}
+					}
+				}
+				return;
+			}
 #pragma unroll
 			for (int t = 0; t < MT; ++t)
 			{
@@ -1269,8 +1315,22 @@ namespace litenn_hip
 			int grid_x, grid_y;
 			gemm_grid_position(grid_x, grid_y);
 			LITENN_GEMM_PICK_MATRIX(mats, grid_x);
-			gemm_q_body<F, MT, NG, WAVES>(w, y, n, block_x, mats.partial, xf, unscale, residual, k, m, m_tiles, row_bytes,
-			                              grid_y);
+			gemm_q_body<F, MT, NG, WAVES>(w, nullptr, y, n, block_x, mats.partial, xf, unscale, residual, k, m, m_tiles,
+			                              row_bytes, grid_y);
+		}
+
+		// gate (mats.w[0]) and up (mats.w[1]) projections of n[0] rows each with SwiGLU's product in the
+		// epilogue: y[0][M, n[0]] = silu(x . gate^T) * (x . up^T); strips along grid x are strips of both
+		template <typename F, int MT, int WAVES>
+		__global__ __launch_bounds__(64 * WAVES) void gemm_q_gated_kernel(const GemmMats mats,
+		                                                                   const uint8_t* __restrict__ xf,
+		                                                                   const float* __restrict__ unscale, int k, int m,
+		                                                                   int m_tiles, size_t row_bytes)
+		{
+			int grid_x, grid_y;
+			gemm_grid_position(grid_x, grid_y);
+			gemm_q_body<F, MT, 2, WAVES, true>(mats.w[0], mats.w[1], mats.y[0], mats.n[0], grid_x, mats.partial, xf, unscale,
+			                                   nullptr, k, m, m_tiles, row_bytes, grid_y);
 		}
 
 		// Matrices of two formats that share their activations (q and k in one, v in another): the
@@ -1293,12 +1353,12 @@ namespace litenn_hip
 			// compiler's inliner fall over)
 			if (grid_x < second_block)
 			{
-				gemm_q_body<F0, MT, NG, WAVES>(w, y, n, block_x, mats.partial, xf0, unscale0, nullptr, k, m, m_tiles, row_bytes0,
+				gemm_q_body<F0, MT, NG, WAVES>(w, nullptr, y, n, block_x, mats.partial, xf0, unscale0, nullptr, k, m, m_tiles, row_bytes0,
 				                               grid_y);
 			}
 			else
 			{
-				gemm_q_body<F1, MT, NG, WAVES>(w, y, n, block_x, mats.partial, xf1, unscale1, nullptr, k, m, m_tiles, row_bytes1,
+				gemm_q_body<F1, MT, NG, WAVES>(w, nullptr, y, n, block_x, mats.partial, xf1, unscale1, nullptr, k, m, m_tiles, row_bytes1,
 				                               grid_y);
 			}
 		}
@@ -1902,6 +1962,39 @@ namespace litenn_hip
 				    c.y[0], c.partial, total, c.k_splits - 1);
 			}
 		}
+		// gate and up projections with SwiGLU's product in the epilogue; only where the two-group tile
+		// is the one the two matrices would get anyway (the format has it and it nearly fills the card)
+		template <typename F>
+		bool launch_gated(GemmCall& c, const float* x, const float* norm_w, double eps, uint8_t* xf, float* unscale,
+		                  int m_pad, int cus)
+		{
+			if constexpr (!F::kWideTile || gemm_lds_bytes<F, 8, 2, 8>() > kLdsLimit)
+			{
+				return false;
+			}
+			else
+			{
+				choose_tile<F>(c, cus);
+				if (c.tile != 828 || c.k_splits != 1)
+				{
+					return false;
+				}
+				to_half_kernel<F><<<dim3(static_cast<unsigned>(m_pad)), dim3(256), 0, c.stream>>>(x, xf, unscale, c.m, c.k,
+				                                                                                 norm_w, eps, nullptr);
+				constexpr size_t lds = gemm_lds_bytes<F, 8, 2, 8>();
+				allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_q_gated_kernel<F, 8, 8>), lds);
+				GemmMats mats{};
+				mats.w[0] = c.w[0];
+				mats.w[1] = c.w[1];
+				mats.y[0] = c.y[0];
+				mats.n[0] = c.n[0];
+				const dim3 grid((c.n[0] + 127) / 128, (c.m_tiles + 7) / 8, 1);
+				gemm_q_gated_kernel<F, 8, 8><<<grid, dim3(512), lds, c.stream>>>(mats, c.xf, c.unscale, c.k, c.m, c.m_tiles,
+				                                                                c.row_bytes);
+				return true;
+			}
+		}
+
 		template <typename F0, typename F1>
 		void launch_pair(GemmCall& c, int second, const float* x, const float* norm_w, double eps, uint8_t* xf0,
 		                 uint8_t* xf1, float* unscale0, float* unscale1, size_t row_bytes1, int m_pad, int cus)
@@ -1915,6 +2008,32 @@ namespace litenn_hip
 			case 414: launch_pair_variant<F0, F1, 4, 4>(c, second, xf1, unscale1, row_bytes1); break;
 			case 214: launch_pair_variant<F0, F1, 2, 4>(c, second, xf1, unscale1, row_bytes1); break;
 			default: launch_pair_variant<F0, F1, 1, 4>(c, second, xf1, unscale1, row_bytes1); break;
+			}
+		}
+
+		int compute_unit_count()
+		{
+			static const int cus = [] {
+				int dev = 0;
+				hipDeviceProp_t prop;
+				if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+				{
+					return 256;
+				}
+				return prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+			}();
+			return cus;
+		}
+
+		bool is_gemm_format(int fmt)
+		{
+			switch (fmt)
+			{
+			case LITENN_FMT_Q4_0: case LITENN_FMT_Q4_1: case LITENN_FMT_Q5_0: case LITENN_FMT_Q5_1: case LITENN_FMT_Q8_0:
+			case LITENN_FMT_Q2_K: case LITENN_FMT_Q3_K: case LITENN_FMT_Q4_K: case LITENN_FMT_Q5_K: case LITENN_FMT_Q6_K:
+				return true;
+			default:
+				return false;
 			}
 		}
 
@@ -1948,12 +2067,8 @@ namespace litenn_hip
 	                       hipStream_t stream)
 	{
 		const size_t rb = row_bytes(fmt, k);
-		switch (fmt)
+		if (!is_gemm_format(fmt))
 		{
-		case LITENN_FMT_Q4_0: case LITENN_FMT_Q4_1: case LITENN_FMT_Q5_0: case LITENN_FMT_Q5_1: case LITENN_FMT_Q8_0:
-		case LITENN_FMT_Q2_K: case LITENN_FMT_Q3_K: case LITENN_FMT_Q4_K: case LITENN_FMT_Q5_K: case LITENN_FMT_Q6_K:
-			break;
-		default:
 			return false;
 		}
 		if (count < 1 || count > 3 || (count > 1 && residual) || (norm_w && up))
@@ -1976,15 +2091,7 @@ namespace litenn_hip
 		{
 			return false;
 		}
-		static const int cus = [] {
-			int dev = 0;
-			hipDeviceProp_t prop;
-			if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
-			{
-				return 256;
-			}
-			return prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-		}();
+		const int cus = compute_unit_count();
 		const size_t m_pad = (m + 15) / 16 * 16;
 		uint8_t* xf = static_cast<uint8_t*>(scratch_halves);
 		float* unscale = reinterpret_cast<float*>(xf + 2 * m_pad * k); // after the fp16 tiles
@@ -2021,6 +2128,58 @@ namespace litenn_hip
 		default: launch_prepass_and_gemm<Q6_KFrag>(c, x, norm_w, eps, up, xf, unscale, mp, cus); break;
 		}
 		return true;
+	}
+
+	// h[M, n] = silu(X' . deq(W_gate)^T) * (X' . deq(W_up)^T) with X' = x or RMSNorm(x) * norm_w: the gate and up
+	// projections of a feed-forward block with SwiGLU's product (SwiGLU.h:63-66) in the launch's
+	// epilogue, so that neither projection is written out.  Takes the shapes whose two matrices would
+	// run on the 128 x 256 tile; returns false, launching nothing, for anything else (the caller then
+	// multiplies the two and lets the next pre-pass form the product).
+	bool launch_gemm_gated(int fmt, const void* w_gate, const void* w_up, size_t n, size_t k, const float* x, size_t m,
+	                       float* h, const float* norm_w, double eps, void* scratch_halves, hipStream_t stream)
+	{
+		const size_t rb = row_bytes(fmt, k);
+		const uintptr_t w_align = weight_alignment(fmt);
+		if (!is_gemm_format(fmt) || reinterpret_cast<uintptr_t>(w_gate) % w_align != 0 ||
+		    reinterpret_cast<uintptr_t>(w_up) % w_align != 0 || n == 0 || n > 0x3fffffffu || k % kChunk != 0 || rb == 0 ||
+		    rb % w_align != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0 || !scratch_halves ||
+		    reinterpret_cast<uintptr_t>(scratch_halves) % 16 != 0 || 2 * ((m + 15) / 16 * 16) * k >= (size_t{ 1 } << 32) ||
+		    k > static_cast<size_t>(kHeldItems) * 256 * 8 || (norm_w && reinterpret_cast<uintptr_t>(norm_w) % 16 != 0))
+		{
+			return false;
+		}
+		const int cus = compute_unit_count();
+		const size_t m_pad = (m + 15) / 16 * 16;
+		uint8_t* xf = static_cast<uint8_t*>(scratch_halves);
+		float* unscale = reinterpret_cast<float*>(xf + 2 * m_pad * k);
+		GemmCall c{};
+		c.count = 2;
+		c.w[0] = static_cast<const uint8_t*>(w_gate);
+		c.w[1] = static_cast<const uint8_t*>(w_up);
+		c.y[0] = h;
+		c.y[1] = nullptr;
+		c.n[0] = c.n[1] = static_cast<int>(n);
+		c.xf = xf;
+		c.unscale = unscale;
+		c.k = static_cast<int>(k);
+		c.m = static_cast<int>(m);
+		c.m_tiles = static_cast<int>(m_pad / 16);
+		c.row_bytes = rb;
+		c.stream = stream;
+		const int mp = static_cast<int>(m_pad);
+		switch (fmt)
+		{
+		case LITENN_FMT_Q4_0: return launch_gated<Q4_0Frag>(c, x, norm_w, eps, xf, unscale, mp, cus);
+		case LITENN_FMT_Q4_1: return launch_gated<Q4_1Frag>(c, x, norm_w, eps, xf, unscale, mp, cus);
+		case LITENN_FMT_Q5_0: return launch_gated<Q5_0Frag>(c, x, norm_w, eps, xf, unscale, mp, cus);
+		case LITENN_FMT_Q5_1: return launch_gated<Q5_1Frag>(c, x, norm_w, eps, xf, unscale, mp, cus);
+		case LITENN_FMT_Q2_K: return launch_gated<Q2_KFrag>(c, x, norm_w, eps, xf, unscale, mp, cus);
+		case LITENN_FMT_Q3_K: return launch_gated<Q3_KFrag>(c, x, norm_w, eps, xf, unscale, mp, cus);
+		case LITENN_FMT_Q8_0: return launch_gated<Q8_0Frag>(c, x, norm_w, eps, xf, unscale, mp, cus);
+		case LITENN_FMT_Q4_K: return launch_gated<Q4_KFrag>(c, x, norm_w, eps, xf, unscale, mp, cus);
+		case LITENN_FMT_Q5_K: return launch_gated<Q5_KFrag>(c, x, norm_w, eps, xf, unscale, mp, cus);
+		default: return launch_gated<Q6_KFrag>(c, x, norm_w, eps, xf, unscale, mp, cus);
+		}
 	}
 
 	// Two or three matrices in two formats that share the activations (q and k in Q4_K or Q5_K beside
@@ -2077,15 +2236,7 @@ namespace litenn_hip
 		{
 			return false;
 		}
-		static const int cus = [] {
-			int dev = 0;
-			hipDeviceProp_t prop;
-			if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
-			{
-				return 256;
-			}
-			return prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-		}();
+		const int cus = compute_unit_count();
 		uint8_t* xf0 = static_cast<uint8_t*>(scratch_halves);
 		float* unscale0 = reinterpret_cast<float*>(xf0 + 2 * m_pad * k);
 		uint8_t* xf1 = xf0 + 2 * one;

@@ -24,6 +24,8 @@ namespace litenn_hip
 	                       size_t m, float* const* y, const float* residual, const float* norm_w, double eps,
 	                       const float* up, void* scratch_halves, float* partial, size_t partial_floats,
 	                       hipStream_t stream);
+	bool launch_gemm_gated(int fmt, const void* w_gate, const void* w_up, size_t n, size_t k, const float* x, size_t m,
+	                       float* h, const float* norm_w, double eps, void* scratch_halves, hipStream_t stream);
 	bool launch_gemm_group_mixed(const int* fmts, int count, const void* const* wq, const size_t* n, size_t k,
 	                             const float* x, size_t m, float* const* y, const float* norm_w, double eps,
 	                             void* scratch_halves, size_t scratch_capacity, hipStream_t stream);
@@ -432,11 +434,21 @@ namespace
 			matmul(m, L.wo, m->attn, rows, m->x, m->x, flags, s); // x = x + attn . Wo
 			const Weight* gu[2] = { &L.gate, &L.up };
 			float* gu_out[2] = { m->gate, m->up };
-			matmul_group(m, 2, gu, gu_out, m->x, rows, nullptr, L.ffn_norm, nullptr, m->xn, nullptr, flags, s);
+			// gate = silu(x' . Wg) * (x' . Wu) straight from the launch's epilogue where the shape allows,
+			// else the two projections, whose product the down projection's pre-pass then forms
+			const bool gated = rows >= kGemmMinRows && !(flags & LITENN_HIP_MATMUL_PRECISE) && L.gate.fmt == L.up.fmt &&
+			                   L.gate.k == L.up.k && L.gate.n == L.up.n &&
+			                   launch_gemm_gated(L.gate.fmt, L.gate.data, L.up.data, L.gate.n, L.gate.k, m->x, rows, m->gate,
+			                                     L.ffn_norm, m->p.rms_norm_epsilon, m->xh, s);
+			if (!gated)
+			{
+				matmul_group(m, 2, gu, gu_out, m->x, rows, nullptr, L.ffn_norm, nullptr, m->xn, nullptr, flags, s);
+			}
 			const Weight* wd[1] = { &L.down };
 			float* xo[1] = { m->x };
 			// xn is idle here: the GEMM may leave the product of K's second half there
-			matmul_group(m, 1, wd, xo, m->gate, rows, m->x, nullptr, m->up, m->gate2, m->xn, flags, s); // x = x + mlp
+			matmul_group(m, 1, wd, xo, m->gate, rows, m->x, nullptr, gated ? nullptr : m->up, m->gate2, m->xn, flags,
+			             s); // x = x + mlp
 		}
 		const size_t first = rows - logit_rows;
 		launch_rmsnorm(m->x + first * d, m->output_norm, m->p.rms_norm_epsilon, logit_rows, d, m->xn, s);

@@ -60,20 +60,25 @@ static uintptr_t piece_without_redirection(uintptr_t row_start, int c, int chunk
 }
 
 // returns the number of pieces that touch no byte of [base, base + bytes)
+// base_up != 0: the gated form (ng = 2), whose second weight group holds the same rows of a second
+// n-row matrix at base_up
 static long gemm_case(const Format& f, int ng, int waves, int n, int chunks, uintptr_t base, PieceFn piece_fn,
-                      bool check_contents)
+                      bool check_contents, uintptr_t base_up = 0)
 {
+	const bool gated = base_up != 0;
 	const size_t row_bytes = static_cast<size_t>(chunks) * f.chunk_bytes;
-	const uintptr_t end = base + static_cast<size_t>(n) * row_bytes;
+	const size_t bytes = static_cast<size_t>(n) * row_bytes;
 	const int pieces = fm::gemm_weight_pieces(f.chunk_bytes, f.aligned16);
 	const int loads = (ng * 16 * pieces + 63) / 64;
-	const int bn = 16 * waves * ng;
+	const int bn = gated ? 16 * waves : 16 * waves * ng;
+	const auto matrix_of = [&](int slot_row) { return gated && slot_row >= 16 ? base_up : base; };
+	const auto row_of = [&](int slot_row) { return gated ? (slot_row & 15) : slot_row; };
 	long outside = 0;
 	for (int block = 0; block < (n + bn - 1) / bn; ++block)
 	{
 		for (int wave = 0; wave < waves; ++wave)
 		{
-			const int n_base = (block * waves + wave) * 16 * ng;
+			const int n_base = (block * waves + wave) * 16 * (gated ? 1 : ng);
 			for (int c = 0; c < chunks; ++c)
 			{
 				std::map<int, uintptr_t> slot; // slot byte offset of a piece -> where it was fetched from
@@ -88,13 +93,15 @@ static long gemm_case(const Format& f, int ng, int waves, int n, int chunks, uin
 						}
 						CHECK(rq.row >= 0 && rq.row < 16 * ng && rq.offset >= 0 && rq.offset < 16 * pieces, "%s row %d off %d",
 						      f.name, rq.row, rq.offset);
-						const uintptr_t row_start = base + static_cast<size_t>(fm::gemm_weight_row(n_base, rq.row, n)) * row_bytes;
+						const uintptr_t mbase = matrix_of(rq.row), end = mbase + bytes;
+						const uintptr_t row_start =
+						    mbase + static_cast<size_t>(fm::gemm_weight_row(n_base, row_of(rq.row), n)) * row_bytes;
 						const uintptr_t from = piece_fn(row_start, c, f.chunk_bytes, f.aligned16, rq.offset);
 						if (check_contents)
 						{
 							CHECK(from % 16 == 0, "%s n %d: piece at %#zx is not aligned", f.name, n, static_cast<size_t>(from));
 						}
-						if (!(from < end && from + 16 > base))
+						if (!(from < end && from + 16 > mbase))
 						{
 							++outside;
 						}
@@ -110,7 +117,8 @@ static long gemm_case(const Format& f, int ng, int waves, int n, int chunks, uin
 				// chunk_bytes bytes, which must be the chunk's own bytes
 				for (int r = 0; r < 16 * ng; ++r)
 				{
-					const uintptr_t row_start = base + static_cast<size_t>(fm::gemm_weight_row(n_base, r, n)) * row_bytes;
+					const uintptr_t row_start =
+					    matrix_of(r) + static_cast<size_t>(fm::gemm_weight_row(n_base, row_of(r), n)) * row_bytes;
 					const uintptr_t chunk = row_start + static_cast<size_t>(c) * f.chunk_bytes;
 					const int mis = fm::gemm_weight_misalignment(row_start, c, f.chunk_bytes, f.aligned16);
 					for (int b = 0; b < f.chunk_bytes; ++b)
@@ -156,6 +164,15 @@ static void test_gemm_weight_pieces()
 						CHECK(outside == 0, "%s ng %d waves %d n %d chunks %d base %#zx: %ld pieces outside the tensor", f.name, t[0],
 						      t[1], n, chunks, static_cast<size_t>(base), outside);
 						++cases;
+						// the gated form: the gate matrix at `base`, the up matrix ending on a page far behind it
+						const uintptr_t up = 4096 * kPage - bytes;
+						if (t[0] == 2 && up % f.base_align == 0)
+						{
+							const long out2 = gemm_case(f, 2, t[1], n, chunks, base, fm::gemm_weight_piece, true, up);
+							CHECK(out2 == 0, "%s gated n %d chunks %d base %#zx: %ld pieces outside their matrix", f.name, n, chunks,
+							      static_cast<size_t>(base), out2);
+							++cases;
+						}
 					}
 				}
 			}

@@ -143,6 +143,24 @@ def test_prompt_pass_with_a_q6_k_value_projection(hip, oracle, main_fmt, d_model
     dev.close()
 
 
+@pytest.mark.parametrize("fmt,ff,rows", [(Q4_K, 5120, 512), (Q4_0, 5024, 500)])
+def test_prompt_pass_with_swiglu_in_the_gate_up_launch(hip, oracle, fmt, ff, rows):
+    """With enough rows and a wide enough feed-forward block the gate and up projections of a prompt
+    run as one matrix-core launch whose epilogue stores silu(gate) * up.  The second case has a
+    feed-forward width that is no multiple of the launch's 128-column strips and a row count that is
+    no multiple of its 128-row blocks.  Logits of the last row against the checker, and against the
+    Float32 path of the device, which forms the product in its own kernel."""
+    cfg = synth.tiny_llama(fmt, block_count=1, d_model=512, heads=8, kv_heads=2, ff=ff, vocab=333,
+                           context_length=rows + 4)
+    toks = synth.prompt_tokens(cfg, rows, 21)
+    dev, ref = hip_model(hip, cfg, 8, kv_dtype=DT_F32), oracle_model(oracle, cfg, 8, kv_f16=False)
+    got, want = dev.eval(toks, all_logits=False), ref.eval(toks, all_logits=False)
+    assert rel_l2(got, want) < 3e-3
+    dev.reset()
+    assert rel_l2(dev.eval(toks, all_logits=False, precise=True), want) < 1e-4
+    dev.close()
+
+
 def test_error_paths(hip):
     cfg = synth.tiny_llama(Q4_0, context_length=8)
     m = hip_model(hip, cfg, 1)
