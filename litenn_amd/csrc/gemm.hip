@@ -1363,6 +1363,8 @@ namespace litenn_hip
 			}
 		}
 
+#undef LITENN_GEMM_PICK_MATRIX
+
 		// ---- the GEMM for few activation rows ------------------------------------------------------
 		// With 16 or 32 activation rows the product is a stream of the weights, like the single-row
 		// GEMV, and is built like it: one workgroup of eight or sixteen wavefronts per CU, always a single round,
