@@ -135,8 +135,9 @@ int litenn_hip_permute(int dev, void* dst, int dtype, const size_t* src_shape, s
  * from and returned to the device's memory pool in stream order, see below).
  * residual (f32 [m, n]) may be NULL; when given, y = residual + x.W
  * (the Add at tools/gguf/LLaMABuilder.cpp:652-653,661-663).  residual may alias y.
- * m == 1..15 runs the streaming GEMV.  m >= 16 (with k a multiple of 256) runs on the matrix
- * cores: weights and activations are rounded to fp16 once each (activation rows are first scaled
+ * m == 1..3 runs the streaming GEMV, row by row.  m >= 4 (with k a multiple of 256) runs on the
+ * matrix cores (the rows padded to a multiple of 16; one padded tile costs about as much as three
+ * single-row launches): weights and activations are rounded to fp16 once each (activation rows are first scaled
  * by a power of two into the fp16 range), products accumulate in f32; relative L2 error about
  * 4e-4.  LITENN_HIP_MATMUL_PRECISE in `flags` keeps f32 operands (GEMV path) for any m.
  * The matrix-core path needs a device workspace of litenn_hip_mul_mat_q_workspace_bytes(m, k):
@@ -295,7 +296,7 @@ int litenn_hip_llama_past(const litenn_hip_llama* model);
 /* LowerLLaMACausalLMDecode(sequenceLength = m, pastLength = positionOffset = past) executed
  * against the cache the model holds (tools/gguf/LLaMABuilder.cpp:826-872); tokens are host
  * I32.  logits (host f32 [m, vocab]) and last_logits (host f32 [vocab]) may be NULL.
- * flags: LITENN_HIP_MATMUL_PRECISE keeps f32 activations for m >= 16. */
+ * flags: LITENN_HIP_MATMUL_PRECISE keeps f32 activations for m >= 4. */
 int litenn_hip_llama_eval(litenn_hip_llama* model, const int32_t* tokens, size_t m, float* logits, float* last_logits,
                           unsigned flags);
 /* Greedy loop kept on the device: eval(prompt), then n_new times argmax -> eval of that

@@ -736,9 +736,13 @@ static bool is_weight_format(int fmt)
 	return block_elements(fmt) != 0;
 }
 
+// From this many activation rows on a quantised matmul goes to the matrix cores: one padded 16-row
+// tile costs about as much as three single-row GEMVs (Q4_K 14336 x 4096: 14.6 us against 8.2 each).
+static constexpr size_t kMatrixCoreMinRows = 4;
+
 extern "C" size_t litenn_hip_mul_mat_q_workspace_bytes(size_t m, size_t k)
 {
-	return m >= 16 ? 2 * gemm_scratch_halves(m, k) : 0;
+	return m >= kMatrixCoreMinRows ? 2 * gemm_scratch_halves(m, k) : 0;
 }
 
 extern "C" int litenn_hip_mul_mat_q(int dev, int fmt, const void* wq, size_t n, size_t k, const void* x, int x_dtype,
@@ -799,7 +803,7 @@ extern "C" int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t 
 	float* yf = static_cast<float*>(y);
 	const float* rf = static_cast<const float*>(residual);
 	const bool quant = fmt != LITENN_FMT_F16 && fmt != LITENN_FMT_F32;
-	if (m >= 16 && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && k % 256 == 0)
+	if (m >= kMatrixCoreMinRows && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && k % 256 == 0)
 	{
 		// the matrix-core path rounds the activations to fp16 into a workspace
 		const size_t need = 2 * gemm_scratch_halves(m, k);

@@ -51,6 +51,18 @@ def test_gemm_matches_checker(hip, oracle, fmt, m, n, k):
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("m,n,k", [(4, 100, 256), (5, 999, 2048), (11, 64, 768), (15, 300, 4096)])
+def test_four_to_fifteen_rows_take_the_matrix_cores(hip, oracle, fmt, m, n, k):
+    """From four rows on the call pads the rows to a 16-row tile (the padding rows are zeros and are
+    never stored); two and three rows go row by row through the Float32 GEMV."""
+    err = run_case(hip, oracle, fmt, m, n, k, seed=m + n + k)
+    assert 1e-6 < err <= TOL, err
+    assert run_case(hip, oracle, fmt, m, n, k, seed=m + n + k + 1, residual=True) <= TOL
+    assert run_case(hip, oracle, fmt, m, n, k, seed=m + n + k, flags=MATMUL_PRECISE) <= 1e-5
+    assert run_case(hip, oracle, fmt, 3, n, k, seed=n + k) <= 1e-5
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
 def test_gemm_residual_and_precise_flag(hip, oracle, fmt):
     assert run_case(hip, oracle, fmt, 48, 200, 512, seed=9, residual=True) <= TOL
     # the flag keeps f32 activations (GEMV path): error drops to summation-order level
