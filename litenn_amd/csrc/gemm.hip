@@ -1353,13 +1353,13 @@ namespace litenn_hip
 			// compiler's inliner fall over)
 			if (grid_x < second_block)
 			{
-				gemm_q_body<F0, MT, NG, WAVES>(w, nullptr, y, n, block_x, mats.partial, xf0, unscale0, nullptr, k, m, m_tiles, row_bytes0,
-				                               grid_y);
+				gemm_q_body<F0, MT, NG, WAVES>(w, nullptr, y, n, block_x, mats.partial, xf0, unscale0, nullptr, k, m, m_tiles,
+				                               row_bytes0, grid_y);
 			}
 			else
 			{
-				gemm_q_body<F1, MT, NG, WAVES>(w, nullptr, y, n, block_x, mats.partial, xf1, unscale1, nullptr, k, m, m_tiles, row_bytes1,
-				                               grid_y);
+				gemm_q_body<F1, MT, NG, WAVES>(w, nullptr, y, n, block_x, mats.partial, xf1, unscale1, nullptr, k, m, m_tiles,
+				                               row_bytes1, grid_y);
 			}
 		}
 
