@@ -276,9 +276,13 @@ namespace litenn_hip
 		{
 			static constexpr int E = 8;
 			using Raw = uint4;
+			// non-temporal like the weight rows of the GEMV: a cached key or value is read once per launch
+			// by the query heads of its group (7B-shape decode 728.7 -> 737.1 tok/s, 8B shape 635.7 -> 641.3)
 			__device__ static Raw load(const uint16_t* p, int first, int, int)
 			{
-				return *reinterpret_cast<const uint4*>(p + first);
+				typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+				const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p + first));
+				return make_uint4(v.x, v.y, v.z, v.w);
 			}
 			__device__ static void unpack(const Raw& raw, float (&out)[E])
 			{
