@@ -633,15 +633,6 @@ namespace litenn_hip
 			}
 		};
 
-		// The products leave through non-temporal stores: nobody reads them before the launch ends, and
-		// written past the caches they do not push weights and activation fragments out of the L2s
-		// while other workgroups still walk (Q4_K 14336 x 4096 at 512 rows: 86 -> 82 us with its pre-pass).
-		typedef float f32x4_nt __attribute__((ext_vector_type(4)));
-		__device__ __forceinline__ void st4_out(float* p, float4 v)
-		{
-			__builtin_nontemporal_store(f32x4_nt{ v.x, v.y, v.z, v.w }, reinterpret_cast<f32x4_nt*>(p));
-		}
-
 		// ---- activations to fp16, in fragment order ----------------------------------------------------
 		// One workgroup per row.  Every row is scaled by a power of two so that its largest magnitude
 		// lands in [2^14, 2^15): nothing overflows fp16 whatever the activations' range, small rows keep
@@ -1255,7 +1246,7 @@ namespace litenn_hip
 						}
 						if (vec_ok && n0 + 3 < n)
 						{
-							st4_out(dst, float4{ vals[0], vals[1], vals[2], vals[3] });
+							*reinterpret_cast<float4*>(dst) = float4{ vals[0], vals[1], vals[2], vals[3] };
 						}
 						else
 						{
@@ -1297,7 +1288,7 @@ namespace litenn_hip
 								const float4 rv = *reinterpret_cast<const float4*>(res);
 								out.x += rv.x, out.y += rv.y, out.z += rv.z, out.w += rv.w;
 							}
-							st4_out(dst, out);
+							*reinterpret_cast<float4*>(dst) = out;
 						}
 						else
 						{
@@ -1557,7 +1548,7 @@ namespace litenn_hip
 								const float4 rv = *reinterpret_cast<const float4*>(res);
 								out.x += rv.x, out.y += rv.y, out.z += rv.z, out.w += rv.w;
 							}
-							st4_out(dst, out);
+							*reinterpret_cast<float4*>(dst) = out;
 						}
 						else
 						{
