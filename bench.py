@@ -242,6 +242,7 @@ def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=8):
     tl.litenn_hip_mul_mat_q.argtypes = [C.c_int, C.c_int, vp, sz, sz, vp, C.c_int, sz, vp, vp, C.c_uint, C.POINTER(Exec)]
     tl.litenn_hip_mb_empty.argtypes = [C.c_int, C.c_int, sz, vp]
     tl.litenn_hip_mb_read.argtypes = [vp, sz, C.c_int, C.c_int, vp, vp]
+    tl.litenn_hip_mb_read_policy.argtypes = [vp, sz, C.c_int, C.c_int, C.c_int, vp, vp]
     tl.litenn_hip_gemv_trace_read.argtypes = [vp, sz]
     tl.litenn_hip_gemv_trace_skip_arithmetic.argtypes = [C.c_int]
 
@@ -296,9 +297,22 @@ def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=8):
     best = min(reads, key=lambda r: r["us"])
     out["read_kernel_best"] = best
     out["read_kernel_all"] = reads
+    # the same with non-temporal loads (the policy of the GEMV's weight rows)
+    reads_nt = []
+    for blocks in (256, 512, 1024, 2048):
+        for depth in (2, 4, 8):
+            us = per_launch_us(lambda i: ok(tl.litenn_hip_mb_read_policy(weights[i % n_buffers].ptr, w_bytes, blocks,
+                                                                         depth, 1, sink.ptr, stream.handle)))
+            reads_nt.append({"blocks": blocks, "loads_in_flight_per_lane": depth, "us": round(us, 3),
+                             "gbps": round(w_bytes / us / 1e3, 1)})
+    best_nt = min(reads_nt, key=lambda r: r["us"])
+    out["read_kernel_nontemporal_best"] = best_nt
+    out["read_kernel_nontemporal_all"] = reads_nt
     log(f"[bench] microbench: empty kernel {out['empty_kernel_us']} us/launch (one workgroup of 64 threads: "
         f"{out['empty_kernel_one_workgroup_us']}); read-only kernel best "
-        f"{best['us']} us = {best['gbps']} GB/s ({best['blocks']} workgroups, {best['loads_in_flight_per_lane']} loads/lane)")
+        f"{best['us']} us = {best['gbps']} GB/s ({best['blocks']} workgroups, {best['loads_in_flight_per_lane']} loads/lane); "
+        f"with non-temporal loads {best_nt['us']} us = {best_nt['gbps']} GB/s ({best_nt['blocks']} workgroups, "
+        f"{best_nt['loads_in_flight_per_lane']} loads/lane)")
 
     def gemv(i):
         ok(tl.litenn_hip_mul_mat_q(0, fmt, weights[i % n_buffers].ptr, n, k, x.ptr, 0, 1, y.ptr, None, 0, C.byref(opts)))

@@ -17,7 +17,21 @@ namespace litenn_hip
 		// Every workgroup reads a contiguous share of the buffer with 128-bit loads, `depth` of them
 		// in flight per lane, and folds what it read into one value that is stored only if it
 		// equals a sentinel (so the loads cannot be dropped and nothing is written).
-		template <int DEPTH>
+		// ONCE: the loads carry the non-temporal bit, like the weight rows of the streaming GEMV.
+		template <bool ONCE>
+		__device__ __forceinline__ u32x4 mb_load(const u32x4* p)
+		{
+			if constexpr (ONCE)
+			{
+				return __builtin_nontemporal_load(p);
+			}
+			else
+			{
+				return *p;
+			}
+		}
+
+		template <int DEPTH, bool ONCE>
 		__global__ __launch_bounds__(512) void mb_read_kernel(const u32x4* __restrict__ src, size_t pieces,
 		                                                       unsigned* __restrict__ sink)
 		{
@@ -32,7 +46,7 @@ namespace litenn_hip
 #pragma unroll
 				for (int j = 0; j < DEPTH; ++j)
 				{
-					v[j] = src[i + static_cast<size_t>(j) * blockDim.x];
+					v[j] = mb_load<ONCE>(src + i + static_cast<size_t>(j) * blockDim.x);
 				}
 #pragma unroll
 				for (int j = 0; j < DEPTH; ++j)
@@ -42,7 +56,7 @@ namespace litenn_hip
 			}
 			for (; i < end; i += blockDim.x)
 			{
-				const u32x4 v = src[i];
+				const u32x4 v = mb_load<ONCE>(src + i);
 				acc ^= v.x ^ v.y ^ v.z ^ v.w;
 			}
 			if (acc == 0x9E3779B9u)
@@ -188,9 +202,10 @@ extern "C" int litenn_hip_mb_empty(int blocks, int threads, size_t lds_bytes, vo
 }
 
 // One launch that reads `bytes` (a multiple of 16) at `src` once: `blocks` workgroups of 512
-// threads, `depth` (1, 2, 4 or 8) 128-bit loads in flight per lane.  `sink` is 4 bytes of device
-// memory that is never written in practice.
-extern "C" int litenn_hip_mb_read(const void* src, size_t bytes, int blocks, int depth, void* sink, void* stream)
+// threads, `depth` (1, 2, 4 or 8) 128-bit loads in flight per lane, with the non-temporal bit when
+// `nontemporal` is non-zero.  `sink` is 4 bytes of device memory that is never written in practice.
+extern "C" int litenn_hip_mb_read_policy(const void* src, size_t bytes, int blocks, int depth, int nontemporal,
+                                         void* sink, void* stream)
 {
 	using namespace litenn_hip;
 	if (!src || !sink || bytes % 16 != 0 || blocks < 1)
@@ -200,16 +215,33 @@ extern "C" int litenn_hip_mb_read(const void* src, size_t bytes, int blocks, int
 	const u32x4* p = static_cast<const u32x4*>(src);
 	unsigned* s = static_cast<unsigned*>(sink);
 	hipStream_t st = static_cast<hipStream_t>(stream);
+#define LITENN_MB_READ(D)                                                                                           \
+	case D:                                                                                                          \
+		if (nontemporal)                                                                                             \
+		{                                                                                                            \
+			mb_read_kernel<D, true><<<dim3(blocks), dim3(512), 0, st>>>(p, bytes / 16, s);                           \
+		}                                                                                                            \
+		else                                                                                                         \
+		{                                                                                                            \
+			mb_read_kernel<D, false><<<dim3(blocks), dim3(512), 0, st>>>(p, bytes / 16, s);                          \
+		}                                                                                                            \
+		break;
 	switch (depth)
 	{
-	case 1: mb_read_kernel<1><<<dim3(blocks), dim3(512), 0, st>>>(p, bytes / 16, s); break;
-	case 2: mb_read_kernel<2><<<dim3(blocks), dim3(512), 0, st>>>(p, bytes / 16, s); break;
-	case 4: mb_read_kernel<4><<<dim3(blocks), dim3(512), 0, st>>>(p, bytes / 16, s); break;
-	case 8: mb_read_kernel<8><<<dim3(blocks), dim3(512), 0, st>>>(p, bytes / 16, s); break;
+		LITENN_MB_READ(1)
+		LITENN_MB_READ(2)
+		LITENN_MB_READ(4)
+		LITENN_MB_READ(8)
 	default: return fail("launch the read kernel", "depth must be 1, 2, 4 or 8");
 	}
+#undef LITENN_MB_READ
 	LITENN_HIP_TRY("launch the read kernel", hipGetLastError());
 	return 0;
+}
+
+extern "C" int litenn_hip_mb_read(const void* src, size_t bytes, int blocks, int depth, void* sink, void* stream)
+{
+	return litenn_hip_mb_read_policy(src, bytes, blocks, depth, 0, sink, stream);
 }
 
 // The GEMM's instruction mix without its memory traffic: `blocks` workgroups of `threads` (256 or
