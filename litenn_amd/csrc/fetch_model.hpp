@@ -111,10 +111,25 @@ namespace litenn_hip
 		{
 			int row0, count;
 		};
-		LITENN_FETCH_FN StreamRows stream_group_rows(int block, int g, int groups, int rows_per_group, int n_total)
+		// A workgroup's groups walk consecutive runs of its groups * rows_per_group rows.  With
+		// skew > 0 (an even number of groups) the first half of the groups walk rows_per_group + skew
+		// rows each and the second half rows_per_group - skew: of the two wavefronts that share a
+		// SIMD the one that arrived first (the lower index) gets ahead of the other, and the
+		// longer run levels the two.
+		LITENN_FETCH_FN int stream_group_run(int g, int groups, int rows_per_group, int skew)
 		{
-			const int row0 = (block * groups + g) * rows_per_group;
-			return { row0, imax(0, imin(rows_per_group, n_total - row0)) };
+			return 2 * g < groups ? rows_per_group + skew : rows_per_group - skew;
+		}
+		LITENN_FETCH_FN int stream_group_first(int g, int groups, int rows_per_group, int skew)
+		{
+			const int half = groups / 2;
+			return 2 * g < groups ? g * (rows_per_group + skew)
+			                      : half * (rows_per_group + skew) + (g - half) * (rows_per_group - skew);
+		}
+		LITENN_FETCH_FN StreamRows stream_group_rows(int block, int g, int groups, int rows_per_group, int skew, int n_total)
+		{
+			const int row0 = block * groups * rows_per_group + stream_group_first(g, groups, rows_per_group, skew);
+			return { row0, imax(0, imin(stream_group_run(g, groups, rows_per_group, skew), n_total - row0)) };
 		}
 
 		// first float of the 128-bit activation load j of thread `tid` (clamped: every lane issues

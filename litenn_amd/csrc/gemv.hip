@@ -1033,6 +1033,7 @@ namespace litenn_hip
 			uint32_t row_bytes;
 			int slices, groups;
 			int rows_per_group;    // consecutive rows one wavefront group walks (<= 64)
+			int skew;              // the first half of the groups walk this many rows more, the second half as many fewer
 			int silu_mul;          // 1: w[0] = gate, w[1] = up, row 2i + m; y[0][i] = silu(gate_i) * up_i
 		};
 
@@ -1595,9 +1596,34 @@ namespace litenn_hip
 				++rows;
 			}
 			a.rows_per_group = rows;
+			// Of the two wavefronts that share a SIMD the one that arrived first wins the issue
+			// arbitration and finishes about a seventh of the walk ahead of the other (north-star
+			// launch: 5.85 against 6.79 us): it is given that many more rows and the other as many fewer
+			// (7.80 -> 7.42 us; 7B-shape decode 729 -> 738 tok/s).  Only with eight wavefronts in an even
+			// number of groups, where the first half of the groups are the wavefronts that arrive first
+			// (the six wavefronts of K = 11008 gain nothing from it: 8.9 -> 8.85 us); gate/up pairs keep
+			// both runs even.
+			static const int forced_skew = env_int("LITENN_HIP_GEMV_SKEW", -1);
+			int skew = 0;
+			if (nwaves == 8 && a.groups % 2 == 0)
+			{
+				// about a seventh of the run, at least one row (4096 x 4096, runs of 2: 6.28 -> 5.97 us)
+				skew = a.silu_mul ? 2 * ((rows + 4) / 14) : (rows >= 2 ? std::max(1, (2 * rows + 7) / 14) : 0);
+				if (forced_skew >= 0)
+				{
+					skew = a.silu_mul ? (forced_skew & ~1) : forced_skew;
+				}
+				skew = std::min(std::min(skew, rows - 1), kMaxStreamRows - rows);
+				if (a.silu_mul)
+				{
+					skew &= ~1;
+				}
+				skew = std::max(skew, 0);
+			}
+			a.skew = skew;
 			blocks = (a.n_total + a.groups * rows - 1) / (a.groups * rows);
 			lds = x_bytes + static_cast<size_t>(nwaves) * kPrefetchRows * U::kSliceBytes +
-			      ((sizeof(float) * nwaves * rows + 7) & ~size_t{ 7 }) + sizeof(double) * nwaves;
+			      ((sizeof(float) * nwaves * (rows + skew) + 7) & ~size_t{ 7 }) + sizeof(double) * nwaves;
 			return lds <= kStreamLdsLimit;
 		}
 

@@ -384,28 +384,40 @@ static void test_stream_rows_and_pieces()
 						int rows = (n_total + max_blocks * groups - 1) / (max_blocks * groups);
 						rows = rows < 1 ? 1 : (rows > 64 ? 64 : rows);
 						const int blocks = (n_total + groups * rows - 1) / (groups * rows);
-						std::vector<int> walked(n_total, 0);
-						for (int block = 0; block < blocks; ++block)
+						// the uneven split between the halves of a workgroup's groups: every skew the
+						// launcher may choose (an even number of groups, both runs at least one row
+						// and at most 64)
+						for (int skew = 0; skew < rows && rows + skew <= 64 && (skew == 0 || groups % 2 == 0); ++skew)
 						{
-							for (int g = 0; g < groups; ++g)
+							std::vector<int> walked(n_total, 0);
+							for (int block = 0; block < blocks; ++block)
 							{
-								const fm::StreamRows r = fm::stream_group_rows(block, g, groups, rows, n_total);
-								CHECK(r.count >= 0 && r.count <= rows, "count %d", r.count);
-								for (int q = 0; q < r.count; ++q)
+								int expect = block * groups * rows; // the groups' runs follow each other
+								for (int g = 0; g < groups; ++g)
 								{
-									CHECK(r.row0 + q < n_total, "%s k %d n %d: row %d", f.name, k, n_total, r.row0 + q);
-									if (r.row0 + q < n_total)
+									const fm::StreamRows r = fm::stream_group_rows(block, g, groups, rows, skew, n_total);
+									const int run = fm::stream_group_run(g, groups, rows, skew);
+									CHECK(r.row0 == expect && run >= 1 && run <= 64, "run %d of group %d starts at %d, expected %d", run, g,
+									      r.row0, expect);
+									CHECK(r.count >= 0 && r.count <= run, "count %d", r.count);
+									expect += run;
+									for (int q = 0; q < r.count; ++q)
 									{
-										++walked[r.row0 + q];
+										CHECK(r.row0 + q < n_total, "%s k %d n %d: row %d", f.name, k, n_total, r.row0 + q);
+										if (r.row0 + q < n_total)
+										{
+											++walked[r.row0 + q];
+										}
 									}
 								}
+								CHECK(expect == (block + 1) * groups * rows, "a workgroup's runs cover %d rows", expect - block * groups * rows);
 							}
+							for (int r = 0; r < n_total; ++r)
+							{
+								CHECK(walked[r] == 1, "%s k %d n %d skew %d: row %d walked %d times", f.name, k, n_total, skew, r, walked[r]);
+							}
+							++cases;
 						}
-						for (int r = 0; r < n_total; ++r)
-						{
-							CHECK(walked[r] == 1, "%s k %d n %d: row %d walked %d times", f.name, k, n_total, r, walked[r]);
-						}
-						++cases;
 					}
 				}
 			}
