@@ -111,25 +111,24 @@ namespace litenn_hip
 		{
 			int row0, count;
 		};
-		// A workgroup's groups walk consecutive runs of its groups * rows_per_group rows.  With
-		// skew > 0 (an even number of groups) the first half of the groups walk rows_per_group + skew
-		// rows each and the second half rows_per_group - skew: of the two wavefronts that share a
-		// SIMD the one that arrived first (the lower index) gets ahead of the other, and the
-		// longer run levels the two.
-		LITENN_FETCH_FN int stream_group_run(int g, int groups, int rows_per_group, int skew)
+		// A workgroup's groups walk consecutive runs of its rows.  The first half of the groups walk
+		// `run` rows each and the second half `run - diff` (diff > 0 only with an even number of
+		// groups): of the two wavefronts that share a SIMD the one that arrived first (the lower
+		// index) gets ahead of the other, and the longer run levels the two.
+		LITENN_FETCH_FN int stream_group_run(int g, int groups, int run, int diff)
 		{
-			return 2 * g < groups ? rows_per_group + skew : rows_per_group - skew;
+			return 2 * g < groups ? run : run - diff;
 		}
-		LITENN_FETCH_FN int stream_group_first(int g, int groups, int rows_per_group, int skew)
+		LITENN_FETCH_FN int stream_group_first(int g, int groups, int run, int diff)
 		{
 			const int half = groups / 2;
-			return 2 * g < groups ? g * (rows_per_group + skew)
-			                      : half * (rows_per_group + skew) + (g - half) * (rows_per_group - skew);
+			return 2 * g < groups ? g * run : g * run - (g - half) * diff;
 		}
-		LITENN_FETCH_FN StreamRows stream_group_rows(int block, int g, int groups, int rows_per_group, int skew, int n_total)
+		LITENN_FETCH_FN int stream_block_rows(int groups, int run, int diff) { return groups * run - (groups / 2) * diff; }
+		LITENN_FETCH_FN StreamRows stream_group_rows(int block, int g, int groups, int run, int diff, int n_total)
 		{
-			const int row0 = block * groups * rows_per_group + stream_group_first(g, groups, rows_per_group, skew);
-			return { row0, imax(0, imin(stream_group_run(g, groups, rows_per_group, skew), n_total - row0)) };
+			const int row0 = block * stream_block_rows(groups, run, diff) + stream_group_first(g, groups, run, diff);
+			return { row0, imax(0, imin(stream_group_run(g, groups, run, diff), n_total - row0)) };
 		}
 
 		// first float of the 128-bit activation load j of thread `tid` (clamped: every lane issues

@@ -1032,8 +1032,8 @@ namespace litenn_hip
 			int k;
 			uint32_t row_bytes;
 			int slices, groups;
-			int rows_per_group;    // consecutive rows one wavefront group walks (<= 64)
-			int skew;              // the first half of the groups walk this many rows more, the second half as many fewer
+			int rows_per_group;    // consecutive rows a wavefront group of the first half walks (<= 64)
+			int run_diff;          // the groups of the second half walk this many rows fewer
 			int silu_mul;          // 1: w[0] = gate, w[1] = up, row 2i + m; y[0][i] = silu(gate_i) * up_i
 		};
 
@@ -1595,35 +1595,51 @@ namespace litenn_hip
 			{
 				++rows;
 			}
-			a.rows_per_group = rows;
+			int diff = 0;
 			// Of the two wavefronts that share a SIMD the one that arrived first wins the issue
 			// arbitration and finishes about a seventh of the walk ahead of the other (north-star
-			// launch: 5.85 against 6.79 us): it is given that many more rows and the other as many fewer
-			// (7.80 -> 7.42 us; 7B-shape decode 729 -> 738 tok/s).  Only with eight wavefronts in an even
-			// number of groups, where the first half of the groups are the wavefronts that arrive first
-			// (the six wavefronts of K = 11008 gain nothing from it: 8.9 -> 8.85 us); gate/up pairs keep
-			// both runs even.
-			static const int forced_skew = env_int("LITENN_HIP_GEMV_SKEW", -1);
-			int skew = 0;
-			if (nwaves == 8 && a.groups % 2 == 0)
+			// launch, 7 rows each: 5.85 against 6.79 us).  So the rows are dealt out per pair of
+			// groups that share SIMDs - with eight wavefronts in an even number of groups, group g of
+			// the first half and group g of the second - and the first takes about a seventh of the
+			// pair's rows more than the second (8 and 6 rows: 7.80 -> 7.42 us; 7B-shape decode
+			// 729 -> 738 tok/s; runs of 3 and 1 for 4096 x 4096: 6.28 -> 5.87 us).  The pair's total need
+			// not be even (11 rows as 6 + 5 where equal runs would take 6 + 6 on fewer workgroups);
+			// gate/up pairs keep both runs even.  The six wavefronts of K = 11008 gain nothing from an
+			// uneven split (8.9 -> 8.85 us) and keep equal runs.
+			static const int forced_diff = env_int("LITENN_HIP_GEMV_SKEW", -1); // 0: equal runs
+			if (nwaves == 8 && a.groups % 2 == 0 && forced_rows <= 0 && forced_diff != 0)
 			{
-				// about a seventh of the run, at least one row (4096 x 4096, runs of 2: 6.28 -> 5.97 us)
-				skew = a.silu_mul ? 2 * ((rows + 4) / 14) : (rows >= 2 ? std::max(1, (2 * rows + 7) / 14) : 0);
-				if (forced_skew >= 0)
+				const int unit = a.silu_mul ? 2 : 1; // a run is a whole number of these
+				const int half_groups = a.groups / 2;
+				int total = (a.n_total + max_blocks * half_groups - 1) / (max_blocks * half_groups); // rows of a pair
+				total = std::max((total + unit - 1) / unit * unit, 2 * unit);
+				// the nearest difference to a seventh of the total (at least one unit) that leaves both
+				// runs whole numbers of units
+				int best = -1;
+				for (int d = 0; d < total; d += unit)
 				{
-					skew = a.silu_mul ? (forced_skew & ~1) : forced_skew;
+					if ((total + d) % (2 * unit) != 0 || (total - d) / 2 < unit || (total + d) / 2 > kMaxStreamRows)
+					{
+						continue;
+					}
+					const int target = forced_diff > 0 ? 7 * forced_diff : std::max(total, 7 * unit);
+					if (best < 0 || std::abs(7 * d - target) <= std::abs(7 * best - target))
+					{
+						best = d;
+					}
 				}
-				skew = std::min(std::min(skew, rows - 1), kMaxStreamRows - rows);
-				if (a.silu_mul)
+				if (best >= 0)
 				{
-					skew &= ~1;
+					rows = (total + best) / 2;
+					diff = best;
 				}
-				skew = std::max(skew, 0);
 			}
-			a.skew = skew;
-			blocks = (a.n_total + a.groups * rows - 1) / (a.groups * rows);
+			a.rows_per_group = rows;
+			a.run_diff = diff;
+			const int block_rows = fetch::stream_block_rows(a.groups, rows, diff);
+			blocks = (a.n_total + block_rows - 1) / block_rows;
 			lds = x_bytes + static_cast<size_t>(nwaves) * kPrefetchRows * U::kSliceBytes +
-			      ((sizeof(float) * nwaves * (rows + skew) + 7) & ~size_t{ 7 }) + sizeof(double) * nwaves;
+			      ((sizeof(float) * nwaves * rows + 7) & ~size_t{ 7 }) + sizeof(double) * nwaves;
 			return lds <= kStreamLdsLimit;
 		}
 

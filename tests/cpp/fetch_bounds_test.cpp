@@ -383,21 +383,21 @@ static void test_stream_rows_and_pieces()
 					{
 						int rows = (n_total + max_blocks * groups - 1) / (max_blocks * groups);
 						rows = rows < 1 ? 1 : (rows > 64 ? 64 : rows);
-						const int blocks = (n_total + groups * rows - 1) / (groups * rows);
-						// the uneven split between the halves of a workgroup's groups: every skew the
-						// launcher may choose (an even number of groups, both runs at least one row
-						// and at most 64)
-						for (int skew = 0; skew < rows && rows + skew <= 64 && (skew == 0 || groups % 2 == 0); ++skew)
+						// every pair of runs the launcher may choose: the first half of the groups walk `run`
+						// rows, the second half `run - diff` (an even number of groups, both at least one row)
+						for (int diff = 0; diff < rows && (diff == 0 || groups % 2 == 0); ++diff)
 						{
+							const int block_rows = fm::stream_block_rows(groups, rows, diff);
+							const int blocks = (n_total + block_rows - 1) / block_rows;
 							std::vector<int> walked(n_total, 0);
 							for (int block = 0; block < blocks; ++block)
 							{
-								int expect = block * groups * rows; // the groups' runs follow each other
+								int expect = block * block_rows; // the groups' runs follow each other
 								for (int g = 0; g < groups; ++g)
 								{
-									const fm::StreamRows r = fm::stream_group_rows(block, g, groups, rows, skew, n_total);
-									const int run = fm::stream_group_run(g, groups, rows, skew);
-									CHECK(r.row0 == expect && run >= 1 && run <= 64, "run %d of group %d starts at %d, expected %d", run, g,
+									const fm::StreamRows r = fm::stream_group_rows(block, g, groups, rows, diff, n_total);
+									const int run = fm::stream_group_run(g, groups, rows, diff);
+									CHECK(r.row0 == expect && run >= 1 && run <= rows, "run %d of group %d starts at %d, expected %d", run, g,
 									      r.row0, expect);
 									CHECK(r.count >= 0 && r.count <= run, "count %d", r.count);
 									expect += run;
@@ -410,11 +410,11 @@ static void test_stream_rows_and_pieces()
 										}
 									}
 								}
-								CHECK(expect == (block + 1) * groups * rows, "a workgroup's runs cover %d rows", expect - block * groups * rows);
+								CHECK(expect == (block + 1) * block_rows, "a workgroup's runs cover %d rows", expect - block * block_rows);
 							}
 							for (int r = 0; r < n_total; ++r)
 							{
-								CHECK(walked[r] == 1, "%s k %d n %d skew %d: row %d walked %d times", f.name, k, n_total, skew, r, walked[r]);
+								CHECK(walked[r] == 1, "%s k %d n %d diff %d: row %d walked %d times", f.name, k, n_total, diff, r, walked[r]);
 							}
 							++cases;
 						}
