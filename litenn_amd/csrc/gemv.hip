@@ -967,6 +967,7 @@ namespace litenn_hip
 		}
 
 		constexpr int kMaxSlices = 8;       // K <= 32768
+		constexpr int kTwelveXp = 4;        // activation loads per thread of the twelve-wavefront instance
 		constexpr int kMaxRowsPerWave = 64; // rows a wavefront of the register kernel may own
 		constexpr int kLdsUnitStride = 68;  // floats between the staged activations of consecutive units
 		constexpr int kXPerThread = 8;      // most 128-bit activation loads a thread issues while staging
@@ -1149,8 +1150,8 @@ namespace litenn_hip
 		// six of them), so the activation loads and the first row requests do not wait for the block to
 		// be read from memory; on a card whose firmware does not preload, the kernel's compatibility
 		// prologue loads them like any other argument.
-		template <typename U, int XP, bool WHOLE>
-		__global__ __launch_bounds__(512) void gemv_stream_kernel(const float* x_first, int k_first,
+		template <typename U, int XP, bool WHOLE, int THREADS = 512>
+		__global__ __launch_bounds__(THREADS) void gemv_stream_kernel(const float* x_first, int k_first,
 		                                                           const uint8_t* w0_first, uint32_t row_bytes_first,
 		                                                           int rows_per_group_first, int n_total_first,
 		                                                           const GemvArgs block_args)
@@ -1537,6 +1538,17 @@ namespace litenn_hip
 						                                                                         g.rows_per_group, g.n_total, g);
 					}
 				}
+				else if (threads > 512)
+				{
+					// twelve wavefronts (three-slice rows): an instance compiled for that many
+					if constexpr (XP == kTwelveXp)
+					{
+						allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, XP, false, 768>), kStreamLdsLimit);
+						const GemvArgs& g = launch.part[0];
+						gemv_stream_kernel<U0, XP, false, 768><<<dim3(blocks), dim3(threads), lds, stream>>>(
+						    g.x, g.k, g.w[0], g.row_bytes, g.rows_per_group, g.n_total, g);
+					}
+				}
 				else
 				{
 					allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, XP, false>), kStreamLdsLimit);
@@ -1557,8 +1569,10 @@ namespace litenn_hip
 		// Fills the launch geometry of one part for a budget of `max_blocks` workgroups (one round, at
 		// most one per CU, every group walking the same number of rows, an even number when gate/up
 		// rows are paired).  Returns false when the shape does not fit the streaming kernel.
+		// twelve: the launch may use twelve wavefronts (the single-format kernel has an instance for
+		// them; the two-format kernel has not)
 		template <typename U>
-		bool plan_stream(GemvArgs& a, int max_blocks, int& blocks, size_t& lds)
+		bool plan_stream(GemvArgs& a, int max_blocks, int& blocks, size_t& lds, bool twelve = false)
 		{
 			const int k = a.k;
 			a.slices = (k + 4095) / 4096;
@@ -1578,6 +1592,17 @@ namespace litenn_hip
 				return false;
 			}
 			a.groups = 8 / a.slices;
+			// Rows of three slices (8192 < K <= 12288, the last slice shorter): two groups of three
+			// wavefronts put two full slices on one SIMD and a short one alone on another; four groups
+			// give every SIMD two full slices and a short one (4096 x 11008: 8.9 -> 8.1 us, 7B-shape
+			// decode 752 -> 767 tok/s).
+			static const int use_twelve = env_int("LITENN_HIP_GEMV_TWELVE", 1);
+			if (twelve && use_twelve && a.slices == 3 && (k / 4 + 767) / 768 <= kTwelveXp && (k / 4 + 767) / 768 > kTwelveXp / 2 &&
+			    sizeof(float) * (static_cast<size_t>(k) / 64) * kLdsUnitStride + 12 * kPrefetchRows * U::kSliceBytes + 4096 <=
+			        kStreamLdsLimit)
+			{
+				a.groups = 4;
+			}
 			const int nwaves = a.slices * a.groups;
 			if (k > 64 * nwaves * 4 * kXPerThread)
 			{
@@ -1676,7 +1701,7 @@ namespace litenn_hip
 		{
 			int blocks = 0;
 			size_t lds = 0;
-			if (!plan_stream<U>(a, compute_units(), blocks, lds))
+			if (!plan_stream<U>(a, compute_units(), blocks, lds, true))
 			{
 				return false;
 			}

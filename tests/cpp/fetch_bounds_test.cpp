@@ -307,8 +307,10 @@ static void test_stream_rows_and_pieces()
 			{
 				continue; // the launcher sends such a shape to the register kernel
 			}
-			const int groups = 8 / slices;
-			if (k > 64 * slices * groups * 4 * 8)
+			// three-slice rows also run with twelve wavefronts (four groups)
+			for (int groups : { 8 / slices, slices == 3 ? 4 : 0 })
+			{
+			if (groups == 0 || k > 64 * slices * groups * 4 * 8)
 			{
 				continue; // more than eight 128-bit activation loads per thread: register kernel as well
 			}
@@ -420,6 +422,7 @@ static void test_stream_rows_and_pieces()
 						}
 					}
 				}
+			}
 			}
 		}
 	}
