@@ -1592,10 +1592,9 @@ namespace litenn_hip
 				return false;
 			}
 			a.groups = 8 / a.slices;
-			// Rows of three slices (8192 < K <= 12288, the last slice shorter): two groups of three
-			// wavefronts put two full slices on one SIMD and a short one alone on another; four groups
-			// give every SIMD two full slices and a short one (4096 x 11008: 8.9 -> 8.1 us, 7B-shape
-			// decode 752 -> 767 tok/s).
+			// Rows of three slices (8192 < K <= 12288): two groups of three wavefronts put two
+			// wavefronts on two of the SIMDs and one on the other two; four groups give every SIMD
+			// three (4096 x 11008: 8.9 -> 8.1 us, 7B-shape decode 752 -> 767 tok/s).
 			static const int use_twelve = env_int("LITENN_HIP_GEMV_TWELVE", 1);
 			if (twelve && use_twelve && a.slices == 3 && (k / 4 + 767) / 768 <= kTwelveXp && (k / 4 + 767) / 768 > kTwelveXp / 2 &&
 			    sizeof(float) * (static_cast<size_t>(k) / 64) * kLdsUnitStride + 12 * kPrefetchRows * U::kSliceBytes + 4096 <=
