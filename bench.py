@@ -594,7 +594,7 @@ def main() -> int:
             "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": measured_traffic_bytes(),
             "traffic_unit": "bytes/launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
             "algorithmic_bytes": algo_bytes,
-            "kernel": "gemv_stream_kernel<Q4_KUnit, 2, true>",
+            "kernel": "gemv_stream_kernel<Q4_KUnit, 2, true, 512>",
         },
     }
     if args.microbench:
