@@ -52,6 +52,29 @@ def measured_traffic_bytes():
         return None
 
 
+def traffic_source():
+    """Where `roofline.traffic` comes from: the committed summary and the commit that last touched it."""
+    import subprocess
+    rel = os.path.relpath(TRAFFIC_SUMMARY, ROOT)
+    try:
+        rev = subprocess.run(["git", "-C", ROOT, "log", "-1", "--format=%h", "--", rel], capture_output=True, text=True,
+                             timeout=10).stdout.strip()
+    except (OSError, subprocess.SubprocessError):
+        rev = ""
+    return {"file": rel, "commit": rev or None,
+            "note": "a property of the kernel and the shape, measured with rocprofv3 --pmc when the kernel last "
+                    "changed; not re-measured by this run"}
+
+
+def last_gemv_launch():
+    """The instance and geometry of the streaming kernel this thread launched last, as the library reports it."""
+    import ctypes as C
+    from litenn_amd._lib import check, load
+    buf = C.create_string_buffer(512)
+    check(load().litenn_hip_gemv_last_launch(buf, len(buf)))
+    return buf.value.decode()
+
+
 def measured_config_traffic():
     """{(format name, n, k): HBM bytes per launch} of the other single-row configurations, from their
     committed profiler summary (same method as the headline's); empty when the summary is not there."""
@@ -113,14 +136,23 @@ def bench_gemv(ln, hiprt, fmt, n, k, steps, warmup, n_buffers, seed=1, graph_rot
         return g
 
     graph = capture(graph_len) if graph_len else None
+    priming = None if graph_len else capture(DIRECT_PRIMING)
     rest = capture(steps % graph_len) if graph_len and steps % graph_len else None
     e0, e1 = hiprt.Event(), hiprt.Event()
     hiprt.device_synchronize()
+    if graph is None:
+        # A short run starts on a queue that is already busy: a graph of DIRECT_PRIMING untimed
+        # launches goes out right before the first event with no synchronisation in between, and the
+        # host issues the timed launches while the device works through it (a direct launch costs
+        # the host about as long as the kernel runs, so launches issued one by one onto an idle
+        # queue would be timed at the host's pace).  The timed launches then follow each other back
+        # to back on the device, as they do in the replayed graphs of a long run.
+        priming.launch(stream)
     t0 = time.perf_counter()
     e0.record(stream)
     if graph is None:
         for i in range(steps):
-            launch(i)
+            launch(DIRECT_PRIMING + i)
     else:
         for _ in range(steps // graph_len):
             graph.launch(stream)
@@ -131,7 +163,7 @@ def bench_gemv(ln, hiprt, fmt, n, k, steps, warmup, n_buffers, seed=1, graph_rot
     hiprt.device_synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     event_ms = e0.elapsed_ms(e1)
-    for g in (graph, rest):
+    for g in (graph, rest, priming):
         if g is not None:
             g.destroy()
     result = y.numpy()
@@ -139,6 +171,9 @@ def bench_gemv(ln, hiprt, fmt, n, k, steps, warmup, n_buffers, seed=1, graph_rot
     for w in weights:
         w.free()
     stream.destroy()
+    bench_gemv.last_mode = (f"graphs of {graph_len} launches replayed" if graph_len else
+                            f"launched directly behind a graph of {DIRECT_PRIMING} untimed launches on the same "
+                            f"stream (no synchronisation between it and the timed ones)")
     return event_ms / steps, wall_ms / steps
 
 
@@ -156,6 +191,9 @@ def traffic_probe(ln, launches=8, n_elems=16 * 1024 * 1024):
     dst.free()
     log(f"[bench] traffic probe: {launches} launches of unary_kernel<float>, {4 * n_elems} B read + "
         f"{4 * n_elems} B written each")
+
+
+DIRECT_PRIMING = 64  # untimed launches (one graph) queued right before a directly launched (short) timed run
 
 
 FP16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 matrix rate
@@ -428,13 +466,18 @@ ORACLE_TENSOR_IDS = {"token_embd": 0, "output": 1, "attn_q": 2, "attn_k": 3, "at
                      "ffn_gate": 6, "ffn_up": 7, "ffn_down": 8, "output_norm": 9, "attn_norm": 10, "ffn_norm": 11}
 
 
-def cpu_decode_rate(cfg, tensors, prompt, steps=4):
-    """Tokens per second of the CPU checker's decoder on the same model (all cores, rows
-    dequantised on the fly; the reference's own interpreter is single-threaded on f32 weights
-    dequantised at lowering): `steps` single-token evaluations behind a two-token prompt."""
+FIXTURE_7B = os.path.join(ROOT, "tests", "golden", "llama7b_q4_0_tokens.json")
+
+
+def cpu_decode_rate(cfg, tensors, prompt, steps, threads):
+    """Tokens per second of the CPU checker's decoder on the same model: `steps` single-token
+    evaluations behind a one-token prompt, on `threads` threads.  One thread is the reference's
+    case (its Interpreter and DeviceTraits<CPU> are single-threaded,
+    src/LiteNN/Runtime/Interpreter.h:89-104, src/LiteNN/Device.h:645-658); the checker dequantises
+    each row on the fly where the reference multiplies f32 weights dequantised at lowering, the same
+    f32 sequence per output."""
     from oracle import oracle as orc
-    cores = os.cpu_count() or 1
-    orc.set_threads(cores)
+    orc.set_threads(threads)
     m = orc.LLaMA(cfg.block_count, cfg.embedding_length, cfg.head_count, cfg.head_count_kv, cfg.feed_forward_length,
                   cfg.vocab, cfg.context_length, rms_eps=cfg.rms_eps, rope_base=cfg.rope_freq_base,
                   rope_freq_scale=cfg.rope_freq_scale, rope_dims=cfg.rope_dimension_count, kv_f16=True)
@@ -445,16 +488,37 @@ def cpu_decode_rate(cfg, tensors, prompt, steps=4):
     for _ in range(steps):
         logits = m.eval([int(np.argmax(logits))], all_logits=False)
     dt = time.perf_counter() - t0
-    return steps / dt, cores
+    return steps / dt
+
+
+def fixture_7b(n_prompt, n_new):
+    """The committed token fixture of the 7B-shape run (written from the CPU checker by
+    tests/golden/make_llama7b_tokens.py; data, not code), when it covers these lengths."""
+    try:
+        with open(FIXTURE_7B) as f:
+            fx = json.load(f)
+    except OSError:
+        return None
+    if not fx.get("complete") or fx["prompt_length"] != n_prompt or fx["new_tokens"] < n_new:
+        return None
+    return fx
 
 
 def bench_decode(ln, n_prompt=128, n_new=256, seed=4, model_name="7b", cpu_steps=0):
     from litenn_amd import synth
     from litenn_amd.formats import DT_F16
+    fx = None
     if model_name == "8b":
         cfg = synth.llama_8b_gqa_mixed(context_length=max(4096, n_prompt + n_new))
     else:
         cfg = synth.llama_7b_q4_0(context_length=n_prompt + n_new)
+        fx = fixture_7b(n_prompt, n_new)
+    prompt_seed = seed
+    if fx is not None and fx["model"] == cfg.name and fx["context_length"] == cfg.context_length:
+        # the model and the prompt of the fixture, so that the timed run's tokens can be held to it
+        seed, prompt_seed = fx["seed"], fx["prompt_seed"]
+    else:
+        fx = None
     t0 = time.perf_counter()
     model = ln.LLaMA.from_config(cfg, kv_dtype=DT_F16)
     tensors = []
@@ -463,7 +527,7 @@ def bench_decode(ln, n_prompt=128, n_new=256, seed=4, model_name="7b", cpu_steps
         if cpu_steps:
             tensors.append(item)
     log(f"[bench] {cfg.name} resident after {time.perf_counter() - t0:.1f} s")
-    prompt = synth.prompt_tokens(cfg, n_prompt, seed)
+    prompt = synth.prompt_tokens(cfg, n_prompt, prompt_seed)
     model.generate(prompt, 8, precise=False)  # warm-up: captures the step graph
     model.reset()
     # prompt pass on the matrix cores (fp16 operands), then the captured single-token step
@@ -472,27 +536,52 @@ def bench_decode(ln, n_prompt=128, n_new=256, seed=4, model_name="7b", cpu_steps
     weight_bytes = cfg.matmul_weight_bytes_per_token()
     kv_bytes_mean = 2 * cfg.block_count * cfg.head_count_kv * cfg.head_dim * 2 * (n_prompt + n_new / 2)
     tok_s = steps / (decode_ms / 1e3)
-    model.close()
     out = {
         "workload": f"{cfg.name}: prompt {n_prompt} + {n_new} greedy tokens, context {cfg.context_length}, "
-                    f"fp16 KV cache, f32 activations",
+                    f"fp16 KV cache, f32 activations, model seed {seed}, prompt seed {prompt_seed}",
         "tokens_per_s": round(tok_s, 2),
         "ms_per_token": round(decode_ms / steps, 4),
         "prefill_ms": round(prefill_ms, 3),
         "prefill_tokens_per_s": round(n_prompt / (prefill_ms / 1e3), 1),
+        "prompt_pass": "matrix cores, Float16 operands (flags = 0, the C ABI's default)",
         "weight_bytes_per_token": weight_bytes,
         "roofline_tokens_per_s": round(HBM_PEAK_GBPS * 1e9 / (weight_bytes + kv_bytes_mean), 1),
         "frac_of_hbm_roofline": round(tok_s * (weight_bytes + kv_bytes_mean) / (HBM_PEAK_GBPS * 1e9), 4),
         "distinct_tokens": int(len(set(tokens.tolist()))),
         "first_tokens": tokens[:8].tolist(),
     }
+    if fx is not None:
+        want = np.array(fx["tokens"][:n_new])
+        same = tokens == want
+        first_off = int(np.argmin(same)) if not same.all() else n_new
+        out["tokens_matching_fixture"] = int(same.sum())
+        out["fixture"] = {"file": os.path.relpath(FIXTURE_7B, ROOT), "tokens": int(n_new),
+                          "matching": int(same.sum()), "matching_prefix": first_off,
+                          "source": fx.get("source"),
+                          "note": "the timed run's tokens against the CPU checker's; its prompt pass has Float16 "
+                                  "operands, the fixture's Float32 ones"}
+        if first_off < n_new:
+            out["fixture"]["checker_margin_at_first_difference"] = fx["margins"][first_off]
+        # the same generation behind the Float32-operand prompt pass (untimed): the path the reference's
+        # arithmetic is restated on
+        model.reset()
+        exact, _, _ = model.generate(prompt, n_new, precise=True)
+        out["fixture"]["matching_with_f32_prompt_pass"] = int((exact == want).sum())
+        log(f"[bench] tokens matching the committed fixture: {out['tokens_matching_fixture']} of {n_new} "
+            f"(Float32 prompt pass: {out['fixture']['matching_with_f32_prompt_pass']})")
+    model.close()
     if cpu_steps:
-        rate, cores = cpu_decode_rate(cfg, tensors, prompt, cpu_steps)
-        out["cpu_tokens_per_s"] = round(rate, 3)
-        out["cpu_baseline"] = {"value": round(rate, 3), "unit": "tokens/s", "cores": cores,
-                               "kind": "port-omp (not the reference)",
-                               "sample": f"{cpu_steps} single-token steps of the CPU checker's decoder on the same "
-                                         f"model, rows dequantised on the fly, {cores} threads"}
+        cores = os.cpu_count() or 1
+        rate_all = cpu_decode_rate(cfg, tensors, prompt, cpu_steps, cores)
+        rate_one = cpu_decode_rate(cfg, tensors, prompt, max(1, cpu_steps // 2), 1)
+        out["cpu_tokens_per_s"] = round(rate_one, 4)
+        out["cpu_baseline"] = {"value": round(rate_one, 4), "unit": "tokens/s", "cores": 1, "kind": "port",
+                               "sample": f"{max(1, cpu_steps // 2)} single-token steps of the CPU checker's decoder on "
+                                         f"the same model on one thread (the reference's interpreter is "
+                                         f"single-threaded), rows dequantised on the fly",
+                               "all_cores": {"value": round(rate_all, 3), "unit": "tokens/s", "cores": cores,
+                                             "kind": "port-omp (not the reference)",
+                                             "sample": f"{cpu_steps} steps of the same decoder on {cores} threads"}}
     return out
 
 
@@ -566,6 +655,9 @@ def main() -> int:
     ms_event, ms_wall = bench_gemv(ln, hiprt, Q4_K, n, k, args.steps, args.warmup, args.buffers,
                                    graph_rotations=max(1, args.graph_rotations))
     gbps = algo_bytes / (ms_event * 1e-3) / 1e9
+    launch_mode = bench_gemv.last_mode
+    launched = last_gemv_launch()
+    log(f"[bench] kernel: {launched}")
     log(f"[bench] Q4_K GEMV {n}x{k}: {ms_event * 1e3:.2f} us/launch (events), {ms_wall * 1e3:.2f} us (wall), "
         f"{gbps:.0f} GB/s = {100 * gbps / HBM_PEAK_GBPS:.1f}% of HBM peak")
 
@@ -584,7 +676,8 @@ def main() -> int:
         "data": "synthetic",
         "config": {
             "workload": f"Q4_K GEMV W[{n}x{k}] . x[{k}], batch 1, {args.buffers} rotating weight buffers "
-                        f"({args.buffers * n * row_bytes(Q4_K, k) / 1e6:.0f} MB), one launch per step",
+                        f"({args.buffers * n * row_bytes(Q4_K, k) / 1e6:.0f} MB), one launch per step, "
+                        f"{launch_mode}",
             "format": "Q4_K", "n": n, "k": k, "batch": 1, "algorithmic_bytes_per_step": algo_bytes,
             "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2),
             "wall_ms_per_step": round(ms_wall, 6),
@@ -593,8 +686,10 @@ def main() -> int:
             "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": measured_traffic_bytes(),
             "traffic_unit": "bytes/launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
+            "traffic_source": traffic_source(),
             "algorithmic_bytes": algo_bytes,
-            "kernel": "gemv_stream_kernel<Q4_KUnit, 2, true, 512>",
+            "kernel": launched.split(" grid ")[0],
+            "launch": launched,
         },
     }
     if args.microbench:
@@ -632,7 +727,8 @@ def main() -> int:
             line["decode"] = bench_decode(ln, args.decode_prompt, args.decode_new, model_name="7b",
                                           cpu_steps=cpu_steps)
             log(f"[bench] decode: {line['decode']['tokens_per_s']} tok/s"
-                + (f" (CPU checker: {line['decode']['cpu_tokens_per_s']} tok/s)" if cpu_steps else ""))
+                + (f" (CPU checker on one thread: {line['decode']['cpu_tokens_per_s']} tok/s, on all cores "
+                   f"{line['decode']['cpu_baseline']['all_cores']['value']})" if cpu_steps else ""))
             if args.decode_model == "both":
                 line["decode_8b"] = bench_decode(ln, 512, 512, model_name="8b")
         if "decode_8b" in line:

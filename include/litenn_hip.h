@@ -135,7 +135,10 @@ int litenn_hip_permute(int dev, void* dst, int dtype, const size_t* src_shape, s
  * from and returned to the device's memory pool in stream order, see below).
  * residual (f32 [m, n]) may be NULL; when given, y = residual + x.W
  * (the Add at tools/gguf/LLaMABuilder.cpp:652-653,661-663).  residual may alias y.
- * m == 1..3 runs the streaming GEMV, row by row.  m >= 4 (with k a multiple of 256) runs on the
+ * m == 1..3 runs the streaming GEMV, row by row (f32 operands).  m >= 4 (with k a multiple of 256;
+ * the threshold was 16 in earlier versions of this library, and a caller that sized a workspace
+ * for 4 <= m < 16 by that rule - zero bytes - must size it with
+ * litenn_hip_mul_mat_q_workspace_bytes now) runs on the
  * matrix cores (the rows padded to a multiple of 16; one padded tile costs about as much as three
  * single-row launches): weights and activations are rounded to fp16 once each (activation rows are first scaled
  * by a power of two into the fp16 range), products accumulate in f32; relative L2 error about
@@ -156,6 +159,12 @@ int litenn_hip_permute(int dev, void* dst, int dtype, const size_t* src_shape, s
 int litenn_hip_mul_mat_q(int dev, int fmt, const void* wq, size_t n, size_t k, const void* x, int x_dtype, size_t m,
                          void* y, const void* residual, unsigned flags, const litenn_hip_exec* opts);
 size_t litenn_hip_mul_mat_q_workspace_bytes(size_t m, size_t k);
+/* Measurement aid, no reference counterpart: writes into out (capacity bytes, always terminated)
+ * which instance of the streaming single-row kernel the calling thread's last m == 1 matmul or
+ * linear group launched and with what geometry, e.g.
+ * "gemv_stream_kernel<Q4_KUnit, 2, true, 512> grid 256 x 512 threads, 83968 B LDS, runs of 8 and 6 rows"
+ * ("none" before the first such launch).  The name is the one a kernel trace shows. */
+int litenn_hip_gemv_last_launch(char* out, size_t capacity);
 int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t n, size_t k, const void* x, int x_dtype, size_t m,
                             void* y, const void* residual, unsigned flags, void* workspace, size_t workspace_bytes,
                             const litenn_hip_exec* opts);
@@ -210,8 +219,8 @@ int litenn_hip_attn_decode(int dev, const void* q, const void* kcache, const voi
  * GPU, held until the process ends) instead of memory allocated and freed by the call.  No
  * counterpart in the reference.  The call allocates nothing, records no memset node, and honours
  * opts->synchronize like every other entry point.  It refuses a launch whose chunks do not fit:
- * a single row (m == 1) is cut into c = min(16, ceil(keys / 64), round(2.2 * sqrt(keys / 64)),
- * ceil(1024 / n_head)) chunks and needs n_head * c * (head_dim + 2) <= 262144 floats, which holds
+ * a single row (m == 1) is cut into c = min(16, max(1, round(2.2 * sqrt(keys / 64))),
+ * ceil(1024 / n_head)) chunks (2 from 30 keys on, 3 at 128, 6 at 512, 16 from 3400 on) and needs n_head * c * (head_dim + 2) <= 262144 floats, which holds
  * for every head_dim <= 128 and, at the 16 chunks of a long cache, e.g. for 48 heads of 256
  * features but not for 64.  Every call on one GPU shares that GPU's array:
  * calls that overlap on one GPU (two streams, two threads) race and must be serialised by the
@@ -252,7 +261,12 @@ typedef struct litenn_hip_attn_ext_opts
  * uses none of the options and goes through litenn_hip_attn_decode / litenn_hip_attn_rows; this
  * entry point is a plain f32 row kernel.  The tanh is (exp(2x) - 1) / (exp(2x) + 1) in f32 as in the
  * reference, NaN once 2x exceeds 88.  Refused: max_bias without a mask (the reference's text), a
- * causal mask that hides every key from the first row. */
+ * causal mask that hides every key from the first row (key_position_offset beyond
+ * query_position_offset; the reference computes a softmax over scores of -1e9 there), more than
+ * 65535 query rows or heads.  Keys hidden by the causal mask are skipped, where the reference adds
+ * -1e9 to their scores (src/LiteNN/Layer/FlashAttnExt.h:169): the same result whenever a row keeps
+ * a visible key whose score is far above -1e9; a user mask that drives every visible key of a row to
+ * about -1e9 or to -inf is outside what the tests pin against the reference. */
 int litenn_hip_flash_attn_ext(int dev, const void* q, const void* k, const void* v, int kv_dtype, size_t m, size_t keys,
                               size_t n_head, size_t n_kv_head, size_t head_dim, const litenn_hip_attn_ext_opts* o,
                               void* out, const litenn_hip_exec* opts);

@@ -5,6 +5,7 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <vector>
 
@@ -17,7 +18,7 @@ namespace litenn_hip
 	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
 	                 const float* residual, void* scratch_halves, float* partial, size_t partial_floats,
 	                 hipStream_t stream);
-	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
+	bool launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
 	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
 	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream);
 	void launch_dequantize(int fmt, const void* wq, size_t rows, size_t k, float* dst, hipStream_t stream);
@@ -120,12 +121,17 @@ namespace litenn_hip
 		return 0;
 	}
 
-	// Device memory a call needs beyond its operands, in stream order: hipMallocAsync takes it from the
-	// device's pool and hipFreeAsync returns it once the work queued before has run, so such a call
-	// neither waits for the stream nor stalls the device the way hipMalloc / hipFree do.  The pool keeps
-	// what was returned (release threshold: everything) for the next call.  Where the stream-ordered
-	// allocator is not available the memory comes from hipMalloc and the call drains the stream before
-	// freeing it; `blocking()` tells the caller which it was.
+	// Device memory a call needs beyond its operands, in stream order: it comes from a memory pool of
+	// the library's own (one per device, created on first use) through hipMallocFromPoolAsync, and
+	// hipFreeAsync returns it once the work queued before has run, so such a call neither waits for the
+	// stream nor stalls the device the way hipMalloc / hipFree do.  The pool keeps up to
+	// kScratchPoolKeepBytes of what was returned for the next call and hands the rest back to the
+	// device at the next synchronisation; the device's default pool, which other users of
+	// hipMallocAsync in the process share, is left as it is.  A stream that is being captured gets no
+	// allocation (the caller passes a workspace there).  Where the stream-ordered allocator is not
+	// available the memory comes from hipMalloc and the call drains the stream before freeing it;
+	// `blocking()` tells the caller which it was.
+	constexpr unsigned long long kScratchPoolKeepBytes = 256ull << 20;
 	class StreamScratch
 	{
 	public:
@@ -151,9 +157,17 @@ namespace litenn_hip
 		hipError_t allocate(size_t bytes)
 		{
 			static const bool use_pool = env_int("LITENN_HIP_STREAM_ORDERED_SCRATCH", 1) != 0;
-			if (use_pool && pool_ready())
+			hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+			if (stream_ && hipStreamIsCapturing(stream_, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone)
 			{
-				if (hipMallocAsync(&ptr_, bytes ? bytes : 1, stream_) == hipSuccess)
+				// neither an allocation node in the caller's graph nor a hipMalloc under capture
+				return hipErrorStreamCaptureUnsupported;
+			}
+			(void)hipGetLastError();
+			hipMemPool_t pool = use_pool ? scratch_pool() : nullptr;
+			if (pool)
+			{
+				if (hipMallocFromPoolAsync(&ptr_, bytes ? bytes : 1, pool, stream_) == hipSuccess)
 				{
 					async_ = true;
 					return hipSuccess;
@@ -168,39 +182,45 @@ namespace litenn_hip
 		bool blocking() const { return ptr_ && !async_; }
 
 	private:
-		// once per device: the default pool keeps freed memory instead of handing it back at every
-		// synchronisation
-		static bool pool_ready()
+		// the library's pool of the current device, created on first use; null where the device has no
+		// stream-ordered allocator
+		static hipMemPool_t scratch_pool()
 		{
 			static std::mutex mutex;
-			static std::set<int> ready, refused;
+			static std::map<int, hipMemPool_t> pools; // a null entry: refused once, not tried again
 			int dev = 0;
 			if (hipGetDevice(&dev) != hipSuccess)
 			{
-				return false;
+				return nullptr;
 			}
 			std::lock_guard<std::mutex> lock(mutex);
-			if (ready.count(dev))
+			const auto found = pools.find(dev);
+			if (found != pools.end())
 			{
-				return true;
-			}
-			if (refused.count(dev))
-			{
-				return false;
+				return found->second;
 			}
 			int supported = 0;
 			hipMemPool_t pool = nullptr;
-			unsigned long long keep = ~0ull;
-			if (hipDeviceGetAttribute(&supported, hipDeviceAttributeMemoryPoolsSupported, dev) == hipSuccess && supported &&
-			    hipDeviceGetDefaultMemPool(&pool, dev) == hipSuccess &&
-			    hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep) == hipSuccess)
+			hipMemPoolProps props{};
+			props.allocType = hipMemAllocationTypePinned;
+			props.handleTypes = hipMemHandleTypeNone;
+			props.location.type = hipMemLocationTypeDevice;
+			props.location.id = dev;
+			unsigned long long keep = kScratchPoolKeepBytes;
+			if (hipDeviceGetAttribute(&supported, hipDeviceAttributeMemoryPoolsSupported, dev) != hipSuccess || !supported ||
+			    hipMemPoolCreate(&pool, &props) != hipSuccess)
 			{
-				ready.insert(dev);
-				return true;
+				(void)hipGetLastError();
+				pool = nullptr;
 			}
-			(void)hipGetLastError();
-			refused.insert(dev);
-			return false;
+			else if (hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep) != hipSuccess)
+			{
+				(void)hipGetLastError();
+				(void)hipMemPoolDestroy(pool);
+				pool = nullptr;
+			}
+			pools[dev] = pool;
+			return pool;
 		}
 		void* ptr_ = nullptr;
 		hipStream_t stream_ = nullptr;
@@ -892,14 +912,20 @@ extern "C" int litenn_hip_linear_group(int dev, int fmt, size_t count, const voi
 	}
 	GUARD(action, dev);
 	hipStream_t s = stream_of(opts);
-	// scratch for the composed form, taken and returned in stream order
+	// the single-launch form needs no memory of its own; the composed form takes its scratch from the
+	// library's pool and returns it in stream order
 	StreamScratch scratch_mem(s);
-	const size_t scratch_floats = k + 2 * n[0];
-	LITENN_HIP_TRY(action, scratch_mem.allocate(sizeof(float) * scratch_floats));
-	float* scratch = static_cast<float*>(scratch_mem.get());
-	launch_linear_group(fmt, static_cast<int>(count), wq, ys, n, k, static_cast<const float*>(x),
-	                    static_cast<const float*>(residual), static_cast<const float*>(norm_w), eps, silu, scratch,
-	                    scratch + k, scratch + k + n[0], s);
+	if (!launch_linear_group(fmt, static_cast<int>(count), wq, ys, n, k, static_cast<const float*>(x),
+	                         static_cast<const float*>(residual), static_cast<const float*>(norm_w), eps, silu, nullptr,
+	                         nullptr, nullptr, s))
+	{
+		const size_t scratch_floats = k + 2 * n[0];
+		LITENN_HIP_TRY(action, scratch_mem.allocate(sizeof(float) * scratch_floats));
+		float* scratch = static_cast<float*>(scratch_mem.get());
+		launch_linear_group(fmt, static_cast<int>(count), wq, ys, n, k, static_cast<const float*>(x),
+		                    static_cast<const float*>(residual), static_cast<const float*>(norm_w), eps, silu, scratch,
+		                    scratch + k, scratch + k + n[0], s);
+	}
 	return finish_with(scratch_mem, action, opts);
 }
 

@@ -26,7 +26,9 @@
 #include <type_traits>
 
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
+#include <cstring>
 
 namespace litenn_hip
 {
@@ -1523,46 +1525,98 @@ namespace litenn_hip
 			return cus;
 		}
 
+		// What the calling thread's last streaming launch was (litenn_hip_gemv_last_launch formats it)
+		struct StreamLaunchRecord
+		{
+			const char* kernel = nullptr; // gemv_stream_kernel or gemv_stream_pair_kernel
+			const char* unit0 = "";
+			const char* unit1 = "";
+			int xp = 0, whole = 0, instance_threads = 0;
+			int blocks = 0, threads = 0, rows = 0, run_diff = 0;
+			size_t lds = 0;
+		};
+		thread_local StreamLaunchRecord t_last_stream_launch;
+
+		template <typename U> constexpr const char* unit_name() { return "Unit"; }
+		template <> constexpr const char* unit_name<Q4_0Unit>() { return "Q4_0Unit"; }
+		template <> constexpr const char* unit_name<Q4_1Unit>() { return "Q4_1Unit"; }
+		template <> constexpr const char* unit_name<Q5_0Unit>() { return "Q5_0Unit"; }
+		template <> constexpr const char* unit_name<Q5_1Unit>() { return "Q5_1Unit"; }
+		template <> constexpr const char* unit_name<Q8_0Unit>() { return "Q8_0Unit"; }
+		template <> constexpr const char* unit_name<Q2_KUnit>() { return "Q2_KUnit"; }
+		template <> constexpr const char* unit_name<Q3_KUnit>() { return "Q3_KUnit"; }
+		template <> constexpr const char* unit_name<Q4_KUnit>() { return "Q4_KUnit"; }
+		template <> constexpr const char* unit_name<Q5_KUnit>() { return "Q5_KUnit"; }
+		template <> constexpr const char* unit_name<Q6_KUnit>() { return "Q6_KUnit"; }
+
+		template <typename U0, typename U1>
+		void record_stream_launch(const char* kernel, int xp, bool whole, int instance_threads, const GemvLaunch& launch,
+		                          int blocks, int threads, size_t lds)
+		{
+			StreamLaunchRecord& r = t_last_stream_launch;
+			r.kernel = kernel;
+			r.unit0 = unit_name<U0>();
+			r.unit1 = unit_name<U1>();
+			r.xp = xp;
+			r.whole = whole ? 1 : 0;
+			r.instance_threads = instance_threads;
+			r.blocks = blocks;
+			r.threads = threads;
+			r.rows = launch.part[0].rows_per_group;
+			r.run_diff = launch.part[0].run_diff;
+			r.lds = lds;
+		}
+
+		// Returns false, with nothing launched, when no instance of the kernel was compiled for the
+		// geometry (the caller then takes the register kernel).
 		template <typename U0, typename U1, int XP>
-		void launch_stream_variant(const GemvLaunch& launch, int blocks, int threads, size_t lds, hipStream_t stream)
+		bool launch_stream_variant(const GemvLaunch& launch, int blocks, int threads, size_t lds, hipStream_t stream)
 		{
 			if constexpr (std::is_same<U0, U1>::value)
 			{
+				const GemvArgs& g = launch.part[0];
 				// K = 4096 is most of a decoder's launches: its own instance with the slice geometry folded
-				if (XP == 2 && launch.part[0].k == 4096)
+				if (XP == 2 && g.k == 4096 && threads == 512)
 				{
 					allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, 2, true>), kStreamLdsLimit);
-					{
-						const GemvArgs& g = launch.part[0];
-						gemv_stream_kernel<U0, 2, true><<<dim3(blocks), dim3(threads), lds, stream>>>(g.x, g.k, g.w[0], g.row_bytes,
-						                                                                         g.rows_per_group, g.n_total, g);
-					}
+					gemv_stream_kernel<U0, 2, true><<<dim3(blocks), dim3(threads), lds, stream>>>(g.x, g.k, g.w[0], g.row_bytes,
+					                                                                         g.rows_per_group, g.n_total, g);
+					record_stream_launch<U0, U1>("gemv_stream_kernel", 2, true, 512, launch, blocks, threads, lds);
+					return true;
 				}
-				else if (threads > 512)
+				if (threads > 512)
 				{
 					// twelve wavefronts (three-slice rows): an instance compiled for that many
 					if constexpr (XP == kTwelveXp)
 					{
+						if (threads != 768)
+						{
+							return false;
+						}
 						allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, XP, false, 768>), kStreamLdsLimit);
-						const GemvArgs& g = launch.part[0];
 						gemv_stream_kernel<U0, XP, false, 768><<<dim3(blocks), dim3(threads), lds, stream>>>(
 						    g.x, g.k, g.w[0], g.row_bytes, g.rows_per_group, g.n_total, g);
+						record_stream_launch<U0, U1>("gemv_stream_kernel", XP, false, 768, launch, blocks, threads, lds);
+						return true;
 					}
+					return false;
 				}
-				else
-				{
-					allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, XP, false>), kStreamLdsLimit);
-					{
-						const GemvArgs& g = launch.part[0];
-						gemv_stream_kernel<U0, XP, false><<<dim3(blocks), dim3(threads), lds, stream>>>(g.x, g.k, g.w[0], g.row_bytes,
-						                                                                         g.rows_per_group, g.n_total, g);
-					}
-				}
+				allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_kernel<U0, XP, false>), kStreamLdsLimit);
+				gemv_stream_kernel<U0, XP, false><<<dim3(blocks), dim3(threads), lds, stream>>>(g.x, g.k, g.w[0], g.row_bytes,
+				                                                                         g.rows_per_group, g.n_total, g);
+				record_stream_launch<U0, U1>("gemv_stream_kernel", XP, false, 512, launch, blocks, threads, lds);
+				return true;
 			}
 			else
 			{
+				if (threads > 512)
+				{
+					return false;
+				}
 				allow_dynamic_lds(reinterpret_cast<const void*>(&gemv_stream_pair_kernel<U0, U1, XP>), kStreamLdsLimit);
 				gemv_stream_pair_kernel<U0, U1, XP><<<dim3(blocks), dim3(threads), lds, stream>>>(launch);
+				record_stream_launch<U0, U1>("gemv_stream_pair_kernel", XP, false, 512, launch, blocks, threads, lds);
+				return true;
 			}
 		}
 
@@ -1676,23 +1730,20 @@ namespace litenn_hip
 		}
 
 		template <typename U0, typename U1>
-		void launch_stream_xp(const GemvLaunch& launch, int blocks, size_t lds, hipStream_t stream)
+		bool launch_stream_xp(const GemvLaunch& launch, int blocks, size_t lds, hipStream_t stream)
 		{
 			const GemvArgs& a = launch.part[0];
 			const int threads = 64 * a.slices * a.groups;
 			const int per_thread = (a.k / 4 + threads - 1) / threads; // 128-bit activation loads per thread
 			if (per_thread <= 2)
 			{
-				launch_stream_variant<U0, U1, 2>(launch, blocks, threads, lds, stream);
+				return launch_stream_variant<U0, U1, 2>(launch, blocks, threads, lds, stream);
 			}
-			else if (per_thread <= 4)
+			if (per_thread <= 4)
 			{
-				launch_stream_variant<U0, U1, 4>(launch, blocks, threads, lds, stream);
+				return launch_stream_variant<U0, U1, 4>(launch, blocks, threads, lds, stream);
 			}
-			else
-			{
-				launch_stream_variant<U0, U1, kXPerThread>(launch, blocks, threads, lds, stream);
-			}
+			return launch_stream_variant<U0, U1, kXPerThread>(launch, blocks, threads, lds, stream);
 		}
 
 		template <typename U>
@@ -1707,8 +1758,7 @@ namespace litenn_hip
 			GemvLaunch launch{};
 			launch.part[0] = a;
 			launch.blocks0 = blocks;
-			launch_stream_xp<U, U>(launch, blocks, exclusive_lds(lds), stream);
-			return true;
+			return launch_stream_xp<U, U>(launch, blocks, exclusive_lds(lds), stream);
 		}
 
 		// Two parts of different block formats over the same activations in one launch.  The CUs are
@@ -1748,8 +1798,7 @@ namespace litenn_hip
 			launch.part[0] = a0;
 			launch.part[1] = a1;
 			launch.blocks0 = blocks0;
-			launch_stream_xp<U0, U1>(launch, blocks0 + blocks1, exclusive_lds(std::max(lds0, lds1)), stream);
-			return true;
+			return launch_stream_xp<U0, U1>(launch, blocks0 + blocks1, exclusive_lds(std::max(lds0, lds1)), stream);
 		}
 
 		template <typename U>
@@ -1987,14 +2036,20 @@ namespace litenn_hip
 	// residual (optional): one fused launch when the streaming kernel takes the shape, otherwise the
 	// same operators from separate launches.  scratch_x holds k floats (used when norm_w is given and
 	// the fused kernel is not applicable); scratch_gate / scratch_up hold n[0] floats (same, SwiGLU).
-	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
+	// Returns false, with nothing launched, when the group needs the composed form and no scratch
+	// was handed over (scratch_x null): the caller allocates k + 2 n[0] floats and calls again.
+	bool launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
 	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
 	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream)
 	{
 		static const int fuse = env_int("LITENN_HIP_FUSE", 1);
 		if (fuse && launch_gemv_fused(fmt, count, w, y, n, k, x, residual, norm_w, eps, silu_mul, stream))
 		{
-			return;
+			return true;
+		}
+		if (!scratch_x && (norm_w || silu_mul))
+		{
+			return false;
 		}
 		const float* xin = x;
 		if (norm_w)
@@ -2007,12 +2062,13 @@ namespace litenn_hip
 			launch_gemv(fmt, w[0], n[0], k, xin, 1, scratch_gate, nullptr, stream);
 			launch_gemv(fmt, w[1], n[1], k, xin, 1, scratch_up, nullptr, stream);
 			launch_silu_mul(scratch_gate, scratch_up, y[0], n[0], stream);
-			return;
+			return true;
 		}
 		for (int m = 0; m < count; ++m)
 		{
 			launch_gemv(fmt, w[m], n[m], k, xin, 1, y[m], m == 0 ? residual : nullptr, stream);
 		}
+		return true;
 	}
 
 	void launch_dequantize(int fmt, const void* wq, size_t rows, size_t k, float* dst, hipStream_t stream)
@@ -2029,6 +2085,34 @@ namespace litenn_hip
 		                                                          row_bytes(fmt, k), ids, out, err_flag);
 	}
 } // namespace litenn_hip
+
+extern "C" int litenn_hip_gemv_last_launch(char* out, size_t capacity)
+{
+	using namespace litenn_hip;
+	if (!out || capacity == 0)
+	{
+		return fail("describe the last GEMV launch", "destination is null or empty");
+	}
+	const StreamLaunchRecord& r = t_last_stream_launch;
+	if (!r.kernel)
+	{
+		std::snprintf(out, capacity, "none");
+		return 0;
+	}
+	char name[160];
+	if (std::strcmp(r.unit0, r.unit1) == 0)
+	{
+		std::snprintf(name, sizeof name, "%s<%s, %d, %s, %d>", r.kernel, r.unit0, r.xp, r.whole ? "true" : "false",
+		              r.instance_threads);
+	}
+	else
+	{
+		std::snprintf(name, sizeof name, "%s<%s, %s, %d>", r.kernel, r.unit0, r.unit1, r.xp);
+	}
+	std::snprintf(out, capacity, "%s grid %d x %d threads, %zu B LDS, runs of %d and %d rows", name, r.blocks, r.threads,
+	              r.lds, r.rows, r.rows - r.run_diff);
+	return 0;
+}
 
 #ifdef LITENN_GEMV_TRACE
 // Timeline build only: copies the stamps of the last streaming launch to the host

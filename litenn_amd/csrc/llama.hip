@@ -13,6 +13,8 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <exception>
+#include <string>
 #include <vector>
 
 namespace litenn_hip
@@ -32,7 +34,7 @@ namespace litenn_hip
 	bool launch_gemm(int fmt, const void* wq, size_t n, size_t k, const float* x, size_t m, float* y,
 	                 const float* residual, void* scratch_halves, float* partial, size_t partial_floats,
 	                 hipStream_t stream);
-	void launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
+	bool launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
 	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
 	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream);
 	bool launch_gemv_fused_mixed(const int* fmts, int count, const void* const* w, float* const* y, const size_t* n,
@@ -471,7 +473,33 @@ namespace
 	}
 } // namespace
 
+namespace
+{
+	int llama_create_impl(int dev, const litenn_hip_llama_params* params, litenn_hip_llama** out, litenn_hip_llama*& m);
+}
+
 extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* params, litenn_hip_llama** out)
+{
+	// host containers sized by the caller's context length live in the body: an allocation that
+	// fails there must come back as a status, not leave through the C boundary
+	litenn_hip_llama* m = nullptr;
+	try
+	{
+		return llama_create_impl(dev, params, out, m);
+	}
+	catch (const std::exception& ex)
+	{
+		if (m)
+		{
+			litenn_hip_llama_free(m);
+		}
+		return fail(kAction, std::string("host memory for the model's tables: ") + ex.what());
+	}
+}
+
+namespace
+{
+int llama_create_impl(int dev, const litenn_hip_llama_params* params, litenn_hip_llama** out, litenn_hip_llama*& m)
 {
 	if (!params || !out)
 	{
@@ -523,7 +551,7 @@ extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* p
 	{
 		return fail_hip(kAction, guard.error());
 	}
-	auto* m = new litenn_hip_llama();
+	m = new litenn_hip_llama();
 	m->dev = dev;
 	m->p = p;
 	m->p.rope_dimension_count = rope_dims;
@@ -531,6 +559,7 @@ extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* p
 	m->layers.resize(static_cast<size_t>(p.block_count));
 	auto bail = [&](hipError_t e) {
 		litenn_hip_llama_free(m);
+		m = nullptr;
 		return fail_hip(kAction, e);
 	};
 	// Non-blocking: a stream that synchronises with the legacy default stream would, while its
@@ -607,6 +636,7 @@ extern "C" int litenn_hip_llama_create(int dev, const litenn_hip_llama_params* p
 	*out = m;
 	return 0;
 }
+} // namespace
 
 // Hands a device allocation to the model: it is released by litenn_hip_llama_free.  Used by
 // the GGUF loader; not part of the C ABI.

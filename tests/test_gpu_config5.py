@@ -15,9 +15,12 @@ import pytest
 from conftest import rel_l2
 from litenn_amd import synth
 from litenn_amd.formats import DT_F16, DT_F32, Q4_K, Q6_K
-from llama_util import hip_model, oracle_model
+from llama_util import adopt_device_cache, hip_model, oracle_model
 
 pytestmark = pytest.mark.gpu
+
+# a single-token step against the checker once both read the same Float16 cache
+F16_TWIN_TOL = 1e-4
 
 MIXED = {"default": Q4_K, "attn_v": Q6_K, "ffn_down": Q6_K, "output": Q6_K}
 
@@ -33,6 +36,10 @@ def test_8b_gqa_shape_two_blocks_against_checker(hip, oracle):
     # is held to the checker at 1e-4.  With the Float16 cache a key or value within a Float32
     # rounding of a half's midpoint lands on the other half on the device; over 512 keys a few do,
     # and the softmax of this random model turns such a 2^-11 into a few 1e-3 of a step's logits.
+    # That those entries, and nothing else, are the difference is shown by a second checker that is
+    # handed the device's cache before every step (every entry within one half of its own, counted):
+    # its logits agree with the device's as closely as with the Float32 cache (measured: 6e-6 to 1e-5
+    # where the checker on its own cache is 4e-5 to 8e-4 away).
     for kv, tol in ((DT_F32, 1e-4), (DT_F16, 1e-2)):
         ref = oracle_model(oracle, cfg, 11, kv_f16=(kv == DT_F16), tensors=tensors)
         dev = hip_model(hip, cfg, 11, kv_dtype=kv, tensors=tensors)
@@ -42,6 +49,16 @@ def test_8b_gqa_shape_two_blocks_against_checker(hip, oracle):
         print("Float32 prompt pass: %.2e" % rel_l2(got, want), flush=True)
         assert rel_l2(got, want) < tol
         assert int(np.argmax(got)) == int(np.argmax(want))
+        twin = None
+        if kv == DT_F16:
+            # the checker again, from here on reading the device's cache
+            twin = oracle_model(oracle, cfg, 11, kv_f16=True, tensors=tensors)
+            for layer in range(2):
+                twin.set_kv(layer, *ref.get_kv(layer))
+            twin.set_past(512)
+            entries, differing = adopt_device_cache(twin, dev, 2, deeper_slack=1e-2)
+            print("cache after the prompt: %d of %d entries differ" % (differing, entries), flush=True)
+            assert 0 < differing < entries // 4
         tok = int(np.argmax(want))
         fed = []
         for step in range(16):
@@ -49,8 +66,15 @@ def test_8b_gqa_shape_two_blocks_against_checker(hip, oracle):
             w = ref.eval([tok], all_logits=False)
             g = dev.eval([tok], all_logits=False)
             err = rel_l2(g, w)
-            print("step %d: %.2e" % (step, err), flush=True)
             assert err < tol, step
+            if twin is not None:
+                err_twin = rel_l2(g, twin.eval([tok], all_logits=False))
+                entries, differing = adopt_device_cache(twin, dev, 2, deeper_slack=2e-4)
+                print("step %d: %.2e against the checker, %.2e against the checker reading the device's cache "
+                      "(%d entries of its new rows differ)" % (step, err, err_twin, differing), flush=True)
+                assert err_twin < F16_TWIN_TOL, step
+            else:
+                print("step %d: %.2e" % (step, err), flush=True)
             top2 = np.sort(w)[-2:]
             if top2[1] - top2[0] > 4 * tol * np.abs(w).max():
                 assert int(np.argmax(g)) == int(np.argmax(w))

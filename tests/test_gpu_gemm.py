@@ -104,6 +104,32 @@ def test_config3_q6_k_4096x4096(hip, oracle, m):
     assert run_case(hip, oracle, Q6_K, m, 4096, 4096, seed=40 + m, rows=rows) <= TOL
 
 
+@pytest.mark.parametrize("fmt,n", [(Q4_K, 14336), (Q6_K, 4096)])
+def test_config3_bf16_activations_at_full_size(hip, oracle, fmt, n):
+    """BASELINE config 3 names fp32 and bf16 activations: M = 64, K = 4096, both matrices at full size
+    with BFloat16 activations (src/LiteNN/DType.h:17-30), bit-equal to the call on their exact
+    Float32 values and within the bar of the CPU checker on a 768-row sample of N."""
+    from litenn_amd.formats import DT_BF16
+    m, k = 64, 4096
+    wq = synth.quant_weights(fmt, n, k, 50 + n % 7, 1)
+    x = synth.activations(m, k, 51, 2)
+    bits = ((x.view(np.uint32) + 0x8000) >> 16).astype(np.uint16)  # the nearest BFloat16 (no ties to worry about)
+    wide = (bits.astype(np.uint32) << 16).view(np.float32)
+    assert 1e-3 < rel_l2(wide, x) < 4e-3  # really rounded to eight bits
+    w = hip.Tensor.from_numpy(wq)
+    bf = hip.Tensor((m, k), DT_BF16)
+    hip.DeviceTraits.CopyFromCPU(bf.device, DT_BF16, bf.ptr, DT_BF16, bits, bits.size)
+    got = hip.mul_mat_q(fmt, w, n, k, bf).numpy()
+    want = hip.mul_mat_q(fmt, w, n, k, hip.Tensor.from_numpy(wide)).numpy()
+    assert got.shape == (m, n) and np.array_equal(got, want)
+    rows = np.sort(np.random.default_rng(n).choice(n, 768, replace=False))
+    rows[0], rows[-1] = 0, n - 1
+    sub = np.ascontiguousarray(wq.reshape(n, row_bytes(fmt, k))[rows]).reshape(-1)
+    err = rel_l2(got[:, rows], oracle.mul_mat_q(fmt, sub, len(rows), k, wide))
+    print("BFloat16 activations, M=64, %d x %d: %.2e" % (n, k, err), flush=True)
+    assert 1e-6 < err <= TOL
+
+
 @pytest.mark.parametrize("fmt", FORMATS)
 @pytest.mark.parametrize("m,n,k", [(144, 26400, 512),    # 128-row tiles, one row group per wavefront
                                    (130, 52500, 256),    # 128-row tiles, two row groups (nibble formats)

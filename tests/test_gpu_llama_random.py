@@ -8,7 +8,7 @@ import pytest
 from conftest import rel_l2
 from litenn_amd import synth
 from litenn_amd.formats import (DT_F16, DT_F32, Q2_K, Q3_K, Q4_0, Q4_1, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0)
-from llama_util import hip_model, oracle_model
+from llama_util import adopt_device_cache, hip_model, oracle_model
 
 pytestmark = pytest.mark.gpu
 SMALL_BLOCK = [Q4_0, Q4_1, Q5_0, Q5_1, Q8_0]
@@ -46,6 +46,9 @@ def draw_config(rng):
 # in a GPU memory fault: the matrix-core kernel fetched a 16-byte piece lying wholly behind the
 # tensor.  Fixed in the kernel; tests/test_gpu_gemm.py::test_weights_that_end_on_a_page_boundary.
 SEEDS = list(range(64))
+# Float16-cache runs, logits of a piece against the checker: [pieces of several rows, whose own rows'
+# halves may fall either way; single rows behind a cache the checker shares]
+F16_PIECE_TOL = {False: 5e-4, True: 2e-4}  # measured over the 64 cases: at most 1.4e-4 and 7.3e-5
 
 
 @pytest.mark.parametrize("seed", SEEDS)
@@ -64,16 +67,25 @@ def test_random_model_matches_checker(hip, oracle, seed):
     # a prompt pass, single-token steps, then several rows on top of a filled cache
     pieces = [toks[:first], toks[first:first + 1], toks[first + 1:first + 2], toks[first + 2:first + 3],
               toks[first + 3:first + 3 + later]]
+    synced = 0
     for piece in pieces:
         want = ref.eval(piece)
         got = dev.eval(piece)
         # With the Float16 cache a key or value that lands within an f32 rounding of a half's
         # midpoint rounds the other way on the device (one unit of a half, 5e-4 relative, on a few
-        # elements per thousand), and a random block amplifies such a difference several times: the
-        # Float32-cache cases carry the sharp bar, the Float16 ones the rounding-tolerant one.
+        # elements per thousand), and a random block amplifies such a difference several times.  So
+        # the checker is handed the device's cache after every piece (every entry held to one half
+        # of its own first): a piece then differs from the checker's only by the entries of its own
+        # rows that fell the other way, and single rows carry the Float32 cases' sharp bar.
         err = rel_l2(got, want)
         print("piece of %d rows: %.2e" % (len(piece), err), flush=True)
-        assert err < (2e-3 if kv == DT_F16 else 5e-5), (what, len(piece), dev.past)
+        if kv == DT_F16:
+            assert err < F16_PIECE_TOL[len(piece) == 1 and synced > 0], (what, len(piece), dev.past)
+            entries, differing = adopt_device_cache(ref, dev, cfg.block_count, slack=2e-5, deeper_slack=2e-2)
+            print("  cache: %d of %d entries differ" % (differing, entries), flush=True)
+            synced += 1
+        else:
+            assert err < 5e-5, (what, len(piece), dev.past)
     assert dev.past == ref.past
     kd, vd = dev.get_kv(cfg.block_count - 1)
     kr, vr = ref.get_kv(cfg.block_count - 1)
