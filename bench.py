@@ -417,11 +417,57 @@ def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=8):
     out["mfma_mix_note"] = ("v_mfma_f32_16x16x32_f16 from registers, fragment reads from LDS, independent f32 multiply-adds; "
                             "256 workgroups, shader-clock cycles of the slowest wavefront of a workgroup")
     cyc.free()
+    out["xcd_exchange"] = xcd_exchange(ln, hiprt, tl, ok, stream)
     for w in weights:
         w.free()
     for tns in (x, y, sink):
         tns.free()
     stream.destroy()
+    return out
+
+
+def xcd_exchange(ln, hiprt, tl, ok, stream, phases=2000, blocks=256):
+    """What a phase boundary inside one launch costs when only the workgroups of one XCD (32 CUs that
+    share an L2) have to meet: 256 workgroups, one per CU, each publishing one value per phase and
+    collecting the 32 values of its own XCD (csrc/microbench.hip, mb_xcd_exchange_kernel)."""
+    import ctypes as C
+    vp = C.c_void_p
+    tl.litenn_hip_mb_xcd_exchange.argtypes = [C.c_int] * 5 + [vp] * 5
+    mem, err = ln.Tensor((2048 + 512 * phases,)), ln.Tensor((4,))
+    result, stamps = ln.Tensor((2 * blocks,)), ln.Tensor((2 * phases,))
+    want = 1
+    for _ in range(phases):
+        want = (32 * want + 1) & 0xFFFFFFFF
+    out = []
+    for mode, name in ((0, "counter in the L2, values loaded past the L1"),
+                       (1, "values carry their phase, polled past the L1"),
+                       (2, "values carry their phase, device-scope loads and stores"),
+                       (3, "a flag per workgroup polled by atomics in the L2, values by ordinary stores and loads"),
+                       (4, "a flag per workgroup polled by device-scope loads, values by ordinary stores and loads")):
+        best = None
+        for rep in range(3):
+            e0, e1 = hiprt.Event(), hiprt.Event()
+            e0.record(stream)
+            ok(tl.litenn_hip_mb_xcd_exchange(mode, blocks, phases, 4000, 32, mem.ptr, err.ptr, result.ptr, stamps.ptr,
+                                              stream.handle))
+            e1.record(stream)
+            stream.synchronize()
+            us = e0.elapsed_ms(e1) * 1e3
+            best = us if best is None else min(best, us)
+        flag = int(err.numpy().view(np.int32)[0])
+        res = result.numpy().view(np.uint32).reshape(blocks, 2)
+        per_xcd = np.bincount(res[:, 1] // 64, minlength=8).tolist()
+        ticks = stamps.numpy().view(np.uint64)[:phases].astype(np.float64)
+        per_phase = float(np.median(np.diff(ticks))) * 0.01
+        entry = {"mode": name, "phases": phases, "us_per_phase": round(best / phases, 3),
+                 "us_per_phase_median_by_clock": round(per_phase, 3), "waits_ran_out": flag,
+                 "workgroups_per_xcd": per_xcd, "values_correct": bool(flag == 0 and np.all(res[:, 0] == want))}
+        out.append(entry)
+        log(f"[bench] microbench: exchange within an XCD, {name}: {entry['us_per_phase']} us per phase "
+            f"(median by the card's clock {entry['us_per_phase_median_by_clock']}), waits that ran out: {flag}, "
+            f"workgroups per XCD {per_xcd}, values correct: {entry['values_correct']}")
+    for t in (mem, err, result, stamps):
+        t.free()
     return out
 
 

@@ -307,6 +307,13 @@ int litenn_hip_llama_set_tensor(litenn_hip_llama* model, int which, int layer, i
                                 size_t k);
 int litenn_hip_llama_reset(litenn_hip_llama* model);
 int litenn_hip_llama_past(const litenn_hip_llama* model);
+/* How the single-token step runs a decoder block's attention half (no reference counterpart): 1 = as
+ * one launch (norm + q/k/v, rotation + append + attention, output projection; models 4096 wide
+ * with 32 heads of 128, a Float16 cache and Q4_0 / Q4_K weights on a card of 256 CUs), -1 = as
+ * separate launches (the shape is another, LITENN_HIP_ATTN_BLOCK=0 was set when the step was first
+ * built, or a bounded wait inside the launch once ran out and the step was repeated), 0 = not yet
+ * decided (no single-token step has run since the model's tensors were set). */
+int litenn_hip_llama_block_form(const litenn_hip_llama* m);
 /* LowerLLaMACausalLMDecode(sequenceLength = m, pastLength = positionOffset = past) executed
  * against the cache the model holds (tools/gguf/LLaMABuilder.cpp:826-872); tokens are host
  * I32.  logits (host f32 [m, vocab]) and last_logits (host f32 [vocab]) may be NULL.

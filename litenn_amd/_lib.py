@@ -87,6 +87,7 @@ SIGNATURES = {
     "litenn_hip_llama_set_tensor": [_vp, _i, _i, _i, _vp, _sz, _sz],
     "litenn_hip_llama_reset": [_vp],
     "litenn_hip_llama_past": [_vp],
+    "litenn_hip_llama_block_form": [_vp],
     "litenn_hip_llama_eval": [_vp, _vp, _sz, _vp, _vp, _u],
     "litenn_hip_llama_generate": [_vp, _vp, _sz, _sz, _vp, _u, C.POINTER(_d), C.POINTER(_d)],
     "litenn_hip_llama_get_kv": [_vp, _i, _vp, _vp],

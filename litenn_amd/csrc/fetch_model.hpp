@@ -135,6 +135,49 @@ namespace litenn_hip
 		// every load)
 		LITENN_FETCH_FN int stream_x_index(int tid, int j, int threads, int k) { return imin((tid + j * threads) * 4, k - 4); }
 
+		// ---- decoder-block kernel: rows dealt out per XCD, and the output projection's columns ---
+		// The launch's 256 workgroups form eight teams of 32 (workgroup b: team b % 8, place b / 8;
+		// the dispatcher deals workgroups to the card's eight XCDs in that order, so a team shares
+		// an L2).  Team t takes an eighth of the rows of each of the up to three matrices of the
+		// first phase: virtual row v of the team lies in matrix m at row t * (n[m] / 8) + r.
+		struct TeamRow
+		{
+			int m, local;
+		};
+		LITENN_FETCH_FN TeamRow team_row(int v, int team, int n0, int n1, int n2)
+		{
+			const int r0 = n0 >> 3, r1 = n1 >> 3, r2 = n2 >> 3;
+			if (v < r0)
+			{
+				return { 0, team * r0 + v };
+			}
+			if (v < r0 + r1)
+			{
+				return { 1, team * r1 + (v - r0) };
+			}
+			return { 2, team * r2 + imin(v - r0 - r1, r2 > 0 ? r2 - 1 : 0) };
+		}
+
+		// The third phase multiplies a column slice of the output projection: team t owns `seg_bytes`
+		// bytes of every row (the blocks of its heads' columns), from byte t * seg_bytes of the row.
+		// A wavefront fetches the segments of `rows_per_fetch` consecutive rows (4096 weights in all)
+		// as one run of 16-byte pieces, piece p of the run being piece p % seg_pieces of row
+		// p / seg_pieces; load instruction i moves pieces 64 i .. 64 i + 63 to consecutive LDS
+		// addresses, so the slot holds what a 4096-wide slice of a row would.
+		struct SegmentPiece
+		{
+			int row;         // 0 .. rows_per_fetch - 1
+			uint32_t offset; // from the segment's first byte
+			bool issued;
+		};
+		LITENN_FETCH_FN SegmentPiece segment_piece(int i, int lane, int seg_pieces, int rows_per_fetch)
+		{
+			const int total = seg_pieces * rows_per_fetch;
+			const int p = 64 * i + lane;
+			const int q = imin(p, total - 1);
+			return { q / seg_pieces, static_cast<uint32_t>(q % seg_pieces) * 16u, p < total };
+		}
+
 		// ---- tiled prompt attention: key / value rows of a 64-key tile -------------------------
 		// keys any query row of the 64-row tile starting at q_first may see
 		LITENN_FETCH_FN int attn_tile_kv_len(int past, int q_first, int q_tile, int m)

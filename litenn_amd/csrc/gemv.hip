@@ -21,6 +21,7 @@
 //   * quants enter the FMA as binary16 subnormals (value * 2^-24), so no int->float conversion
 //     is issued: a mask produces the operand of v_fma_mix_f32.
 #include "common.hpp"
+#include "attn_math.hpp"
 #include "fetch_model.hpp"
 
 #include <type_traits>
@@ -993,8 +994,20 @@ namespace litenn_hip
 	{                                                                                                                  \
 		g_trace[(blockIdx.x * 8 + wave) % kTraceWaves * kTraceSlots + (slot)] = __builtin_amdgcn_s_memrealtime();      \
 	}
+		// the decoder-block kernel's own points (attn_block.inc): 0 entry, 1 first phase's rows stored,
+		// 2 first meeting passed, 3 second phase's triple stored, 4 second meeting passed, 5 activations
+		// of the third phase in registers, 6 end
+		constexpr int kBlockTraceSlots = 8;
+		__device__ unsigned long long g_block_trace[kTraceWaves * kBlockTraceSlots];
+#define BLOCK_TRACE(slot)                                                                                              \
+	if (lane == 0)                                                                                                     \
+	{                                                                                                                  \
+		g_block_trace[(blockIdx.x * 8 + wave) % kTraceWaves * kBlockTraceSlots + (slot)] =                             \
+		    __builtin_amdgcn_s_memrealtime();                                                                          \
+	}
 #else
 #define GEMV_TRACE(slot)
+#define BLOCK_TRACE(slot)
 #endif
 
 		// ------------------------------------------------------------------
@@ -1038,7 +1051,16 @@ namespace litenn_hip
 			int rows_per_group;    // consecutive rows a wavefront group of the first half walks (<= 64)
 			int run_diff;          // the groups of the second half walk this many rows fewer
 			int silu_mul;          // 1: w[0] = gate, w[1] = up, row 2i + m; y[0][i] = silu(gate_i) * up_i
+			// kBlockTeams vectors, partial_stride floats apart, that the decoder-block kernel left in place
+			// of the attention half's result: added, in team order, onto x while it is staged
+			// (partials_on == 1; K = 4096 only) or onto the residual in the epilogue (partials_on == 2)
+			const float* partials;
+			uint32_t partial_stride;
+			int partials_on;
 		};
+
+		// teams of the decoder-block kernel (the card's XCDs)
+		constexpr int kBlockTeams = 8;
 
 		__device__ __forceinline__ void locate_row(const GemvArgs& a, int vr, int& m, int& local)
 		{
@@ -1168,6 +1190,10 @@ namespace litenn_hip
 			const int block = static_cast<int>(blockIdx.x);
 			constexpr bool kWholeSlices = WHOLE;
 			constexpr bool kEarlyActivations = true;
+			constexpr bool kTeamRows = false;
+			constexpr int team = 0;
+			constexpr int kTeamExtraLoads = 0;
+			const auto team_prefetch = [] {};
 #include "gemv_stream_body.inc"
 		}
 
@@ -1176,6 +1202,10 @@ namespace litenn_hip
 		{
 			constexpr bool kWholeSlices = false;
 			constexpr bool kEarlyActivations = false;
+			constexpr bool kTeamRows = false;
+			constexpr int team = 0;
+			constexpr int kTeamExtraLoads = 0;
+			const auto team_prefetch = [] {};
 #include "gemv_stream_body.inc"
 		}
 
@@ -1747,13 +1777,17 @@ namespace litenn_hip
 		}
 
 		template <typename U>
-		bool launch_stream(GemvArgs a, hipStream_t stream)
+		bool launch_stream(GemvArgs a, hipStream_t stream, bool plan_only = false)
 		{
 			int blocks = 0;
 			size_t lds = 0;
 			if (!plan_stream<U>(a, compute_units(), blocks, lds, true))
 			{
 				return false;
+			}
+			if (plan_only)
+			{
+				return true;
 			}
 			GemvLaunch launch{};
 			launch.part[0] = a;
@@ -1828,7 +1862,7 @@ namespace litenn_hip
 			       fmt == LITENN_FMT_Q5_K || fmt == LITENN_FMT_Q6_K;
 		}
 
-		bool stream_dispatch(int fmt, const GemvArgs& a, hipStream_t stream)
+		bool stream_dispatch(int fmt, const GemvArgs& a, hipStream_t stream, bool plan_only = false)
 		{
 			// LITENN_HIP_GEMV_STREAM=0 keeps the rows in registers instead of LDS
 			static const int use_stream = env_int("LITENN_HIP_GEMV_STREAM", 1);
@@ -1838,16 +1872,16 @@ namespace litenn_hip
 			}
 			switch (fmt)
 			{
-			case LITENN_FMT_Q4_0: return launch_stream<Q4_0Unit>(a, stream);
-			case LITENN_FMT_Q4_1: return launch_stream<Q4_1Unit>(a, stream);
-			case LITENN_FMT_Q5_0: return launch_stream<Q5_0Unit>(a, stream);
-			case LITENN_FMT_Q5_1: return launch_stream<Q5_1Unit>(a, stream);
-			case LITENN_FMT_Q8_0: return launch_stream<Q8_0Unit>(a, stream);
-			case LITENN_FMT_Q2_K: return launch_stream<Q2_KUnit>(a, stream);
-			case LITENN_FMT_Q3_K: return launch_stream<Q3_KUnit>(a, stream);
-			case LITENN_FMT_Q4_K: return launch_stream<Q4_KUnit>(a, stream);
-			case LITENN_FMT_Q5_K: return launch_stream<Q5_KUnit>(a, stream);
-			default: return launch_stream<Q6_KUnit>(a, stream);
+			case LITENN_FMT_Q4_0: return launch_stream<Q4_0Unit>(a, stream, plan_only);
+			case LITENN_FMT_Q4_1: return launch_stream<Q4_1Unit>(a, stream, plan_only);
+			case LITENN_FMT_Q5_0: return launch_stream<Q5_0Unit>(a, stream, plan_only);
+			case LITENN_FMT_Q5_1: return launch_stream<Q5_1Unit>(a, stream, plan_only);
+			case LITENN_FMT_Q8_0: return launch_stream<Q8_0Unit>(a, stream, plan_only);
+			case LITENN_FMT_Q2_K: return launch_stream<Q2_KUnit>(a, stream, plan_only);
+			case LITENN_FMT_Q3_K: return launch_stream<Q3_KUnit>(a, stream, plan_only);
+			case LITENN_FMT_Q4_K: return launch_stream<Q4_KUnit>(a, stream, plan_only);
+			case LITENN_FMT_Q5_K: return launch_stream<Q5_KUnit>(a, stream, plan_only);
+			default: return launch_stream<Q6_KUnit>(a, stream, plan_only);
 			}
 		}
 
@@ -1911,8 +1945,13 @@ namespace litenn_hip
 			a.k = static_cast<int>(k);
 			a.row_bytes = static_cast<uint32_t>(rb);
 			a.silu_mul = silu_mul ? 1 : 0;
+			a.partials = nullptr;
+			a.partial_stride = 0;
+			a.partials_on = 0;
 			return true;
 		}
+
+#include "attn_block.inc"
 	} // namespace
 
 	// One fused launch over up to three same-format matrices that share x (see GemvArgs).  Returns
@@ -2071,6 +2110,125 @@ namespace litenn_hip
 		return true;
 	}
 
+
+	// The launches that follow the decoder-block kernel: an operator group as launch_gemv_fused runs it,
+	// with the kernel's eight partial vectors (`stride` floats apart) added in team order onto x while
+	// it is staged (on_x; k must be 4096) or onto the residual in the epilogue (!on_x).  Returns false,
+	// with nothing launched, when the streaming kernel does not take the shape; plan_only launches
+	// nothing in either case.
+	bool launch_gemv_fused_partials(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
+	                                const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
+	                                const float* partials, size_t stride, bool on_x, bool plan_only, hipStream_t stream)
+	{
+		GemvArgs a;
+		if (!fill_args(a, fmt, count, w, y, n, k, x, residual, norm_w, eps, silu_mul) || !partials ||
+		    (on_x && k != 4096) || (!on_x && !residual))
+		{
+			return false;
+		}
+		a.partials = partials;
+		a.partial_stride = static_cast<uint32_t>(stride);
+		a.partials_on = on_x ? 1 : 2;
+		return stream_dispatch(fmt, a, stream, plan_only);
+	}
+
+	// The attention half of a decoder block for one new row as one launch (attn_block.inc).  Returns
+	// false, with nothing launched, when the shape is not one the kernel is built for: 4096-wide model,
+	// 32 heads of 128, a KV head count that is a multiple of 8, a Float16 cache, a card of 256 CUs, and
+	// one of the format combinations instantiated below.  plan_only launches nothing in either case.
+	// scratch: q / k / v take the first phase's rows (n_head * 128 and n_kv_head * 128 twice), triples
+	// n_head * 8 * 132 floats, flags 512 words (zero before the model's first launch), y_partial 8 * d
+	// floats; counters = {position, tokens emitted, steps run}; bit 1 of *err is set when a wait inside
+	// the kernel ran out (a wait polls at most spin_limit times).
+	bool launch_attn_block(const int* fmts, const void* const* wqkv, const size_t* n_qkv, int fmt_o, const void* wo,
+	                       size_t d, const float* x, const float* norm_w, double eps, float* q, float* k, float* v,
+	                       void* kcache, void* vcache, int cache_dtype, const float* cos_t, const float* sin_t,
+	                       size_t rope_dims, const int* counters, int layer, size_t n_head, size_t n_kv_head,
+	                       size_t head_dim, float* triples, unsigned* flags, float* y_partial, int* err, int spin_limit,
+	                       bool plan_only, hipStream_t stream)
+	{
+		const auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+		if (d != 4096 || n_head != 32 || head_dim != 128 || n_kv_head == 0 || n_kv_head % 8 != 0 ||
+		    n_kv_head > 32 || cache_dtype != LITENN_F16 || rope_dims % 8 != 0 || rope_dims > 128 || rope_dims == 0 ||
+		    compute_units() != 256 || n_qkv[0] != d || n_qkv[1] != n_kv_head * 128 || n_qkv[2] != n_kv_head * 128 ||
+		    !aligned(q) || !aligned(k) || !aligned(v) || !aligned(kcache) || !aligned(vcache) ||
+		    !aligned(cos_t) || !aligned(sin_t) || !aligned(wo) || !aligned(triples) || !aligned(y_partial) || !norm_w ||
+		    layer < 0 || layer > 254)
+		{
+			return false;
+		}
+		float* ys[3] = { q, k, v };
+		AttnBlockPlan plan{};
+		GemvArgs a0, a1;
+		bool ok = false;
+		int variant = -1;
+		if (fmts[0] == fmts[1] && fmts[1] == fmts[2] && fmt_o == fmts[0] && (fmts[0] == LITENN_FMT_Q4_0 || fmts[0] == LITENN_FMT_Q4_K))
+		{
+			if (!fill_args(a0, fmts[0], 3, wqkv, ys, n_qkv, d, x, nullptr, norm_w, eps, false))
+			{
+				return false;
+			}
+			a1 = a0;
+			if (fmts[0] == LITENN_FMT_Q4_0)
+			{
+				variant = 0;
+				ok = plan_attn_block<Q4_0Unit, Q4_0Unit, Q4_0Unit>(plan, a0, a1, false);
+			}
+			else
+			{
+				variant = 2;
+				ok = plan_attn_block<Q4_KUnit, Q4_KUnit, Q4_KUnit>(plan, a0, a1, false);
+			}
+		}
+		else if (fmts[0] == LITENN_FMT_Q4_K && fmts[1] == LITENN_FMT_Q4_K && fmts[2] == LITENN_FMT_Q6_K && fmt_o == LITENN_FMT_Q4_K)
+		{
+			if (!fill_args(a0, fmts[0], 2, wqkv, ys, n_qkv, d, x, nullptr, norm_w, eps, false) ||
+			    !fill_args(a1, fmts[2], 1, wqkv + 2, ys + 2, n_qkv + 2, d, x, nullptr, norm_w, eps, false))
+			{
+				return false;
+			}
+			variant = 1;
+			ok = plan_attn_block<Q4_KUnit, Q6_KUnit, Q4_KUnit>(plan, a0, a1, true);
+		}
+		if (!ok)
+		{
+			return false;
+		}
+		if (plan_only)
+		{
+			return true;
+		}
+		AttnBlockArgs& f = plan.args;
+		f.wo = static_cast<const uint8_t*>(wo);
+		f.wo_row_bytes = static_cast<uint32_t>(row_bytes(fmt_o, d));
+		f.wo_seg_bytes = f.wo_row_bytes / kBlockTeams;
+		f.q = q;
+		f.k_new = k;
+		f.v_new = v;
+		f.kcache = static_cast<uint16_t*>(kcache);
+		f.vcache = static_cast<uint16_t*>(vcache);
+		f.cos_t = cos_t;
+		f.sin_t = sin_t;
+		f.past_dev = counters;
+		f.triples = triples;
+		f.flags = flags;
+		f.layer = layer;
+		f.y_partial = y_partial;
+		f.err = err;
+		f.n_head = static_cast<int>(n_head);
+		f.n_kv_head = static_cast<int>(n_kv_head);
+		f.rope_dims = static_cast<int>(rope_dims);
+		f.d = static_cast<int>(d);
+		f.spin_limit = spin_limit;
+		switch (variant)
+		{
+		case 0: launch_attn_block_variant<Q4_0Unit, Q4_0Unit, Q4_0Unit>(plan, stream); break;
+		case 1: launch_attn_block_variant<Q4_KUnit, Q6_KUnit, Q4_KUnit>(plan, stream); break;
+		default: launch_attn_block_variant<Q4_KUnit, Q4_KUnit, Q4_KUnit>(plan, stream); break;
+		}
+		return true;
+	}
+
 	void launch_dequantize(int fmt, const void* wq, size_t rows, size_t k, float* dst, hipStream_t stream)
 	{
 		dequantize_kernel<<<dim3(rows), dim3(256), 0, stream>>>(fmt, static_cast<const uint8_t*>(wq), dst, rows,
@@ -2131,6 +2289,21 @@ extern "C" int litenn_hip_gemv_trace_read(unsigned long long* dst, size_t entrie
 	void* dev = nullptr;
 	LITENN_HIP_TRY("read the GEMV timeline", hipGetSymbolAddress(&dev, HIP_SYMBOL(g_trace)));
 	LITENN_HIP_TRY("read the GEMV timeline", hipMemset(dev, 0, total * sizeof(unsigned long long)));
+	return 0;
+}
+
+// Timeline build only: the decoder-block kernel's stamps ([wavefront][8 points]) of its last launch
+extern "C" int litenn_hip_block_trace_read(unsigned long long* dst, size_t entries)
+{
+	using namespace litenn_hip;
+	constexpr size_t total = static_cast<size_t>(kTraceWaves) * kBlockTraceSlots;
+	if (!dst || entries > total)
+	{
+		return fail("read the block timeline", "destination is null or asks for more than 4096 x 8 entries");
+	}
+	LITENN_HIP_TRY("read the block timeline", hipDeviceSynchronize());
+	LITENN_HIP_TRY("read the block timeline",
+	               hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_block_trace), entries * sizeof(unsigned long long)));
 	return 0;
 }
 

@@ -4,6 +4,7 @@
 // weight stream; they are written to keep f32 (f64 for the norm) semantics of the
 // reference chains and to read every operand once.
 #include "common.hpp"
+#include "attn_math.hpp"
 
 #include <algorithm>
 
@@ -93,17 +94,6 @@ namespace litenn_hip
 			const double angle = static_cast<double>(pos_offset + pos) * inv_freq * freq_scale;
 			cos_t[idx] = static_cast<float>(cos(angle));
 			sin_t[idx] = static_cast<float>(sin(angle));
-		}
-
-		// f32 rotation with separately rounded products (RoPE.h:93-111), so the four multiplies
-		// round like the reference's Multiply nodes.  The pragma is what keeps them apart: the
-		// compiler contracts a * c - b * s into a fused multiply-add by default.
-		__device__ __forceinline__ void rotate(float a, float b, float c, float s, float& o0, float& o1)
-		{
-#pragma clang fp contract(off)
-			const float ac = a * c, bs = b * s, as = a * s, bc = b * c;
-			o0 = ac - bs;
-			o1 = as + bc;
 		}
 
 		// x,y [m, n_heads, head_dim]; tables indexed by row (positions start at the table's origin)
@@ -334,20 +324,6 @@ namespace litenn_hip
 			return c;
 		}
 
-		__device__ __forceinline__ void device_store(float* p, float v)
-		{
-			__hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-		}
-		__device__ __forceinline__ float device_load(const float* p)
-		{
-			return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-		}
-
-		__device__ __forceinline__ float softmax_weight(float m, float m_all)
-		{
-			return m == -INFINITY ? 0.0f : expf(m - m_all);
-		}
-
 		// What the single-token step adds when the rotation and the cache append ride inside the
 		// attention launch (tools/gguf/LLaMABuilder.cpp:596-622,640-645): q, k_new and v_new are the
 		// un-rotated projections of the one new row; the tables are [ctx, rope_dims / 2].
@@ -359,78 +335,6 @@ namespace litenn_hip
 			const float* sin_t;
 			int rope_dims;
 		};
-
-		template <typename KV>
-		__device__ __forceinline__ float through_cache(float v);
-		template <>
-		__device__ __forceinline__ float through_cache<float>(float v) { return v; }
-		template <>
-		__device__ __forceinline__ float through_cache<uint16_t>(float v)
-		{
-			return f16_bits_to_f32(f32_to_f16_bits_litenn(v));
-		}
-
-		// The new row's key / value as the cache will hold them: rounded through the cache type once,
-		// used from registers and stored from the same values.
-		template <typename KV>
-		__device__ __forceinline__ void round_through_cache(float (&v)[8])
-		{
-#pragma unroll
-			for (int e = 0; e < 8; ++e)
-			{
-				v[e] = through_cache<KV>(v[e]);
-			}
-		}
-		// values already representable in the cache type: the hardware conversion is exact for them
-		__device__ __forceinline__ void store8_exact(float* dst, const float (&v)[8])
-		{
-			reinterpret_cast<float4*>(dst)[0] = make_float4(v[0], v[1], v[2], v[3]);
-			reinterpret_cast<float4*>(dst)[1] = make_float4(v[4], v[5], v[6], v[7]);
-		}
-		__device__ __forceinline__ void store8_exact(uint16_t* dst, const float (&v)[8])
-		{
-			typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-			typedef float float2v __attribute__((ext_vector_type(2)));
-			uint32_t w[4];
-#pragma unroll
-			for (int i = 0; i < 4; ++i)
-			{
-				const float2v f = { v[2 * i], v[2 * i + 1] };
-				w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, half2v));
-			}
-			*reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
-		}
-
-		__device__ __forceinline__ void store8(float* dst, const float (&v)[8])
-		{
-			reinterpret_cast<float4*>(dst)[0] = make_float4(v[0], v[1], v[2], v[3]);
-			reinterpret_cast<float4*>(dst)[1] = make_float4(v[4], v[5], v[6], v[7]);
-		}
-		__device__ __forceinline__ void store8(uint16_t* dst, const float (&v)[8])
-		{
-			uint32_t w[4];
-#pragma unroll
-			for (int i = 0; i < 4; ++i)
-			{
-				w[i] = static_cast<uint32_t>(f32_to_f16_bits_litenn(v[2 * i])) |
-				       (static_cast<uint32_t>(f32_to_f16_bits_litenn(v[2 * i + 1])) << 16);
-			}
-			*reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
-		}
-
-		// the four interleaved pairs a lane owns, rotated by the angles of its position
-		__device__ __forceinline__ void rotate8(float (&v)[8], const float4& c, const float4& sn)
-		{
-			const float cs[4] = { c.x, c.y, c.z, c.w }, ss[4] = { sn.x, sn.y, sn.z, sn.w };
-#pragma unroll
-			for (int i = 0; i < 4; ++i)
-			{
-				float o0, o1;
-				rotate(v[2 * i], v[2 * i + 1], cs[i], ss[i], o0, o1);
-				v[2 * i] = o0;
-				v[2 * i + 1] = o1;
-			}
-		}
 
 		// FUSED (single new row, head_dim 128): q arrives un-rotated and is rotated in registers;
 		// the cache holds positions 0 .. past - 1 and the new position's key/value come from
@@ -1013,7 +917,7 @@ namespace litenn_hip
 			}
 		}
 
-		// one wavefront; counters = {past length, tokens emitted}, out may be null
+		// one wavefront; counters = {past length, tokens emitted, steps run}, out may be null
 		__global__ __launch_bounds__(64) void argmax_merge_step_kernel(const float* __restrict__ pv,
 		                                                                const int* __restrict__ pi, int blocks,
 		                                                                int32_t* __restrict__ next, int* counters,
@@ -1039,6 +943,7 @@ namespace litenn_hip
 					counters[1] += 1;
 				}
 				counters[0] += past_inc;
+				counters[2] += 1;
 			}
 		}
 

@@ -37,6 +37,15 @@ namespace litenn_hip
 	bool launch_linear_group(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
 	                         const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
 	                         float* scratch_x, float* scratch_gate, float* scratch_up, hipStream_t stream);
+	bool launch_gemv_fused_partials(int fmt, int count, const void* const* w, float* const* y, const size_t* n, size_t k,
+	                                const float* x, const float* residual, const float* norm_w, double eps, bool silu_mul,
+	                                const float* partials, size_t stride, bool on_x, bool plan_only, hipStream_t stream);
+	bool launch_attn_block(const int* fmts, const void* const* wqkv, const size_t* n_qkv, int fmt_o, const void* wo,
+	                       size_t d, const float* x, const float* norm_w, double eps, float* q, float* k, float* v,
+	                       void* kcache, void* vcache, int cache_dtype, const float* cos_t, const float* sin_t,
+	                       size_t rope_dims, const int* counters, int layer, size_t n_head, size_t n_kv_head,
+	                       size_t head_dim, float* triples, unsigned* flags, float* y_partial, int* err, int spin_limit,
+	                       bool plan_only, hipStream_t stream);
 	bool launch_gemv_fused_mixed(const int* fmts, int count, const void* const* w, float* const* y, const size_t* n,
 	                             size_t k, const float* x, const float* norm_w, double eps, hipStream_t stream);
 	void launch_get_rows_q(int fmt, const void* table, size_t rows, size_t k, const int32_t* ids, size_t n_ids,
@@ -68,11 +77,13 @@ namespace litenn_hip
 
 	namespace
 	{
-		// counters[0] = past length, counters[1] = tokens emitted so far
+		// counters[0] = past length, counters[1] = tokens emitted so far, counters[2] = steps this model
+		// has run (never reset: it names a step in the values its workgroups hand to each other)
 		__global__ void set_counters_kernel(int* counters, int past, int emitted)
 		{
 			counters[0] = past;
 			counters[1] = emitted;
+			counters[2] += 1;
 		}
 
 		struct Weight
@@ -118,12 +129,19 @@ struct litenn_hip_llama
 	int32_t* d_next = nullptr; // token produced by the last arg-max
 	int32_t* d_out = nullptr;  // generated tokens
 	size_t cap_out = 0;
-	int* d_counters = nullptr; // {past, emitted}
+	int* d_counters = nullptr; // {past, emitted, steps run}
 	int* d_err = nullptr;
 	// single-row attention: key chunks per head, their meeting place and arrival counters
 	size_t attn_splits = 1;
 	float* attn_partial = nullptr;
 	int* attn_counters = nullptr;
+	// The attention half of a block as one launch (launch_attn_block): 0 = not yet decided, 1 = every
+	// block of this model takes it, -1 = it does not apply, or a wait inside it once ran out
+	int block_fused = 0;
+	float* blk_triples = nullptr;  // [head_count][8][132] chunk triples of the launch's second phase
+	unsigned* blk_flags = nullptr; // [2][256] tags of the launch's two meetings
+	float* blk_partial = nullptr; // [8][embedding_length] the launch's result, one vector per team
+	int blk_spins = 8192;         // polls a wait inside the launch may take before it gives up
 	int past = 0;
 	hipGraphExec_t step_exec = nullptr;
 	hipGraph_t step_graph = nullptr;
@@ -308,6 +326,89 @@ namespace
 		                    m->xn, m->gate2, m->up, s);
 	}
 
+	// the three launches of a block's single-token step when its attention half is one launch
+	bool block_step(litenn_hip_llama* m, const Layer& L, int layer, bool plan_only, hipStream_t s)
+	{
+		const size_t d = m->p.embedding_length, ff = m->p.feed_forward_length;
+		const int qkv_fmt[3] = { L.wq.fmt, L.wk.fmt, L.wv.fmt };
+		const void* qkv_w[3] = { L.wq.data, L.wk.data, L.wv.data };
+		const size_t qkv_n[3] = { L.wq.n, L.wk.n, L.wv.n };
+		if (L.wq.k != d || L.wk.k != d || L.wv.k != d || L.wo.k != d || L.wo.n != d || L.gate.fmt != L.up.fmt ||
+		    L.gate.k != d || L.up.k != d || L.gate.n != ff || L.up.n != ff || L.down.k != ff || L.down.n != d)
+		{
+			return false;
+		}
+		if (!launch_attn_block(qkv_fmt, qkv_w, qkv_n, L.wo.fmt, L.wo.data, d, m->x, L.attn_norm, m->p.rms_norm_epsilon, m->q,
+		                       m->k, m->v, L.kcache, L.vcache, m->p.kv_dtype, m->cos_t, m->sin_t,
+		                       static_cast<size_t>(m->p.rope_dimension_count), m->d_counters, layer, m->p.head_count,
+		                       m->p.head_count_kv, m->head_dim, m->blk_triples, m->blk_flags, m->blk_partial, m->d_err,
+		                       m->blk_spins, plan_only, s))
+		{
+			return false;
+		}
+		// gate = silu(x' . Wg) * (x' . Wu) with x' = RMSNorm(x + the eight partial vectors)
+		const void* gu_w[2] = { L.gate.data, L.up.data };
+		const size_t gu_n[2] = { L.gate.n, L.up.n };
+		float* gu_y[2] = { m->gate, nullptr };
+		if (!launch_gemv_fused_partials(L.gate.fmt, 2, gu_w, gu_y, gu_n, d, m->x, nullptr, L.ffn_norm, m->p.rms_norm_epsilon,
+		                                true, m->blk_partial, d, true, plan_only, s))
+		{
+			return false;
+		}
+		// x = (x + the eight partial vectors) + mlp
+		const void* dn_w[1] = { L.down.data };
+		const size_t dn_n[1] = { L.down.n };
+		float* dn_y[1] = { m->x };
+		return launch_gemv_fused_partials(L.down.fmt, 1, dn_w, dn_y, dn_n, ff, m->gate, m->x, nullptr, 0.0, false,
+		                                  m->blk_partial, d, false, plan_only, s);
+	}
+
+	// Decides once per model (and again after a tensor changed) whether its blocks take that form, and
+	// allocates what the launch needs.
+	bool block_fused_ready(litenn_hip_llama* m)
+	{
+		if (m->block_fused != 0)
+		{
+			return m->block_fused > 0;
+		}
+		m->block_fused = -1;
+		// LITENN_HIP_ATTN_BLOCK=0 keeps the separate launches; LITENN_HIP_ATTN_BLOCK_SPINS bounds the
+		// launch's waits (read when the model's step is decided, not per launch)
+		const char* off = getenv("LITENN_HIP_ATTN_BLOCK");
+		if (off && off[0] == '0')
+		{
+			return false;
+		}
+		if (const char* spins = getenv("LITENN_HIP_ATTN_BLOCK_SPINS"))
+		{
+			m->blk_spins = std::max(0, atoi(spins));
+		}
+		const size_t d = m->p.embedding_length;
+		if (!m->blk_partial)
+		{
+			// flags start at 0, which no launch's tag equals
+			const size_t triples = sizeof(float) * static_cast<size_t>(m->p.head_count) * 8 * 132;
+			if (hipMalloc(reinterpret_cast<void**>(&m->blk_triples), triples) != hipSuccess ||
+			    hipMalloc(reinterpret_cast<void**>(&m->blk_flags), sizeof(unsigned) * 512) != hipSuccess ||
+			    hipMalloc(reinterpret_cast<void**>(&m->blk_partial), sizeof(float) * 8 * d) != hipSuccess ||
+			    hipMemsetAsync(m->blk_flags, 0, sizeof(unsigned) * 512, m->stream) != hipSuccess ||
+			    hipStreamSynchronize(m->stream) != hipSuccess)
+			{
+				(void)hipGetLastError();
+				return false;
+			}
+		}
+		for (size_t i = 0; i < m->layers.size(); ++i)
+		{
+			if (!block_step(m, m->layers[i], static_cast<int>(i), true, m->stream))
+			{
+				return false;
+			}
+		}
+		m->block_fused = 1;
+		return true;
+	}
+
 	// The single-token step: six fused launches per decoder block
 	//   [RMSNorm + q/k/v] [RoPE + cache append] [attention] [o + residual] [RMSNorm + gate/up + SwiGLU]
 	//   [down + residual]
@@ -319,8 +420,15 @@ namespace
 		const size_t H = m->p.head_count, KH = m->p.head_count_kv, hd = m->head_dim;
 		const int* past_dev = m->d_counters;
 		launch_get_rows_q(m->tok_embd.fmt, m->tok_embd.data, m->tok_embd.n, d, ids, 1, m->x, m->d_err, s);
+		// three launches per block where the attention half is one launch (block_step), else five;
+		// decided (and its buffers allocated) by the entry points before anything is queued or captured
+		const bool fused_blocks = m->block_fused > 0;
 		for (Layer& L : m->layers)
 		{
+			if (fused_blocks && block_step(m, L, static_cast<int>(&L - m->layers.data()), false, s))
+			{
+				continue;
+			}
 			const Weight* qkv[3] = { &L.wq, &L.wk, &L.wv };
 			float* qkv_out[3] = { m->q, m->k, m->v };
 			// one launch when the three share a format or are one of the two-format mixes the GEMV
@@ -458,6 +566,8 @@ namespace
 		matmul(m, head, m->xn, logit_rows, m->logits, nullptr, flags, s);
 	}
 
+	constexpr int kBlockWaitRanOut = -2;
+
 	int check_error_flag(litenn_hip_llama* m)
 	{
 		int flag = 0;
@@ -467,9 +577,23 @@ namespace
 		{
 			const int zero = 0;
 			(void)hipMemcpy(m->d_err, &zero, sizeof(int), hipMemcpyHostToDevice);
+			if (flag & 2)
+			{
+				return kBlockWaitRanOut;
+			}
 			return fail(kAction, "GetRows index out of range");
 		}
 		return 0;
+	}
+
+	// A wait inside the one-launch attention half ran out (its workgroups were not all running at
+	// once: the card was shared, or is not the one the launch is shaped for).  What that step
+	// computed is void; the model takes the separate launches from now on and the caller repeats
+	// the step.  The flags the launch left behind are never read again.
+	void give_up_block_launch(litenn_hip_llama* m)
+	{
+		m->block_fused = -1;
+		drop_graph(m);
 	}
 } // namespace
 
@@ -608,10 +732,10 @@ int llama_create_impl(int dev, const litenn_hip_llama_params* params, litenn_hip
 			return bail(e);
 		}
 	}
-	if ((e = hipMalloc(reinterpret_cast<void**>(&m->d_counters), 2 * sizeof(int))) != hipSuccess ||
+	if ((e = hipMalloc(reinterpret_cast<void**>(&m->d_counters), 4 * sizeof(int))) != hipSuccess ||
 	    (e = hipMalloc(reinterpret_cast<void**>(&m->d_err), sizeof(int))) != hipSuccess ||
 	    (e = hipMalloc(reinterpret_cast<void**>(&m->d_next), sizeof(int32_t))) != hipSuccess ||
-	    (e = hipMemsetAsync(m->d_counters, 0, 2 * sizeof(int), m->stream)) != hipSuccess ||
+	    (e = hipMemsetAsync(m->d_counters, 0, 4 * sizeof(int), m->stream)) != hipSuccess ||
 	    (e = hipMemsetAsync(m->d_err, 0, sizeof(int), m->stream)) != hipSuccess ||
 	    (e = hipMemsetAsync(m->d_next, 0, sizeof(int32_t), m->stream)) != hipSuccess)
 	{
@@ -666,6 +790,13 @@ extern "C" int litenn_hip_llama_free(litenn_hip_llama* m)
 	}
 	drop_graph(m);
 	free_scratch(m);
+	for (void* p : { static_cast<void*>(m->blk_triples), static_cast<void*>(m->blk_flags), static_cast<void*>(m->blk_partial) })
+	{
+		if (p)
+		{
+			(void)hipFree(p);
+		}
+	}
 	for (Layer& L : m->layers)
 	{
 		if (L.kcache)
@@ -765,6 +896,7 @@ extern "C" int litenn_hip_llama_set_tensor(litenn_hip_llama* m, int which, int l
 	target->n = n;
 	target->k = k;
 	drop_graph(m);
+	m->block_fused = 0; // decided again with the new tensor
 	return 0;
 }
 
@@ -781,6 +913,11 @@ extern "C" int litenn_hip_llama_reset(litenn_hip_llama* m)
 extern "C" int litenn_hip_llama_past(const litenn_hip_llama* m)
 {
 	return m ? m->past : -1;
+}
+
+extern "C" int litenn_hip_llama_block_form(const litenn_hip_llama* m)
+{
+	return m ? m->block_fused : 0;
 }
 
 extern "C" int litenn_hip_llama_eval(litenn_hip_llama* m, const int32_t* tokens, size_t rows, float* logits,
@@ -819,24 +956,35 @@ extern "C" int litenn_hip_llama_eval(litenn_hip_llama* m, const int32_t* tokens,
 	{
 		return 1;
 	}
+	(void)block_fused_ready(m);
 	hipStream_t s = m->stream;
-	LITENN_HIP_TRY(kAction, hipMemcpyAsync(m->d_tokens, tokens, sizeof(int32_t) * rows, hipMemcpyHostToDevice, s));
-	set_counters_kernel<<<1, 1, 0, s>>>(m->d_counters, m->past, 0);
-	forward(m, m->d_tokens, rows, logit_rows, flags);
-	LITENN_HIP_TRY(kAction, hipGetLastError());
-	const size_t vocab = m->p.vocab_size;
-	if (logits)
+	for (int attempt = 0;; ++attempt)
 	{
-		LITENN_HIP_TRY(kAction, hipMemcpyAsync(logits, m->logits, sizeof(float) * rows * vocab, hipMemcpyDeviceToHost, s));
-	}
-	if (last_logits)
-	{
-		LITENN_HIP_TRY(kAction, hipMemcpyAsync(last_logits, m->logits + (logit_rows - 1) * vocab, sizeof(float) * vocab,
-		                                       hipMemcpyDeviceToHost, s));
-	}
-	if (check_error_flag(m) != 0)
-	{
-		return 1;
+		LITENN_HIP_TRY(kAction, hipMemcpyAsync(m->d_tokens, tokens, sizeof(int32_t) * rows, hipMemcpyHostToDevice, s));
+		set_counters_kernel<<<1, 1, 0, s>>>(m->d_counters, m->past, 0);
+		forward(m, m->d_tokens, rows, logit_rows, flags);
+		LITENN_HIP_TRY(kAction, hipGetLastError());
+		const size_t vocab = m->p.vocab_size;
+		if (logits)
+		{
+			LITENN_HIP_TRY(kAction, hipMemcpyAsync(logits, m->logits, sizeof(float) * rows * vocab, hipMemcpyDeviceToHost, s));
+		}
+		if (last_logits)
+		{
+			LITENN_HIP_TRY(kAction, hipMemcpyAsync(last_logits, m->logits + (logit_rows - 1) * vocab, sizeof(float) * vocab,
+			                                       hipMemcpyDeviceToHost, s));
+		}
+		const int rc = check_error_flag(m);
+		if (rc == kBlockWaitRanOut && attempt == 0)
+		{
+			give_up_block_launch(m); // and once more through the separate launches
+			continue;
+		}
+		if (rc != 0)
+		{
+			return rc == kBlockWaitRanOut ? fail(kAction, "a wait inside the decoder step ran out") : 1;
+		}
+		break;
 	}
 	m->past += static_cast<int>(rows);
 	return 0;
@@ -877,6 +1025,7 @@ extern "C" int litenn_hip_llama_generate(litenn_hip_llama* m, const int32_t* pro
 	{
 		return 1;
 	}
+	(void)block_fused_ready(m);
 	if (n_new > m->cap_out)
 	{
 		drop_graph(m);
@@ -980,7 +1129,19 @@ extern "C" int litenn_hip_llama_generate(litenn_hip_llama* m, const int32_t* pro
 	GEN_TRY(hipEventRecord(ev[2], s));
 	GEN_TRY(hipGetLastError());
 	GEN_TRY(hipMemcpyAsync(out_tokens, m->d_out, sizeof(int32_t) * n_new, hipMemcpyDeviceToHost, s));
+	int step_flag = 0;
+	GEN_TRY(hipMemcpyAsync(&step_flag, m->d_err, sizeof(int), hipMemcpyDeviceToHost, s));
 	GEN_TRY(hipStreamSynchronize(s));
+	if ((step_flag & 2) && m->block_fused > 0)
+	{
+		// a wait inside the one-launch attention half ran out: the tokens are void; once more, from
+		// the prompt, through the separate launches (`past` has not moved)
+		const int zero = 0;
+		GEN_TRY(hipMemcpy(m->d_err, &zero, sizeof(int), hipMemcpyHostToDevice));
+		cleanup();
+		give_up_block_launch(m);
+		return litenn_hip_llama_generate(m, prompt, n_prompt, n_new, out_tokens, flags, prefill_ms, decode_ms);
+	}
 	float ms = 0.0f;
 	if (prefill_ms)
 	{

@@ -183,6 +183,248 @@ namespace litenn_hip
 			}
 			return 0;
 		}
+
+		// ---- exchange among the workgroups of one XCD -----------------------------------------
+		// The card's 256 CUs sit in 8 XCDs of 32, each with an L2 of its own; what one CU stores is
+		// visible to the other CUs of its XCD once it has reached that L2, without crossing the
+		// fabric that joins the XCDs.  This kernel measures what a phase boundary inside one launch
+		// costs when only the workgroups of one XCD have to meet: every workgroup reads the XCD it
+		// runs on (XCC_ID), takes a slot among that XCD's workgroups from a ticket counter, and then
+		// walks `phases` phases; in each it publishes one value and needs the values all slots of its
+		// XCD published in the phase before.
+		//   MODE 0: store, wait for the L2's acknowledgement, add one to the XCD's counter (an atomic
+		//           executed in the L2); one lane polls the counter with an atomic add of zero, then
+		//           the values are loaded past the CU's own L1 (sc0).
+		//   MODE 1: every value carries the number of its phase; 32 lanes poll the 32 slots
+		//           themselves with sc0 loads until each shows the phase wanted.
+		//   MODE 2: like 1 with device-scope accesses (sc1 on loads and stores), the form an
+		//           exchange across XCDs needs; here still among the workgroups of one XCD.
+		//   MODE 3: one flag word per workgroup: the value is stored with an ordinary store to an address
+		//           of its own per phase (never in any CU's L1), acknowledged by the L2, then the flag is
+		//           stored; 32 lanes poll the 32 flags with atomic ORs of zero (executed in the L2) and
+		//           then load the values with ordinary loads.
+		//   MODE 4: like 3 with the flags polled by device-scope loads.
+		// Every wait is bounded by `spin_limit` polls; a wait that runs out sets err[0] and the
+		// workgroup walks the remaining phases without waiting, so the grid always drains.
+		// Layout of `mem` (unsigned, zeroed by the host): [0,8) tickets per XCD, [16,24) arrival
+		// counters per XCD, then from word 64 on, per XCD, 2 x 64 words: two parities of 32 slots of
+		// {value, phase tag}.
+		__device__ __forceinline__ unsigned mb_xcc_id()
+		{
+			// HW_REG_XCC_ID (register 20), bits [3:0]
+			return __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11));
+		}
+
+		__device__ __forceinline__ unsigned mb_l2_atomic_add(unsigned* p, unsigned v)
+		{
+			unsigned old;
+			asm volatile("global_atomic_add %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)" : "=v"(old) : "v"(p), "v"(v) : "memory");
+			return old;
+		}
+
+		template <bool DEVICE_SCOPE>
+		__device__ __forceinline__ unsigned long long mb_load_past_l1(const unsigned long long* p)
+		{
+			unsigned long long v;
+			if constexpr (DEVICE_SCOPE)
+			{
+				asm volatile("global_load_dwordx2 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+			}
+			else
+			{
+				asm volatile("global_load_dwordx2 %0, %1, off sc0\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+			}
+			return v;
+		}
+
+		template <bool DEVICE_SCOPE>
+		__device__ __forceinline__ void mb_store_to_l2(unsigned long long* p, unsigned long long v)
+		{
+			if constexpr (DEVICE_SCOPE)
+			{
+				asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : : "v"(p), "v"(v) : "memory");
+			}
+			else
+			{
+				asm volatile("global_store_dwordx2 %0, %1, off\n\ts_waitcnt vmcnt(0)" : : "v"(p), "v"(v) : "memory");
+			}
+		}
+
+		template <int MODE>
+		__global__ __launch_bounds__(512) void mb_xcd_exchange_kernel(unsigned* __restrict__ mem, int phases, int spin_limit,
+		                                                               int expected_per_xcd, int* __restrict__ err,
+		                                                               unsigned* __restrict__ result,
+		                                                               unsigned long long* __restrict__ stamps)
+		{
+			__shared__ unsigned s_value;
+			__shared__ int s_slot;
+			__shared__ volatile int s_dead;
+			const int tid = threadIdx.x;
+			const unsigned xcc = mb_xcc_id() & 7u;
+			constexpr bool kDevice = MODE == 2;
+
+			if (tid == 0)
+			{
+				s_slot = static_cast<int>(mb_l2_atomic_add(mem + xcc, 1u));
+				s_dead = 0;
+				s_value = 1u;
+			}
+			__syncthreads();
+			const int slot = s_slot;
+			if (slot >= 32)
+			{
+				// more workgroups on this XCD than the exchange has slots: not the placement measured
+				if (tid == 0)
+				{
+					atomicExch(err, 2);
+				}
+				return;
+			}
+			if constexpr (MODE >= 3)
+			{
+				// mem: [64, 64 + 8 * 32) flags; fresh[phase][xcc][32] values (8 bytes each) behind them
+				unsigned* flags = mem + 64 + xcc * 32;
+				unsigned long long* fresh = reinterpret_cast<unsigned long long*>(mem + 2048);
+				for (int p = 0; p < phases; ++p)
+				{
+					unsigned long long* row = fresh + (static_cast<size_t>(p) * 8 + xcc) * 32;
+					if (tid == 0)
+					{
+						mb_store_to_l2<false>(row + slot, s_value); // waits for the L2's acknowledgement
+						asm volatile("global_store_dword %0, %1, off" : : "v"(flags + slot), "v"(static_cast<unsigned>(p + 1)) : "memory");
+						if (stamps && blockIdx.x == 0)
+						{
+							stamps[p] = __builtin_amdgcn_s_memrealtime();
+						}
+					}
+					if (tid < 64)
+					{
+						unsigned mine = 0;
+						if (tid < expected_per_xcd)
+						{
+							int spins = 0;
+							for (;;)
+							{
+								unsigned seen;
+								if (MODE == 3)
+								{
+									seen = mb_l2_atomic_add(flags + tid, 0u);
+								}
+								else
+								{
+									asm volatile("global_load_dword %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=v"(seen) : "v"(flags + tid) : "memory");
+								}
+								if (seen == static_cast<unsigned>(p + 1) || s_dead)
+								{
+									break;
+								}
+								if (++spins > spin_limit)
+								{
+									s_dead = 1;
+									atomicExch(err, 1);
+									break;
+								}
+							}
+							unsigned long long got;
+							asm volatile("global_load_dwordx2 %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=v"(got) : "v"(row + tid) : "memory");
+							mine = static_cast<unsigned>(got);
+						}
+						for (int o = 32; o; o >>= 1)
+						{
+							mine += __shfl_xor(mine, o);
+						}
+						if (tid == 0)
+						{
+							s_value = mine + 1u;
+						}
+					}
+					__syncthreads();
+				}
+				if (tid == 0)
+				{
+					result[blockIdx.x * 2] = s_value;
+					result[blockIdx.x * 2 + 1] = xcc * 64u + static_cast<unsigned>(slot);
+				}
+				return;
+			}
+			unsigned long long* values = reinterpret_cast<unsigned long long*>(mem + 64 + xcc * 128);
+			unsigned* counter = mem + 16 + xcc;
+			for (int p = 0; p < phases; ++p)
+			{
+				// publish this workgroup's value of phase p
+				if (tid == 0)
+				{
+					const unsigned long long v = (static_cast<unsigned long long>(p + 1) << 32) | s_value;
+					mb_store_to_l2<kDevice>(values + (p & 1) * 32 + slot, v);
+					if (MODE == 0)
+					{
+						mb_l2_atomic_add(counter, 1u);
+					}
+					if (stamps && blockIdx.x == 0)
+					{
+						stamps[p] = __builtin_amdgcn_s_memrealtime();
+					}
+				}
+				// the first wavefront collects the values of all slots of this XCD
+				if (tid < 64)
+				{
+					if (MODE == 0)
+					{
+						if (tid == 0 && !s_dead)
+						{
+							const unsigned want = static_cast<unsigned>(expected_per_xcd) * static_cast<unsigned>(p + 1);
+							int spins = 0;
+							while (mb_l2_atomic_add(counter, 0u) < want)
+							{
+								if (++spins > spin_limit)
+								{
+									s_dead = 1;
+									atomicExch(err, 1);
+									break;
+								}
+							}
+						}
+						__builtin_amdgcn_wave_barrier();
+					}
+					unsigned mine = 0;
+					if (tid < expected_per_xcd)
+					{
+						const unsigned long long* src = values + (p & 1) * 32 + tid;
+						unsigned long long got = mb_load_past_l1<kDevice>(src);
+						if (MODE != 0)
+						{
+							int spins = 0;
+							while (static_cast<unsigned>(got >> 32) != static_cast<unsigned>(p + 1) && !s_dead)
+							{
+								if (++spins > spin_limit)
+								{
+									s_dead = 1;
+									atomicExch(err, 1);
+									break;
+								}
+								got = mb_load_past_l1<kDevice>(src);
+							}
+						}
+						mine = static_cast<unsigned>(got);
+					}
+					// the next value: the sum of the XCD's values plus one
+					for (int o = 32; o; o >>= 1)
+					{
+						mine += __shfl_xor(mine, o);
+					}
+					if (tid == 0)
+					{
+						s_value = mine + 1u;
+					}
+				}
+				__syncthreads();
+			}
+			if (tid == 0)
+			{
+				result[blockIdx.x * 2] = s_value;
+				result[blockIdx.x * 2 + 1] = xcc * 64u + static_cast<unsigned>(slot);
+			}
+		}
 	} // namespace
 } // namespace litenn_hip
 
@@ -282,5 +524,59 @@ extern "C" int litenn_hip_mb_mix(int mfma, int reads, int valu, int sync, void* 
 		return fail("launch the instruction-mix kernel", "this combination of mfma, reads and valu is not built");
 	}
 	LITENN_HIP_TRY("launch the instruction-mix kernel", hipGetLastError());
+	return 0;
+}
+
+// The exchange among the workgroups of one XCD (see mb_xcd_exchange_kernel): `blocks` workgroups of
+// 512 threads with 90 KB of LDS each (one per CU), `phases` phases, each wait bounded by
+// `spin_limit` polls.  mode 0: counter in the L2; 1: values that carry their phase, polled past the
+// L1; 2: the same with device-scope accesses; 3: flags polled by atomics in the L2, values by ordinary
+// stores and loads at fresh addresses; 4: like 3 with the flags polled by device-scope loads.  `mem` is
+// 8 KB (modes 3 and 4: 8 KB + phases * 2 KB) of device memory that this call clears;
+// result (2 x blocks words) receives each workgroup's final value and 64 * XCD + slot; err (one int,
+// cleared by this call) is 0 when no wait ran out, 1 when one did, 2 when an XCD received more than
+// 32 workgroups; stamps (phases entries, or null) receives workgroup 0's 100 MHz clock per phase.
+extern "C" int litenn_hip_mb_xcd_exchange(int mode, int blocks, int phases, int spin_limit, int expected_per_xcd, void* mem,
+                                          void* err, void* result, void* stamps, void* stream)
+{
+	using namespace litenn_hip;
+	if (!mem || !err || !result || blocks < 1 || blocks > 256 || phases < 1 || spin_limit < 1 || expected_per_xcd < 1 ||
+	    expected_per_xcd > 32 || mode < 0 || mode > 4 || (mode >= 3 && phases > 4000))
+	{
+		return fail("launch the XCD exchange kernel", "null buffer or arguments out of range");
+	}
+	hipStream_t st = static_cast<hipStream_t>(stream);
+	LITENN_HIP_TRY("launch the XCD exchange kernel",
+	               hipMemsetAsync(mem, 0, 8192 + (mode >= 3 ? static_cast<size_t>(phases) * 2048 : 0), st));
+	LITENN_HIP_TRY("launch the XCD exchange kernel", hipMemsetAsync(err, 0, sizeof(int), st));
+	unsigned* m = static_cast<unsigned*>(mem);
+	int* e = static_cast<int*>(err);
+	unsigned* r = static_cast<unsigned*>(result);
+	unsigned long long* t = static_cast<unsigned long long*>(stamps);
+	const size_t lds = 90 * 1024;
+	switch (mode)
+	{
+	case 0:
+		allow_dynamic_lds(reinterpret_cast<const void*>(&mb_xcd_exchange_kernel<0>), 128 * 1024);
+		mb_xcd_exchange_kernel<0><<<dim3(blocks), dim3(512), lds, st>>>(m, phases, spin_limit, expected_per_xcd, e, r, t);
+		break;
+	case 1:
+		allow_dynamic_lds(reinterpret_cast<const void*>(&mb_xcd_exchange_kernel<1>), 128 * 1024);
+		mb_xcd_exchange_kernel<1><<<dim3(blocks), dim3(512), lds, st>>>(m, phases, spin_limit, expected_per_xcd, e, r, t);
+		break;
+	case 2:
+		allow_dynamic_lds(reinterpret_cast<const void*>(&mb_xcd_exchange_kernel<2>), 128 * 1024);
+		mb_xcd_exchange_kernel<2><<<dim3(blocks), dim3(512), lds, st>>>(m, phases, spin_limit, expected_per_xcd, e, r, t);
+		break;
+	case 3:
+		allow_dynamic_lds(reinterpret_cast<const void*>(&mb_xcd_exchange_kernel<3>), 128 * 1024);
+		mb_xcd_exchange_kernel<3><<<dim3(blocks), dim3(512), lds, st>>>(m, phases, spin_limit, expected_per_xcd, e, r, t);
+		break;
+	default:
+		allow_dynamic_lds(reinterpret_cast<const void*>(&mb_xcd_exchange_kernel<4>), 128 * 1024);
+		mb_xcd_exchange_kernel<4><<<dim3(blocks), dim3(512), lds, st>>>(m, phases, spin_limit, expected_per_xcd, e, r, t);
+		break;
+	}
+	LITENN_HIP_TRY("launch the XCD exchange kernel", hipGetLastError());
 	return 0;
 }

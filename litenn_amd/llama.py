@@ -87,6 +87,12 @@ class LLaMA:
     def past(self) -> int:
         return _lib.load().litenn_hip_llama_past(self._h)
 
+    @property
+    def block_form(self) -> int:
+        """1: a block's attention half runs as one launch in the single-token step; -1: as separate
+        launches; 0: not decided yet."""
+        return _lib.load().litenn_hip_llama_block_form(self._h)
+
     def reset(self) -> None:
         check(_lib.load().litenn_hip_llama_reset(self._h))
 

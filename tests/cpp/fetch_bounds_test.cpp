@@ -472,12 +472,125 @@ static void test_attention_tiles()
 	std::printf("attention tiles: %ld query tiles walked\n", cases);
 }
 
+// ---- decoder-block kernel: rows dealt out per team, column segments of the output projection ----
+static void test_team_rows_and_segments()
+{
+	long cases = 0;
+	// first phase: every row of every matrix is walked exactly once over the eight teams
+	for (int n0 : { 4096, 2048, 1024 })
+	{
+		for (int n1 : { 4096, 1024, 512, 0 })
+		{
+			const int n2 = n1;
+			std::vector<int> seen0(n0, 0), seen1(n1, 0), seen2(n2, 0);
+			const int per_team = (n0 >> 3) + (n1 >> 3) + (n2 >> 3);
+			for (int team = 0; team < 8; ++team)
+			{
+				for (int v = 0; v < per_team; ++v)
+				{
+					const fm::TeamRow r = fm::team_row(v, team, n0, n1, n2);
+					std::vector<int>& seen = r.m == 0 ? seen0 : (r.m == 1 ? seen1 : seen2);
+					CHECK(r.m >= 0 && r.m <= 2 && r.local >= 0 && r.local < static_cast<int>(seen.size()),
+					      "team %d row %d -> matrix %d row %d", team, v, r.m, r.local);
+					if (r.local >= 0 && r.local < static_cast<int>(seen.size()))
+					{
+						++seen[r.local];
+					}
+					++cases;
+				}
+			}
+			for (const std::vector<int>* seen : { &seen0, &seen1, &seen2 })
+			{
+				for (size_t i = 0; i < seen->size(); ++i)
+				{
+					CHECK((*seen)[i] == 1, "n %d %d: row %zu walked %d times", n0, n1, i, (*seen)[i]);
+				}
+			}
+		}
+	}
+	// third phase: 4096 x 4096 output projection, team t owns 512 columns (two 256-element chunks) of
+	// every row; a wavefront's fetch holds the segments of eight consecutive rows and must look like a
+	// 4096-wide slice of a row made of those segments
+	for (const Format& f : kFormats)
+	{
+		const int seg_bytes = 2 * f.chunk_bytes;
+		if (seg_bytes % 16 != 0)
+		{
+			continue; // the launcher sends such a format down the separate launches
+		}
+		const int n = 4096, row_bytes = 16 * f.chunk_bytes, seg_pieces = seg_bytes / 16, rows_per_fetch = 8;
+		CHECK(seg_pieces * rows_per_fetch * 16 == f.stream_slice, "%s: eight segments are not one slice", f.name);
+		const int loads = (f.stream_slice + 1023) / 1024;
+		const uintptr_t base = 7 * kPage; // page-exact tensor: 4096 rows x 16 chunks
+		const uintptr_t end = base + static_cast<size_t>(n) * row_bytes;
+		std::vector<unsigned char> covered(static_cast<size_t>(n) * row_bytes, 0);
+		for (int block = 0; block < 256; ++block)
+		{
+			const int team = block & 7, place = block >> 3;
+			for (int wave = 0; wave < 8; ++wave)
+			{
+				for (int fetch = 0; fetch < 2; ++fetch)
+				{
+					const int row0 = place * 128 + (wave * 2 + fetch) * rows_per_fetch;
+					std::map<int, uintptr_t> slot;
+					for (int i = 0; i < loads; ++i)
+					{
+						for (int lane = 0; lane < 64; ++lane)
+						{
+							const fm::SegmentPiece sp = fm::segment_piece(i, lane, seg_pieces, rows_per_fetch);
+							if (!sp.issued)
+							{
+								continue;
+							}
+							CHECK(sp.row >= 0 && sp.row < rows_per_fetch && sp.offset + 16 <= static_cast<uint32_t>(seg_bytes),
+							      "%s: piece row %d offset %u", f.name, sp.row, sp.offset);
+							const uintptr_t from = base + static_cast<size_t>(row0 + sp.row) * row_bytes +
+							                       static_cast<size_t>(team) * seg_bytes + sp.offset;
+							CHECK(from % 16 == 0 && from >= base && from + 16 <= end, "%s: piece at %#zx outside the tensor", f.name,
+							      static_cast<size_t>(from));
+							slot[1024 * i + 16 * lane] = from;
+							if (from >= base && from + 16 <= end)
+							{
+								for (int b = 0; b < 16; ++b)
+								{
+									++covered[from - base + b];
+								}
+							}
+							++cases;
+						}
+					}
+					// the slot, read as a slice: byte b of row r's segment sits at r * seg_bytes + b
+					for (int r = 0; r < rows_per_fetch; ++r)
+					{
+						for (int b = 0; b < seg_bytes; b += 16)
+						{
+							const auto it = slot.find(r * seg_bytes + b);
+							const uintptr_t want = base + static_cast<size_t>(row0 + r) * row_bytes + static_cast<size_t>(team) * seg_bytes + b;
+							CHECK(it != slot.end() && it->second == want, "%s: slot byte %d of row %d", f.name, b, r);
+						}
+					}
+				}
+			}
+		}
+		for (size_t i = 0; i < covered.size(); ++i)
+		{
+			if (covered[i] != 1)
+			{
+				CHECK(false, "%s: byte %zu of the projection fetched %d times", f.name, i, covered[i]);
+				break;
+			}
+		}
+	}
+	std::printf("team rows and column segments: %ld rows and pieces walked\n", cases);
+}
+
 int main()
 {
 	test_gemm_weight_pieces();
 	test_gemm_stream_pieces();
 	test_stream_rows_and_pieces();
 	test_attention_tiles();
+	test_team_rows_and_segments();
 	if (g_failures)
 	{
 		std::printf("%d checks failed\n", g_failures);
