@@ -15,8 +15,9 @@ The same JSON line carries
     with the CPU checker's tokens per second beside it;
   * `decode_8b`: the 8B GQA shape with mixed Q4_K / Q6_K weights, prompt 512 + 512 tokens at
     context 4096;
-  * with --microbench, `microbench`: an empty kernel, a read-only kernel and the GEMV's in-kernel
-    timeline.
+  * with --microbench, `microbench`: an empty kernel, a read-only kernel, the GEMV's in-kernel
+    timeline, the matrix-core GEMM's instruction mix, what a meeting of the workgroups of one XCD
+    costs inside a launch, and the decoder-block kernel's in-kernel timeline.
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-decode] [--no-cpu] [--no-gemm]
        [--no-configs] [--microbench]
@@ -418,6 +419,17 @@ def microbench(ln, hiprt, fmt, n, k, n_buffers=16, replays=8):
                             "256 workgroups, shader-clock cycles of the slowest wavefront of a workgroup")
     cyc.free()
     out["xcd_exchange"] = xcd_exchange(ln, hiprt, tl, ok, stream)
+    # the decoder-block kernel's timeline needs the timeline build as THE library: a child process
+    import subprocess
+    child = subprocess.run([sys.executable, os.path.abspath(__file__), "--block-timeline"], capture_output=True, text=True,
+                           timeout=300)
+    if child.returncode == 0 and child.stdout.strip():
+        out["block_timeline"] = json.loads(child.stdout.strip().splitlines()[-1])
+        for pt in out["block_timeline"]["timeline"]:
+            log(f"[bench] microbench: decoder-block kernel, {pt['point']:40s} mean {pt['mean_us']:6.2f} us  earliest "
+                f"{pt['earliest_us']:6.2f}  latest {pt['latest_us']:6.2f}")
+    else:
+        log("[bench] microbench: the decoder-block timeline did not run: " + child.stderr.strip()[-300:])
     for w in weights:
         w.free()
     for tns in (x, y, sink):
@@ -469,6 +481,53 @@ def xcd_exchange(ln, hiprt, tl, ok, stream, phases=2000, blocks=256):
     for t in (mem, err, result, stamps):
         t.free()
     return out
+
+
+def block_timeline(past=200, steps=6):
+    """The decoder-block kernel's own timeline (csrc/attn_block.inc) from the timeline build of the library:
+    a four-block model of the 7B shape's attention half (4096 wide, 32 heads of 128, Q4_0, small
+    feed-forward part and vocabulary), `past` cached rows, single-token steps launched kernel by
+    kernel; the last block's launch of every step leaves its stamps.  Runs in a process of its own
+    (`python bench.py --block-timeline`): the library this process loads is the timeline build."""
+    import ctypes as C
+    os.environ["LITENN_HIP_GRAPH"] = "0"
+    from litenn_amd import _lib, build as hip_build
+    _lib.LIB_PATH = hip_build.TRACE_LIB_PATH
+    import litenn_amd as ln
+    from litenn_amd import synth
+    from litenn_amd.formats import DT_F16, Q4_0
+    cfg = synth.tiny_llama(Q4_0, block_count=4, d_model=4096, heads=32, kv_heads=32, ff=256, vocab=256,
+                           context_length=past + steps + 8)
+    model = ln.LLaMA.from_config(cfg, kv_dtype=DT_F16)
+    for item in synth.llama_tensors(cfg, 3):
+        model.set_tensor(*item)
+    toks = synth.prompt_tokens(cfg, past + steps + 2, 1)
+    model.eval(toks[:past], all_logits=False, precise=False)
+    lib = _lib.load()
+    lib.litenn_hip_block_trace_read.argtypes = [C.c_void_p, C.c_size_t]
+    waves, slots = 2048, 8
+    buf = (C.c_ulonglong * (waves * slots))()
+    acc = []
+    for t in toks[past:past + steps + 2]:
+        model.eval([t], all_logits=False)
+        if lib.litenn_hip_block_trace_read(buf, waves * slots) != 0:
+            raise RuntimeError(lib.litenn_hip_last_error().decode())
+        a = np.frombuffer(buf, np.uint64).reshape(waves, slots).astype(np.float64)
+        acc.append((a - a[:, 0].min()) * 0.01)  # 100 MHz ticks -> us after the launch's first wavefront entered
+    form = model.block_form
+    model.close()
+    a = np.stack(acc[2:])
+    names = ["entry", "first phase's rows stored", "first meeting passed", "second phase's triple stored",
+             "second meeting passed", "third phase's activations in registers", "end"]
+    points = []
+    for s_, name in enumerate(names):
+        col = a[:, :, s_]
+        points.append({"point": name, "mean_us": round(float(col.mean()), 2),
+                       "earliest_us": round(float(col.min(axis=1).mean()), 2),
+                       "latest_us": round(float(col.max(axis=1).mean()), 2)})
+    return {"block_form": form, "cached_rows": past, "steps": steps, "timeline": points,
+            "note": "us after the launch's first wavefront entered the kernel, over all 2048 wavefronts of the last "
+                    "block's launch; earliest / latest are per-launch extremes, averaged over the steps"}
 
 
 def bench_cpu_baseline(fmt, n, k, budget_s=8.0):
@@ -676,6 +735,8 @@ def main() -> int:
     ap.add_argument("--gemm-case", default=None, help="run only this prefill case, e.g. Q4_K:512")
     ap.add_argument("--microbench", action="store_true",
                     help="also measure an empty kernel, a read-only kernel and the GEMV's in-kernel timeline")
+    ap.add_argument("--block-timeline", action="store_true",
+                    help="print the decoder-block kernel's in-kernel timeline (timeline build of the library) and exit")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch a known-size streaming kernel (profiler counter calibration)")
     args = ap.parse_args()
@@ -683,6 +744,10 @@ def main() -> int:
         print("bench.py measures one GPU: this path has nothing sharded or exchanged between GPUs; "
               "run with --gpus 1", file=sys.stderr)
         return 2
+
+    if args.block_timeline:
+        print(json.dumps(block_timeline()), flush=True)
+        return 0
 
     import litenn_amd as ln
     from litenn_amd import hiprt

@@ -31,8 +31,12 @@ def make_cfg(case, blocks=2, context=96, **extra):
               context_length=context)
     if c["formats"]:
         kw["formats"] = c["formats"]
+    rope_dims = extra.pop("rope_dimension_count", 0)
     kw.update(extra)
-    return synth.tiny_llama(c["fmt"], **kw)
+    cfg = synth.tiny_llama(c["fmt"], **kw)
+    if rope_dims:
+        cfg.rope_dimension_count = rope_dims
+    return cfg
 
 
 @pytest.fixture
@@ -107,6 +111,29 @@ def test_greedy_loop_is_token_exact_and_replays(hip, oracle):
     for i in range(8):
         assert int(np.argmax(lg)) == want[i]
         lg = dev.eval([want[i]], all_logits=False)
+    dev.close()
+
+
+@pytest.mark.parametrize("case,past,rope_dims", [("q4_0-32kv", 7, 0), ("q4_0-32kv", 8, 64), ("q4_k-q6_k-8kv", 9, 0),
+                                                 ("q4_k-16kv", 65, 32), ("q4_k-q6_k-8kv", 1100, 0)])
+def test_cache_lengths_around_the_chunk_boundaries_and_partial_rotation(hip, oracle, case, past, rope_dims):
+    """A head's cached keys are cut into eight chunks of ceil(len / 8): lengths below, at and just above
+    eight keys leave chunks empty or one key long, 65 keys put a second step into the key loop's last
+    lanes, 1100 walk several steps per chunk (the 8B shape's lengths); with rope.dimension_count below
+    the head width some lanes rotate nothing.  One block, logits against the checker reading the
+    device's cache, for the steps that take the cache from `past` to `past + 4` rows."""
+    cfg = make_cfg(case, blocks=1, context=past + 8, **({"rope_dimension_count": rope_dims} if rope_dims else {}))
+    toks = synth.prompt_tokens(cfg, past + 4, 3)
+    dev = hip_model(hip, cfg, 13)
+    ref = oracle_model(oracle, cfg, 13)
+    dev.eval(toks[:past], all_logits=False)
+    ref.eval(toks[:past], all_logits=False)
+    adopt_device_cache(ref, dev, 1, slack=2e-5)
+    for t in toks[past:]:
+        got, want = dev.eval([t], all_logits=False), ref.eval([t], all_logits=False)
+        assert rel_l2(got, want) < 3e-4, (case, dev.past)
+        adopt_device_cache(ref, dev, 1, slack=2e-5)
+    assert dev.block_form == 1 and dev.past == past + 4
     dev.close()
 
 
