@@ -2135,7 +2135,8 @@ namespace litenn_hip
 	// The attention half of a decoder block for one new row as one launch (attn_block.inc).  Returns
 	// false, with nothing launched, when the shape is not one the kernel is built for: 4096-wide model,
 	// 32 heads of 128, a KV head count that is a multiple of 8, a Float16 cache, a card of 256 CUs, and
-	// one of the format combinations instantiated below.  plan_only launches nothing in either case.
+	// one of the format combinations instantiated below (one format throughout, or q, k and the output
+	// projection in Q4_K / Q5_K beside a Q6_K v).  plan_only launches nothing in either case.
 	// scratch: q / k / v take the first phase's rows (n_head * 128 and n_kv_head * 128 twice), triples
 	// n_head * 8 * 132 floats, flags 512 words (zero before the model's first launch), y_partial 8 * d
 	// floats; counters = {position, tokens emitted, steps run}; bit 1 of *err is set when a wait inside
@@ -2161,35 +2162,45 @@ namespace litenn_hip
 		AttnBlockPlan plan{};
 		GemvArgs a0, a1;
 		bool ok = false;
-		int variant = -1;
-		if (fmts[0] == fmts[1] && fmts[1] == fmts[2] && fmt_o == fmts[0] && (fmts[0] == LITENN_FMT_Q4_0 || fmts[0] == LITENN_FMT_Q4_K))
+		const bool one_format = fmts[0] == fmts[1] && fmts[1] == fmts[2] && fmt_o == fmts[0];
+		// q and k in one K-quant format beside a Q6_K v, the attn_v choice of llama.cpp's K-quant mixes
+		const bool k_mix = fmts[0] == fmts[1] && fmts[2] == LITENN_FMT_Q6_K && fmt_o == fmts[0] &&
+		                   (fmts[0] == LITENN_FMT_Q4_K || fmts[0] == LITENN_FMT_Q5_K);
+		if (one_format)
 		{
 			if (!fill_args(a0, fmts[0], 3, wqkv, ys, n_qkv, d, x, nullptr, norm_w, eps, false))
 			{
 				return false;
 			}
 			a1 = a0;
-			if (fmts[0] == LITENN_FMT_Q4_0)
-			{
-				variant = 0;
-				ok = plan_attn_block<Q4_0Unit, Q4_0Unit, Q4_0Unit>(plan, a0, a1, false);
-			}
-			else
-			{
-				variant = 2;
-				ok = plan_attn_block<Q4_KUnit, Q4_KUnit, Q4_KUnit>(plan, a0, a1, false);
-			}
 		}
-		else if (fmts[0] == LITENN_FMT_Q4_K && fmts[1] == LITENN_FMT_Q4_K && fmts[2] == LITENN_FMT_Q6_K && fmt_o == LITENN_FMT_Q4_K)
+		else if (k_mix)
 		{
 			if (!fill_args(a0, fmts[0], 2, wqkv, ys, n_qkv, d, x, nullptr, norm_w, eps, false) ||
 			    !fill_args(a1, fmts[2], 1, wqkv + 2, ys + 2, n_qkv + 2, d, x, nullptr, norm_w, eps, false))
 			{
 				return false;
 			}
-			variant = 1;
-			ok = plan_attn_block<Q4_KUnit, Q6_KUnit, Q4_KUnit>(plan, a0, a1, true);
 		}
+		else
+		{
+			return false;
+		}
+		// the instances: every block format whose 512-column segment of a row is a whole number of
+		// 16-byte pieces (Q2_K, Q3_K and Q6_K output projections are not)
+#define LITENN_BLOCK_INSTANCE(DO)                                                                                      \
+	if (one_format && fmts[0] == LITENN_FMT_Q4_0) { DO(Q4_0Unit, Q4_0Unit, Q4_0Unit, false); }                         \
+	else if (one_format && fmts[0] == LITENN_FMT_Q4_1) { DO(Q4_1Unit, Q4_1Unit, Q4_1Unit, false); }                    \
+	else if (one_format && fmts[0] == LITENN_FMT_Q5_0) { DO(Q5_0Unit, Q5_0Unit, Q5_0Unit, false); }                    \
+	else if (one_format && fmts[0] == LITENN_FMT_Q5_1) { DO(Q5_1Unit, Q5_1Unit, Q5_1Unit, false); }                    \
+	else if (one_format && fmts[0] == LITENN_FMT_Q8_0) { DO(Q8_0Unit, Q8_0Unit, Q8_0Unit, false); }                    \
+	else if (one_format && fmts[0] == LITENN_FMT_Q4_K) { DO(Q4_KUnit, Q4_KUnit, Q4_KUnit, false); }                    \
+	else if (one_format && fmts[0] == LITENN_FMT_Q5_K) { DO(Q5_KUnit, Q5_KUnit, Q5_KUnit, false); }                    \
+	else if (k_mix && fmts[0] == LITENN_FMT_Q4_K) { DO(Q4_KUnit, Q6_KUnit, Q4_KUnit, true); }                          \
+	else if (k_mix && fmts[0] == LITENN_FMT_Q5_K) { DO(Q5_KUnit, Q6_KUnit, Q5_KUnit, true); }
+#define LITENN_BLOCK_PLAN(U0, U1, UO, TWO) ok = (plan_attn_block<U0, U1, UO>(plan, a0, a1, TWO))
+		LITENN_BLOCK_INSTANCE(LITENN_BLOCK_PLAN)
+#undef LITENN_BLOCK_PLAN
 		if (!ok)
 		{
 			return false;
@@ -2220,12 +2231,10 @@ namespace litenn_hip
 		f.rope_dims = static_cast<int>(rope_dims);
 		f.d = static_cast<int>(d);
 		f.spin_limit = spin_limit;
-		switch (variant)
-		{
-		case 0: launch_attn_block_variant<Q4_0Unit, Q4_0Unit, Q4_0Unit>(plan, stream); break;
-		case 1: launch_attn_block_variant<Q4_KUnit, Q6_KUnit, Q4_KUnit>(plan, stream); break;
-		default: launch_attn_block_variant<Q4_KUnit, Q4_KUnit, Q4_KUnit>(plan, stream); break;
-		}
+#define LITENN_BLOCK_LAUNCH(U0, U1, UO, TWO) launch_attn_block_variant<U0, U1, UO>(plan, stream)
+		LITENN_BLOCK_INSTANCE(LITENN_BLOCK_LAUNCH)
+#undef LITENN_BLOCK_LAUNCH
+#undef LITENN_BLOCK_INSTANCE
 		return true;
 	}
 

@@ -10,7 +10,7 @@ import pytest
 
 from conftest import rel_l2
 from litenn_amd import synth
-from litenn_amd.formats import DT_F16, DT_F32, Q4_0, Q4_K, Q6_K, Q8_0
+from litenn_amd.formats import DT_F16, DT_F32, Q4_0, Q4_1, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0
 from llama_util import adopt_device_cache, hip_model, oracle_model
 
 pytestmark = pytest.mark.gpu
@@ -93,6 +93,27 @@ def test_single_token_steps_match_the_checker(hip, oracle, case, block_launch_en
     plain.close()
 
 
+@pytest.mark.parametrize("fmt,mix", [(Q4_1, None), (Q5_0, None), (Q5_1, None), (Q5_K, None), (Q5_K, Q6_K)])
+def test_the_other_formats_with_an_instance(hip, oracle, fmt, mix):
+    formats = {"default": fmt}
+    if mix is not None:
+        formats.update({"attn_v": mix, "ffn_down": mix, "output": mix})
+    cfg = synth.tiny_llama(fmt, block_count=2, d_model=4096, heads=32, kv_heads=8, ff=2048, vocab=444, context_length=48,
+                           formats=formats)
+    toks = synth.prompt_tokens(cfg, 24, 2)
+    dev = hip_model(hip, cfg, 17)
+    ref = oracle_model(oracle, cfg, 17)
+    dev.eval(toks[:18], all_logits=False)
+    ref.eval(toks[:18], all_logits=False)
+    adopt_device_cache(ref, dev, 2, slack=2e-5, deeper_slack=2e-2)
+    for t in toks[18:]:
+        got, want = dev.eval([t], all_logits=False), ref.eval([t], all_logits=False)
+        assert rel_l2(got, want) < 5e-4, (fmt, mix, dev.past)
+        adopt_device_cache(ref, dev, 2, slack=2e-5, deeper_slack=2e-2)
+    assert dev.block_form == 1
+    dev.close()
+
+
 def test_greedy_loop_is_token_exact_and_replays(hip, oracle):
     """The captured step with the one-launch attention half: the device's greedy tokens equal the
     checker's, a second run replays the graph, and stepping from the host gives the same tokens."""
@@ -164,7 +185,8 @@ def test_waits_that_run_out_send_the_model_down_the_separate_launches(hip, oracl
 
 
 def test_shapes_the_launch_is_not_built_for_keep_the_separate_launches(hip, oracle):
-    for kw in (dict(fmt=Q8_0, d_model=4096, heads=32, kv_heads=32),   # a format without an instance
+    for kw in (dict(fmt=Q8_0, d_model=4096, heads=32, kv_heads=32),   # row slots that do not fit the CU's LDS
+               dict(fmt=Q6_K, d_model=4096, heads=32, kv_heads=8),    # column segments of 420 bytes
                dict(fmt=Q4_0, d_model=2048, heads=16, kv_heads=16),   # another width
                dict(fmt=Q4_0, d_model=4096, heads=32, kv_heads=4)):   # KV heads not a multiple of 8
         fmt = kw.pop("fmt")
