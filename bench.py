@@ -123,59 +123,69 @@ def bench_gemv(ln, hiprt, fmt, n, k, steps, warmup, n_buffers, seed=1, graph_rot
     # graph costs about 13 us on the device whatever it holds (measured with empty kernels: 14.4 us
     # for a graph of one, 1.58 us per kernel in a graph of 256, 1.53 us per kernel launched
     # directly), so a graph holds up to 16 rotations; exactly `steps` kernels run, all from graphs.
-    # A short run (fewer than 64 steps) is launched directly instead: the host issues a launch in
-    # about 4 us, less than one takes, and the graph's start would weigh on so few kernels.
-    graph_len = min(steps, graph_rotations * n_buffers) if steps >= 64 else 0
+    # A short run (fewer than 64 steps) is timed as the difference of two graphs: SHORT_RUN_PRIMING
+    # launches followed by the `steps` timed ones, and the SHORT_RUN_PRIMING launches alone, each
+    # between two events, the median of SHORT_RUN_REPEATS replays each.  The timed launches then
+    # follow others back to back on the device, as they do in a long run, and what every graph
+    # replay pays once (its start, the two events) cancels.  Other ways to time 20 launches, all
+    # measured: a graph of the 20 alone pays its start (8.3 us per launch where the long run gives
+    # 7.6); event nodes inside one graph of 64 + 20 launches cost about 5 us themselves (7.9 to 8.2);
+    # launched directly, one host call per kernel, the host is the limit (8.25).
+    graph_len = min(steps, graph_rotations * n_buffers)
 
-    def capture(count):
+    def capture(count, first=0):
         stream.begin_capture()
         for i in range(count):
-            launch(i)
+            launch(first + i)
         g = stream.end_capture()
         g.launch(stream)  # untimed: the first replay uploads the graph
         stream.synchronize()
         return g
 
-    graph = capture(graph_len) if graph_len else None
-    priming = None if graph_len else capture(DIRECT_PRIMING)
-    rest = capture(steps % graph_len) if graph_len and steps % graph_len else None
+    def timed(graphs):
+        e0.record(stream)
+        for g in graphs:
+            g.launch(stream)
+        e1.record(stream)
+        stream.synchronize()
+        return e0.elapsed_ms(e1)
+
+    short_run = steps < 64
     e0, e1 = hiprt.Event(), hiprt.Event()
-    hiprt.device_synchronize()
-    if graph is None:
-        # A short run starts on a queue that is already busy: a graph of DIRECT_PRIMING untimed
-        # launches goes out right before the first event with no synchronisation in between, and the
-        # host issues the timed launches while the device works through it (a direct launch costs
-        # the host about as long as the kernel runs, so launches issued one by one onto an idle
-        # queue would be timed at the host's pace).  The timed launches then follow each other back
-        # to back on the device, as they do in the replayed graphs of a long run.
-        priming.launch(stream)
-    t0 = time.perf_counter()
-    e0.record(stream)
-    if graph is None:
-        for i in range(steps):
-            launch(DIRECT_PRIMING + i)
+    if short_run:
+        graphs = [capture(SHORT_RUN_PRIMING + steps), capture(SHORT_RUN_PRIMING)]
+        hiprt.device_synchronize()
+        t0 = time.perf_counter()
+        both, priming = [], []
+        for _ in range(SHORT_RUN_REPEATS):  # alternating, so that a clock change touches both alike
+            both.append(timed(graphs[:1]))
+            priming.append(timed(graphs[1:]))
+        both, priming = float(np.median(both)), float(np.median(priming))
+        hiprt.device_synchronize()
+        wall_launches = SHORT_RUN_REPEATS * (2 * SHORT_RUN_PRIMING + steps)
+        event_ms = both - priming
     else:
-        for _ in range(steps // graph_len):
-            graph.launch(stream)
-        if rest is not None:
-            rest.launch(stream)
-    e1.record(stream)
-    stream.synchronize()
-    hiprt.device_synchronize()
+        graphs = [capture(graph_len)] * (steps // graph_len)
+        if steps % graph_len:
+            graphs.append(capture(steps % graph_len))
+        hiprt.device_synchronize()
+        t0 = time.perf_counter()
+        event_ms = timed(graphs)
+        hiprt.device_synchronize()
+        wall_launches = steps
     wall_ms = (time.perf_counter() - t0) * 1e3
-    event_ms = e0.elapsed_ms(e1)
-    for g in (graph, rest, priming):
-        if g is not None:
-            g.destroy()
+    for g in set(graphs):
+        g.destroy()
     result = y.numpy()
     assert np.all(np.isfinite(result))
     for w in weights:
         w.free()
     stream.destroy()
-    bench_gemv.last_mode = (f"graphs of {graph_len} launches replayed" if graph_len else
-                            f"launched directly behind a graph of {DIRECT_PRIMING} untimed launches on the same "
-                            f"stream (no synchronisation between it and the timed ones)")
-    return event_ms / steps, wall_ms / steps
+    bench_gemv.last_mode = (f"graphs of {graph_len} launches replayed" if not short_run else
+                            f"a graph of {SHORT_RUN_PRIMING} + {steps} launches minus a graph of {SHORT_RUN_PRIMING} "
+                            f"launches, each between two events, the median of {SHORT_RUN_REPEATS} replays each "
+                            f"(the wall figure is over all of their launches, graph starts included)")
+    return event_ms / steps, wall_ms / wall_launches
 
 
 def traffic_probe(ln, launches=8, n_elems=16 * 1024 * 1024):
@@ -194,7 +204,8 @@ def traffic_probe(ln, launches=8, n_elems=16 * 1024 * 1024):
         f"{4 * n_elems} B written each")
 
 
-DIRECT_PRIMING = 64  # untimed launches (one graph) queued right before a directly launched (short) timed run
+SHORT_RUN_PRIMING = 64  # launches that precede the timed ones in a short run
+SHORT_RUN_REPEATS = 15
 
 
 FP16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 matrix rate
