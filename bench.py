@@ -62,7 +62,15 @@ def traffic_source():
                              timeout=10).stdout.strip()
     except (OSError, subprocess.SubprocessError):
         rev = ""
-    return {"file": rel, "commit": rev or None,
+    try:
+        import hashlib
+        with open(TRAFFIC_SUMMARY, "rb") as f:
+            digest = hashlib.sha256(f.read()).hexdigest()[:16]
+    except OSError:
+        digest = None
+    # the commit is known only where the git history is at hand; the digest names the file's
+    # contents everywhere (sha256sum <file> | cut -c1-16)
+    return {"file": rel, "commit": rev or None, "sha256_16": digest,
             "note": "a property of the kernel and the shape, measured with rocprofv3 --pmc when the kernel last "
                     "changed; not re-measured by this run"}
 
