@@ -829,7 +829,10 @@ extern "C" int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t 
 		const size_t need = 2 * gemm_scratch_halves(m, k);
 		// room for more m x n products behind it lets K be walked in parts
 		const size_t need16 = (need + 15) & ~size_t{ 15 };
-		const size_t with_partial = need16 + sizeof(float) * m * n * (m <= 64 ? 3 : 1);
+		// (three more products, so that K can be walked in four ranges, while a product is at most 16 MB:
+		// larger products belong to launches that fill the card without ranges)
+		const bool small_product = m * n <= (size_t{ 4 } << 20);
+		const size_t with_partial = need16 + sizeof(float) * m * n * (small_product ? 3 : 1);
 		if (workspace)
 		{
 			if (workspace_bytes < need)
@@ -847,7 +850,7 @@ extern "C" int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t 
 		}
 		// none given: this call takes one in stream order and returns it the same way
 		StreamScratch scratch(s);
-		const bool splits = (k >= 8192 && m >= 128) || m <= 64;
+		const bool splits = (k >= 8192 && m >= 128) || small_product;
 		LITENN_HIP_TRY(action, scratch.allocate(splits ? with_partial : need));
 		float* partial = splits ? reinterpret_cast<float*>(static_cast<char*>(scratch.get()) + need16) : nullptr;
 		if (!launch_gemm(fmt, wq, n, k, xf, m, yf, rf, scratch.get(), partial,

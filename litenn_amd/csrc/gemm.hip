@@ -1766,6 +1766,21 @@ namespace litenn_hip
 				// cuts K in two when the caller lends a buffer for the second product: each weight is
 				// then decoded four times instead of eight, and one pass adds the two products.
 				const int m_tiles = c.m_tiles;
+				// the most K ranges (1, 2 or 4) that keep the workgroup count within `limit`, every range at
+				// least four chunks long, and whose extra products fit the room the caller lends
+				const auto ranges = [&](long tiles, long limit) {
+					int r = 1;
+					const size_t one = static_cast<size_t>(c.m) * c.n[0];
+					while (r < 4 && tiles * (2 * r) <= limit && c.k / kChunk / (2 * r) >= 4 &&
+					       c.partial_floats >= static_cast<size_t>(2 * r - 1) * one)
+					{
+						r *= 2;
+					}
+					return r;
+				};
+				const bool may_split = split_ok && c.partial && c.count == 1;
+				const int split8 = may_split && m_tiles >= 8 ? ranges(blocks(8, 128), cus) : 1;
+				const int split4 = may_split && m_tiles >= 4 ? ranges(blocks(4, 64), c.k >= kSplitMinK ? 2L * cus : cus) : 1;
 				// (the wide tile, too, from 5/8 of the CUs on: 22016 x 4096 at M = 256, 172 workgroups,
 				// 74.9 against 84.7 us; 12288 x 4096 at M = 512, 192: 78.9 against 86.2; 5120 x 4096 at
 				// M = 1024, 160: 77.7 against 87.9; at half the CUs and below the narrower tiles win)
@@ -1781,11 +1796,28 @@ namespace litenn_hip
 					// the CUs it loses (4096 x 4096 at M = 512, 128 workgroups: 45.9 against 38.5 us)
 					pick = 818;
 				}
-				else if (split_ok && c.partial && c.partial_floats >= static_cast<size_t>(c.m) * c.n[0] && m_tiles >= 8 &&
-				         c.count == 1 && c.k >= kSplitMinK && 10 * blocks(8, 128) >= 4 * cus)
+				else if (split8 > 1 && 8 * blocks(8, 128) * split8 >= 5 * cus && (c.k >= kSplitMinK || split8 == 2))
 				{
+					// the 128-row tile on few weight rows (N = 4096): K walked in 2 or 4 ranges by as many
+					// workgroups, the ranges' products added in K order by one more pass.  Measured (us, with the
+					// pre-pass and that pass): 4096 x 11008 Q4_0 at M = 256 44.5 in four ranges against 58.5
+					// unsplit on 64 x 64 tiles, 4096 x 14336 Q6_K 65.5 against 94.3; at M = 512 two ranges,
+					// also for K = 4096 (Q6_K 4096 x 4096 43.6 against 49.1, Q4_K 38.3 against 39.5).  Four
+					// ranges of a short K do not pay (4096 x 4096 at M = 256: 28.5 against 27.4).
 					pick = 818;
-					c.k_splits = 2;
+					c.k_splits = split8;
+				}
+				else if (split4 > 1 && 2 * blocks(4, 64) * split4 >= cus && !(m_tiles < 8 && blocks(2, 64) >= cus))
+				{
+					// the 64-row tile, which decodes a weight once per 64 activation rows, on fewer workgroups
+					// than CUs: K ranges bring it to one workgroup per CU (two, which fit a CU side by side,
+					// for a long K).  Measured at M = 64: Q6_K 4096 x 4096 17.9 against 23.2 on 16-row tiles,
+					// 4096 x 14336 33.9 against 60.0, Q4_0 4096 x 11008 25.6 against 33.1, Q4_K 4096 x 4096
+					// 16.5 against 17.3; at M = 128, 4096 x 11008 33.0 against 39.0; Q6_K 1024 x 4096 at
+					// M = 256 19.9 against 24.7.  Where the 32-row tile fills the card without ranges it is
+					// as fast (8192 x 4096 at M = 64: 21.4 against 21.9) and stays.
+					pick = 414;
+					c.k_splits = split4;
 				}
 				else if (m_tiles >= 4 && 5 * blocks(4, 64) >= 4 * cus)
 				{
@@ -1816,6 +1848,15 @@ namespace litenn_hip
 					splits *= 2;
 				}
 				c.k_splits = splits;
+			}
+			// (measurement only: LITENN_HIP_GEMM_KSPLITS forces the number of K ranges for a single matrix
+			// when the caller's workspace holds the extra products and every range keeps two chunks)
+			static const int forced_splits = env_int("LITENN_HIP_GEMM_KSPLITS", 0);
+			if ((forced_splits == 2 || forced_splits == 4) && c.partial && c.count == 1 &&
+			    c.k / kChunk >= 2 * forced_splits &&
+			    c.partial_floats >= static_cast<size_t>(forced_splits - 1) * c.m * c.n[0])
+			{
+				c.k_splits = forced_splits;
 			}
 		}
 

@@ -121,6 +121,7 @@ struct litenn_hip_llama
 	size_t cap_rows = 0, cap_logit_rows = 0;
 	float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *gate = nullptr,
 	      *gate2 = nullptr, *up = nullptr, *logits = nullptr;
+	size_t xn_floats = 0; // what xn holds (rows x embedding_length, three times that for short prompts)
 	void* xh = nullptr; // fp16 copy of a matmul's activations (multi-row path), 16-row padded
 	size_t xh_halves = 0; // its size: room for the widest matmul, and for two copies of the embedding width
 	void* argmax_scratch = nullptr; // per-chunk (value, index) pairs of the vocabulary arg-max
@@ -199,7 +200,11 @@ namespace
 		{
 			drop_graph(m); // the captured step references the old buffers
 			free_scratch(m);
-			struct { float** p; size_t n; } bufs[] = { { &m->x, d }, { &m->xn, d }, { &m->q, qw }, { &m->k, kvw },
+			// xn also takes the products of K's later ranges when a GEMM on few weight rows walks K in up to
+			// four ranges at once: room for three, for prompts where that is used
+			const size_t xn_width = rows <= 1024 ? 3 * d : d;
+			m->xn_floats = rows * xn_width;
+			struct { float** p; size_t n; } bufs[] = { { &m->x, d }, { &m->xn, xn_width }, { &m->q, qw }, { &m->k, kvw },
 				                                        { &m->v, kvw }, { &m->attn, qw }, { &m->gate, ff }, { &m->gate2, ff },
 				                                        { &m->up, ff } };
 			for (auto& b : bufs)
@@ -250,12 +255,13 @@ namespace
 	// From this many rows on the prompt's attention runs tiled on the matrix cores.
 	constexpr size_t kAttnTileMinRows = 16;
 
+	// partial: null, or m->xn while it is idle (the GEMM may leave the products of K's later ranges there)
 	void matmul(litenn_hip_llama* m, const Weight& w, const float* x, size_t rows, float* y, const float* residual,
-	            unsigned flags, hipStream_t s)
+	            float* partial, unsigned flags, hipStream_t s)
 	{
 		const bool quant = w.fmt != LITENN_FMT_F16 && w.fmt != LITENN_FMT_F32;
 		if (rows >= kGemmMinRows && !(flags & LITENN_HIP_MATMUL_PRECISE) && quant && w.k % 256 == 0 &&
-		    launch_gemm(w.fmt, w.data, w.n, w.k, x, rows, y, residual, m->xh, nullptr, 0, s))
+		    launch_gemm(w.fmt, w.data, w.n, w.k, x, rows, y, residual, m->xh, partial, partial ? m->xn_floats : 0, s))
 		{
 			return;
 		}
@@ -287,7 +293,7 @@ namespace
 				n[i] = ws[i]->n;
 			}
 			if (launch_gemm_group(w0.fmt, count, w, n, w0.k, x, rows, ys, residual, norm_w, m->p.rms_norm_epsilon, up,
-			                      m->xh, partial, partial ? rows * static_cast<size_t>(m->p.embedding_length) : 0, s))
+			                      m->xh, partial, partial ? m->xn_floats : 0, s))
 			{
 				return;
 			}
@@ -305,7 +311,7 @@ namespace
 		}
 		for (int i = 0; i < count; ++i)
 		{
-			matmul(m, *ws[i], in, rows, ys[i], residual, flags, s);
+			matmul(m, *ws[i], in, rows, ys[i], residual, nullptr, flags, s);
 		}
 	}
 
@@ -541,7 +547,7 @@ namespace
 				launch_attn_decode(m->q, L.kcache, L.vcache, m->p.kv_dtype, rows, past_dev, 0, H, KH, hd, m->attn,
 				                   rows == 1 ? m->attn_splits : 1, m->attn_partial, m->attn_counters, s);
 			}
-			matmul(m, L.wo, m->attn, rows, m->x, m->x, flags, s); // x = x + attn . Wo
+			matmul(m, L.wo, m->attn, rows, m->x, m->x, m->xn, flags, s); // x = x + attn . Wo (xn is idle here)
 			const Weight* gu[2] = { &L.gate, &L.up };
 			float* gu_out[2] = { m->gate, m->up };
 			// gate = silu(x' . Wg) * (x' . Wu) straight from the launch's epilogue where the shape allows,
@@ -563,7 +569,7 @@ namespace
 		const size_t first = rows - logit_rows;
 		launch_rmsnorm(m->x + first * d, m->output_norm, m->p.rms_norm_epsilon, logit_rows, d, m->xn, s);
 		const Weight& head = m->output.data ? m->output : m->tok_embd;
-		matmul(m, head, m->xn, logit_rows, m->logits, nullptr, flags, s);
+		matmul(m, head, m->xn, logit_rows, m->logits, nullptr, nullptr, flags, s);
 	}
 
 	constexpr int kBlockWaitRanOut = -2;

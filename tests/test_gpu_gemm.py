@@ -142,23 +142,20 @@ def test_gemm_every_tile_shape(hip, oracle, fmt, m, n, k):
     assert run_case(hip, oracle, fmt, m, n, k, seed=n % 97, rows=rows, residual=(k == 512)) <= TOL
 
 
-@pytest.mark.parametrize("fmt,k", [(Q4_0, 11008), (Q6_K, 14336), (Q4_K, 8192)])
-@pytest.mark.parametrize("m", [512, 400])
-def test_long_k_is_walked_in_two_halves(hip, oracle, fmt, k, m):
-    """The down projections of the benchmark shapes (N = 4096, K = 11008 / 14336) at prompt sizes:
-    with room for a second product in the workspace two workgroups per tile share the K walk.
-    Checked against the CPU checker on a sample of weight rows (with a residual), and against the
-    same product computed without the split (same operands, other summation order)."""
+def check_k_ranges(hip, oracle, fmt, m, n, k, products):
+    """One product with a workspace that has no room for K ranges and one with room for `products`
+    more products: the two must differ (another summation order: the ranges ran) by no more than
+    f32 summation noise, the in-place form (residual aliases y, the way the decoder calls it) must
+    equal the second bit for bit, and a sample of weight rows must match the CPU checker."""
     import ctypes as C
     from litenn_amd._lib import Exec, check, load
-    n = 4096
     wq = synth.quant_weights(fmt, n, k, k % 89, 1)
     x = synth.activations(m, k, 5, 2)
     res = synth.activations(m, n, 6, 3)
     lib = load()
     w_t, x_t, r_t = hip.Tensor.from_numpy(wq), hip.Tensor.from_numpy(x), hip.Tensor.from_numpy(res)
     base = lib.litenn_hip_mul_mat_q_workspace_bytes(m, k)
-    roomy = (base + 15) // 16 * 16 + 4 * m * n
+    roomy = (base + 15) // 16 * 16 + 4 * m * n * products
     ws = hip.Tensor(((roomy + 3) // 4,))
     opts = Exec(None, 1)
     outs = []
@@ -169,17 +166,44 @@ def test_long_k_is_walked_in_two_halves(hip, oracle, fmt, k, m):
         outs.append(y.numpy())
     plain, split = outs
     assert rel_l2(split - res, plain - res) < 1e-5
-    assert not np.array_equal(split, plain)  # the split path ran
-    # in place (residual aliases y), the way the decoder calls it
+    assert not np.array_equal(split, plain)  # the ranges ran
     y = hip.Tensor.from_numpy(res)
     check(lib.litenn_hip_mul_mat_q_ws(0, fmt, w_t.ptr, n, k, x_t.ptr, 0, m, y.ptr, y.ptr, 0, ws.ptr, roomy,
                                       C.byref(opts)))
     assert np.array_equal(y.numpy(), split)
-    rows = np.sort(np.random.default_rng(k).choice(n, 256, replace=False))
+    rows = np.sort(np.random.default_rng(k).choice(n, min(n, 256), replace=False))
     rows[0], rows[-1] = 0, n - 1
     sub = np.ascontiguousarray(wq.reshape(n, row_bytes(fmt, k))[rows]).reshape(-1)
     ref = oracle.mul_mat_q(fmt, sub, len(rows), k, x)
     assert rel_l2(split[:, rows] - res[:, rows], ref) <= TOL
+    # without a workspace the call takes its own room and must give the same product
+    y = hip.mul_mat_q(fmt, w_t, n, k, x_t, residual=r_t).numpy()
+    assert rel_l2(y - res, plain - res) < 1e-5
+
+
+@pytest.mark.parametrize("fmt,k", [(Q4_0, 11008), (Q6_K, 14336), (Q4_K, 8192)])
+@pytest.mark.parametrize("m", [512, 400])
+def test_long_k_is_walked_in_two_halves(hip, oracle, fmt, k, m):
+    """The down projections of the benchmark shapes (N = 4096, K = 11008 / 14336) at prompt sizes:
+    with room for a second product in the workspace two workgroups per tile share the K walk."""
+    check_k_ranges(hip, oracle, fmt, m, 4096, k, 1)
+
+
+@pytest.mark.parametrize("fmt,m,n,k", [
+    (Q6_K, 64, 4096, 4096),     # 64-row tiles, four ranges of four chunks: one workgroup per CU
+    (Q4_K, 64, 5120, 4096),     # two ranges
+    (Q4_0, 128, 4096, 11008),   # four ranges of a long K, two workgroups per CU
+    (Q6_K, 256, 1024, 4096),    # k / v of a grouped-head model
+    (Q4_K, 512, 4096, 4096),    # 128-row tiles, two ranges of a short K
+    (Q4_0, 256, 4096, 11008),   # 128-row tiles, four ranges
+    (Q5_K, 70, 4000, 4352),     # ragged rows on both sides, 17 chunks
+    (Q2_K, 64, 4096, 2048),     # ranges of four chunks with the 84-byte blocks
+    (Q8_0, 100, 2048, 8192)])
+def test_k_ranges_on_few_weight_rows(hip, oracle, fmt, m, n, k):
+    """A matrix of few rows (N = 1024 ... 5120: output, down and grouped k / v projections) gives the
+    tall tiles fewer workgroups than the card has CUs; with room for three more products K is walked
+    in up to four ranges at once."""
+    check_k_ranges(hip, oracle, fmt, m, n, k, 3)
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
