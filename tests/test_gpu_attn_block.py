@@ -204,3 +204,40 @@ def test_shapes_the_launch_is_not_built_for_keep_the_separate_launches(hip, orac
     dev.eval([1], all_logits=False)
     assert dev.block_form == -1
     dev.close()
+
+
+def test_two_instances_stepping_at_once(hip, oracle):
+    """Two models of a shape that takes the one-launch attention half, stepping from two host threads
+    on their own streams.  Either launch may find only part of its workgroups resident while the
+    other runs; its waits are bounded, and a model whose wait ran out falls back to the separate
+    launches.  Whatever happened, both must produce the tokens they produce alone."""
+    import threading
+    cfg = make_cfg("q4_0-32kv", blocks=2, context=96)
+    prompts = [synth.prompt_tokens(cfg, 16, s) for s in (3, 4)]
+    alone = []
+    for i, p in enumerate(prompts):
+        dev = hip_model(hip, cfg, 30 + i)
+        alone.append(dev.generate(p, 48)[0].tolist())
+        assert dev.block_form == 1
+        dev.close()
+    models = [hip_model(hip, cfg, 30 + i) for i in range(2)]
+    got, errors = [None, None], []
+
+    def body(i):
+        try:
+            got[i] = models[i].generate(prompts[i], 48)[0].tolist()
+        except Exception as e:  # reported in the main thread
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=body, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not any(t.is_alive() for t in threads), "a worker did not finish"
+    assert not errors, errors
+    print("block forms after stepping side by side:", [m.block_form for m in models], flush=True)
+    for i in range(2):
+        assert models[i].block_form in (1, -1)
+        assert got[i] == alone[i], i
+        models[i].close()
