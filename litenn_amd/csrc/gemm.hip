@@ -881,10 +881,12 @@ namespace litenn_hip
 
 		constexpr size_t kLdsLimit = 160 * 1024;
 
-		template <typename F, int MT, int NG, int WAVES>
+		// KS: groups of WAVES / KS wavefronts that share a tile and split its K walk (each group has its own
+		// ring of activation buffers)
+		template <typename F, int MT, int NG, int WAVES, int KS = 1>
 		constexpr size_t gemm_lds_bytes()
 		{
-			return 3 * MT * 4 * kFragBytes + static_cast<size_t>(WAVES) * NG * 16 * 16 * weight_pieces<F>();
+			return static_cast<size_t>(KS) * 3 * MT * 4 * kFragBytes + static_cast<size_t>(WAVES) * NG * 16 * 16 * weight_pieces<F>();
 		}
 
 		// Up to three matrices of one format and width that share the activations (q/k/v, gate/up):
@@ -940,7 +942,14 @@ namespace litenn_hip
 		// GATED (two weight groups per wavefront): the second group holds the same rows of a second
 		// matrix w_up, and what is stored is silu(x . w^T) * (x . w_up^T), SwiGLU's product with its
 		// separately rounded steps (Activation.h:22-35,56-63; SwiGLU.h:63-66), to the single output y.
-		template <typename F, int MT, int NG, int WAVES, bool GATED = false>
+		// KS = 2: the workgroup's wavefronts form two groups that work on the same tile; group 0 walks the
+		// first half of the workgroup's K range and group 1 the second, each through its own three
+		// activation buffers, and group 1's accumulators are added to group 0's through LDS before the
+		// tile is stored.  A tile that gives a CU one wavefront per SIMD (64 x 64 outputs, four wavefronts)
+		// is bound by that wavefront's in-order instruction stream; this puts a second one beside it
+		// without a second product in memory.  The two groups pass the same barriers, so their ranges
+		// must hold the same number of chunks (the launcher sees to it).
+		template <typename F, int MT, int NG, int WAVES, bool GATED = false, int KS = 1>
 		__device__ __forceinline__ void gemm_q_body(const uint8_t* w, const uint8_t* w_up, float* y, int n, int block_x,
 		                                            float* partial, const uint8_t* __restrict__ xf,
 		                                            const float* __restrict__ unscale,
@@ -948,26 +957,35 @@ namespace litenn_hip
 		                                            size_t row_bytes, int grid_y)
 		{
 			constexpr int kHalfBytes = MT * 4 * kFragBytes; // one activation buffer: four steps of MT tiles
-			constexpr int kXLoads = MT * 4 / WAVES;         // 1 KB pieces a wavefront moves per half
-			static_assert(kXLoads >= 1 && kXLoads * WAVES == MT * 4, "activation pieces / wavefront split");
+			constexpr int WG = WAVES / KS;                  // wavefronts that share one K range
+			static_assert(WG * KS == WAVES && (KS == 1 || (KS == 2 && !GATED)), "K groups");
+			constexpr int kXLoads = MT * 4 / WG;            // 1 KB pieces a wavefront moves per half
+			static_assert(kXLoads >= 1 && kXLoads * WG == MT * 4, "activation pieces / wavefront split");
 			constexpr int P = weight_pieces<F>();
 			constexpr int kRowStride = 16 * P;              // bytes of one row's chunk in the slot
 			constexpr int kSlotBytes = NG * 16 * kRowStride;
 			constexpr int kWLoads = (NG * 16 * P + 63) / 64;
-			extern __shared__ __attribute__((aligned(16))) uint8_t lds[]; // [3][kHalfBytes][WAVES][kSlotBytes]
+			extern __shared__ __attribute__((aligned(16))) uint8_t lds[]; // [KS][3][kHalfBytes][WAVES][kSlotBytes]
 			const int lane = threadIdx.x & 63;
 			const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+			const int kgroup = KS == 1 ? 0 : wave / WG; // which K range of the workgroup's
+			const int wv = KS == 1 ? wave : wave % WG;  // wavefront within its group
 			const int r = lane & 15, g = lane >> 4;
 			static_assert(!GATED || NG == 2, "the gated form pairs the two weight groups of a wavefront");
-			const int n_base = (block_x * WAVES + wave) * 16 * (GATED ? 1 : NG);
+			const int n_base = (block_x * WG + wv) * 16 * (GATED ? 1 : NG);
 			const int mt_base = grid_y * MT;
 			const int chunks = k / kChunk;
-			// grid z splits the K walk: this workgroup multiplies chunks [c_begin, c_end)
-			const int c_begin = static_cast<int>(blockIdx.z) * chunks / static_cast<int>(gridDim.z);
-			const int c_end = (static_cast<int>(blockIdx.z) + 1) * chunks / static_cast<int>(gridDim.z);
+			// grid z (and the workgroup's K groups) split the K walk: these wavefronts multiply chunks
+			// [c_begin, c_end)
+			const int k_part = static_cast<int>(blockIdx.z) * KS + kgroup;
+			const int k_parts = static_cast<int>(gridDim.z) * KS;
+			const int c_begin = k_part * chunks / k_parts;
+			const int c_end = (k_part + 1) * chunks / k_parts;
+			constexpr int kXRegion = KS * 3 * kHalfBytes; // every group's three activation buffers
+			const int x_group = kgroup * 3 * kHalfBytes;  // this group's
 			const uint32_t lds_base =
 			    static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const uint8_t*)(lds)));
-			const uint32_t slot_lds = lds_base + 3 * kHalfBytes + wave * kSlotBytes;
+			const uint32_t slot_lds = lds_base + kXRegion + wave * kSlotBytes;
 			const uint32_t lane_off = lane * 16;
 
 			// ---- activation requests: piece i * WAVES + wave of the half (tile t = piece / 4, step
@@ -976,7 +994,7 @@ namespace litenn_hip
 #pragma unroll
 			for (int i = 0; i < kXLoads; ++i)
 			{
-				const int piece = i * WAVES + wave;
+				const int piece = i * WG + wv;
 				const int t = min(mt_base + (piece >> 2), m_tiles - 1);
 				x_off[i] = static_cast<uint32_t>(t * chunks) * kChunkTileBytes + (piece & 3) * kFragBytes;
 			}
@@ -984,9 +1002,9 @@ namespace litenn_hip
 #pragma unroll
 				for (int i = 0; i < kXLoads; ++i)
 				{
-					const int piece = i * WAVES + wave;
+					const int piece = i * WG + wv;
 					const uint8_t* src = xf + (x_off[i] + static_cast<uint32_t>(half) * (4 * kFragBytes));
-					const uint32_t dst = lds_base + buf_off + piece * kFragBytes;
+					const uint32_t dst = lds_base + x_group + buf_off + piece * kFragBytes;
 					asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
 					             :
 					             : "s"(dst), "v"(lane_off), "s"(src)
@@ -1035,7 +1053,7 @@ namespace litenn_hip
 #pragma unroll
 			for (int q = 0; q < NG; ++q)
 			{
-				slot_rows[q] = (lds_bytes_t)(lds) + 3 * kHalfBytes + wave * kSlotBytes + (16 * q + r) * kRowStride;
+				slot_rows[q] = (lds_bytes_t)(lds) + kXRegion + wave * kSlotBytes + (16 * q + r) * kRowStride;
 			}
 			const uint8_t* lane_rows[NG]; // for the misalignment of a chunk start
 #pragma unroll
@@ -1060,7 +1078,7 @@ namespace litenn_hip
 			u32x4 b[MT]; // fragment t of the current step until its MFMAs are issued, then of the next
 			typename F::Raw raw[NG];
 			typename F::Scale sc[NG];
-			const auto lane_x = (lds_bytes_t)(lds) + lane * 16;
+			const auto lane_x = (lds_bytes_t)(lds) + x_group + lane * 16;
 			const auto read_b = [&](int t, int buf_off, int s4) {
 				b[t] = *(lds_u32x4_t)(lane_x + buf_off + t * (4 * kFragBytes) + s4 * kFragBytes);
 			};
@@ -1218,6 +1236,42 @@ namespace litenn_hip
 			}
 			chunk(false_type{}, c);
 
+			if constexpr (KS == 2)
+			{
+				// group 1 hands its accumulators to group 0 through the activation buffers, which are idle
+				// once every wavefront has passed the first barrier; a lane's 16 bytes per accumulator lie
+				// lane by lane (no bank conflicts).  K order: group 0's range, then group 1's.
+				__syncthreads();
+				auto* const handed = reinterpret_cast<floatx4*>(lds) + (wv * (NG * MT)) * 64 + lane;
+				if (kgroup == 1)
+				{
+#pragma unroll
+					for (int q = 0; q < NG; ++q)
+					{
+#pragma unroll
+						for (int t = 0; t < MT; ++t)
+						{
+							handed[(q * MT + t) * 64] = acc[q][t];
+						}
+					}
+				}
+				__syncthreads();
+				if (kgroup == 1)
+				{
+					return;
+				}
+#pragma unroll
+				for (int q = 0; q < NG; ++q)
+				{
+#pragma unroll
+					for (int t = 0; t < MT; ++t)
+					{
+						acc[q][t] += handed[(q * MT + t) * 64];
+					}
+				}
+				static_assert(static_cast<size_t>(WG) * NG * MT * 64 * 16 <= static_cast<size_t>(kXRegion), "hand-over fits the activation buffers");
+			}
+
 			// D layout: lane holds activation row j = lane % 16 and weight rows 4 (lane / 16) + 0..3
 			const bool vec_ok = (n & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 &&
 			                    (!residual || (reinterpret_cast<uintptr_t>(residual) & 15) == 0);
@@ -1306,7 +1360,7 @@ namespace litenn_hip
 			}
 		}
 
-		template <typename F, int MT, int NG, int WAVES>
+		template <typename F, int MT, int NG, int WAVES, int KS = 1>
 		__global__ __launch_bounds__(64 * WAVES) void gemm_q_kernel(const GemmMats mats, const uint8_t* __restrict__ xf,
 		                                                             const float* __restrict__ unscale,
 		                                                             const float* __restrict__ residual, int k, int m,
@@ -1315,8 +1369,8 @@ namespace litenn_hip
 			int grid_x, grid_y;
 			gemm_grid_position(grid_x, grid_y);
 			LITENN_GEMM_PICK_MATRIX(mats, grid_x);
-			gemm_q_body<F, MT, NG, WAVES>(w, nullptr, y, n, block_x, mats.partial, xf, unscale, residual, k, m, m_tiles,
-			                              row_bytes, grid_y);
+			gemm_q_body<F, MT, NG, WAVES, false, KS>(w, nullptr, y, n, block_x, mats.partial, xf, unscale, residual, k, m,
+			                                         m_tiles, row_bytes, grid_y);
 		}
 
 		// gate (mats.w[0]) and up (mats.w[1]) projections of n[0] rows each with SwiGLU's product in the
@@ -1657,13 +1711,22 @@ namespace litenn_hip
 			hipStream_t stream;
 		};
 
-		template <typename F, int MT, int NG, int WAVES>
+		template <typename F, int MT, int NG, int WAVES, int KS = 1>
 		void launch_variant(const GemmCall& c)
 		{
-			constexpr size_t lds = gemm_lds_bytes<F, MT, NG, WAVES>();
+			if constexpr (KS > 1)
+			{
+				// the K groups of a workgroup pass the same barriers: their ranges must be equally long
+				if ((c.k / kChunk) % (c.k_splits * KS) != 0)
+				{
+					launch_variant<F, MT, NG, WAVES / KS, 1>(c);
+					return;
+				}
+			}
+			constexpr size_t lds = gemm_lds_bytes<F, MT, NG, WAVES, KS>();
 			static_assert(lds <= kLdsLimit, "LDS budget");
-			allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_q_kernel<F, MT, NG, WAVES>), lds);
-			constexpr int bn = 16 * WAVES * NG;
+			allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_q_kernel<F, MT, NG, WAVES, KS>), lds);
+			constexpr int bn = 16 * (WAVES / KS) * NG;
 			GemmMats mats;
 			mats.partial = c.partial;
 			int blocks = 0;
@@ -1676,8 +1739,8 @@ namespace litenn_hip
 				blocks += i < c.count ? (c.n[i] + bn - 1) / bn : 0;
 			}
 			const dim3 grid(blocks, (c.m_tiles + MT - 1) / MT, c.k_splits);
-			gemm_q_kernel<F, MT, NG, WAVES><<<grid, dim3(64 * WAVES), lds, c.stream>>>(mats, c.xf, c.unscale, c.residual,
-			                                                                          c.k, c.m, c.m_tiles, c.row_bytes);
+			gemm_q_kernel<F, MT, NG, WAVES, KS><<<grid, dim3(64 * WAVES), lds, c.stream>>>(mats, c.xf, c.unscale, c.residual,
+			                                                                              c.k, c.m, c.m_tiles, c.row_bytes);
 		}
 
 		// Two formats in one launch: matrices [0, second) in F0, [second, count) in F1, single-group tiles.
@@ -1739,6 +1802,9 @@ namespace litenn_hip
 			}
 		}
 
+		// tile code of the 64 x 64 tile worked by two groups of four wavefronts, each on half of K
+		constexpr int kTileTwoGroups = 2414;
+
 		// K from which splitting pays: the extra pass over y costs about 7 us
 		constexpr int kSplitMinK = 8192;
 
@@ -1796,7 +1862,31 @@ namespace litenn_hip
 					// the CUs it loses (4096 x 4096 at M = 512, 128 workgroups: 45.9 against 38.5 us)
 					pick = 818;
 				}
-				else if (split8 > 1 && 8 * blocks(8, 128) * split8 >= 5 * cus && (c.k >= kSplitMinK || split8 == 2))
+				else if (m_tiles >= 4 && gemm_lds_bytes<F, 4, 1, 8, 2>() <= kLdsLimit && blocks(4, 64) <= cus &&
+				         c.k < kSplitMinK && (c.k / kChunk) % 2 == 0 && split4 != 4)
+				{
+					// 64-row tiles that give a CU one workgroup at most: eight wavefronts in two groups, each on
+					// half of the K range, so that every SIMD has two instruction streams (the four-wavefront tile
+					// is bound by its one in-order stream per SIMD: MFMA busy 17 % of the time, 19 % in waits).
+					// Measured against the tile this replaced (us, pre-pass included), K = 4096: M = 64: Q4_K
+					// 14336 rows 23.1 against 27.1, Q4_0 12288 22.6 against 25.4; M = 128: Q4_K 8192 23.8 against
+					// 28.1, 5120 22.0 against 26.0; M = 192: Q4_K 5120 23.8 against 33.7, 4096 22.8 against 27.4;
+					// M = 256: 4096 24.7 against 28.9, Q6_K 30.3 against 34.0.  With more such tiles than CUs the
+					// four-wavefront tile has two workgroups per CU anyway and wins (M = 64, 22016 rows: 33.4
+					// against 37.2).  Two K ranges on top where they still leave a workgroup per CU (M = 64: Q4_K
+					// 5120 18.4 against 20.1, 8192 19.9 against 20.6); four ranges on the four-wavefront tile stay
+					// ahead where they fit (4096 rows at M = 64: 16.5 against 17.1), a long K keeps its ranges too
+					// (Q6_K 4096 x 14336 at M = 64: 34.5 against 43.8).
+					pick = kTileTwoGroups;
+					const int chunks = c.k / kChunk;
+					if (may_split && 2 * blocks(4, 64) <= cus && chunks % 4 == 0 && chunks >= 8 &&
+					    c.partial_floats >= static_cast<size_t>(c.m) * c.n[0])
+					{
+						c.k_splits = 2;
+					}
+				}
+				else if (split8 > 1 && 8 * blocks(8, 128) * split8 >= 5 * cus &&
+				         (c.k >= kSplitMinK || (split8 == 2 && (m_tiles + 7) / 8 * 8 - m_tiles <= m_tiles / 8)))
 				{
 					// the 128-row tile on few weight rows (N = 4096): K walked in 2 or 4 ranges by as many
 					// workgroups, the ranges' products added in K order by one more pass.  Measured (us, with the
@@ -1875,6 +1965,19 @@ namespace litenn_hip
 			const int pick = c.tile;
 			LITENN_GEMM_CASE(8, 2, 8)
 			LITENN_GEMM_CASE(8, 1, 8)
+			if constexpr (gemm_lds_bytes<F, 4, 1, 8, 2>() <= kLdsLimit)
+			{
+				if (pick == kTileTwoGroups)
+				{
+					launch_variant<F, 4, 1, 8, 2>(c);
+					return;
+				}
+			}
+			if (pick == kTileTwoGroups)
+			{
+				launch_variant<F, 4, 1, 4>(c);
+				return;
+			}
 			LITENN_GEMM_CASE(4, 1, 4)
 			LITENN_GEMM_CASE(2, 1, 4)
 			LITENN_GEMM_CASE(1, 1, 4)
@@ -2048,7 +2151,7 @@ namespace litenn_hip
 			switch (c.tile)
 			{
 			case 828: case 818: launch_pair_variant<F0, F1, 8, 8>(c, second, xf1, unscale1, row_bytes1); break;
-			case 414: launch_pair_variant<F0, F1, 4, 4>(c, second, xf1, unscale1, row_bytes1); break;
+			case 414: case kTileTwoGroups: launch_pair_variant<F0, F1, 4, 4>(c, second, xf1, unscale1, row_bytes1); break;
 			case 214: launch_pair_variant<F0, F1, 2, 4>(c, second, xf1, unscale1, row_bytes1); break;
 			default: launch_pair_variant<F0, F1, 1, 4>(c, second, xf1, unscale1, row_bytes1); break;
 			}

@@ -207,6 +207,28 @@ def test_k_ranges_on_few_weight_rows(hip, oracle, fmt, m, n, k):
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("m,n,k", [(64, 14336, 4096),    # the benchmark's 64-row case: 224 tiles, no ranges
+                                   (100, 5000, 1536),    # ragged on both sides, six chunks (three per group)
+                                   (64, 5120, 4096),     # with two K ranges on top: four chunks per group
+                                   (256, 4096, 2048)])   # one tile per CU, four row blocks
+def test_two_groups_of_wavefronts_share_a_tile(hip, oracle, fmt, m, n, k):
+    """64 x 64 output tiles that give a CU at most one workgroup are worked by eight wavefronts in two
+    groups, each on half of the tile's K range, the second group's accumulators handed to the first
+    through LDS.  Against the checker on a sample of weight rows, with a residual, and against the
+    Float32-operand path on everything."""
+    rng = np.random.default_rng(n + k)
+    rows = np.sort(rng.choice(n, 192, replace=False))
+    rows[0], rows[-1] = 0, n - 1
+    assert run_case(hip, oracle, fmt, m, n, k, seed=7, residual=True, rows=rows) <= TOL
+    wq = hip.Tensor.from_numpy(synth.quant_weights(fmt, n, k, 7, 1))
+    x = hip.Tensor.from_numpy(synth.activations(m, k, 7, 2))
+    exact = hip.mul_mat_q(fmt, wq, n, k, x, flags=MATMUL_PRECISE).numpy()
+    got = hip.mul_mat_q(fmt, wq, n, k, x).numpy()
+    assert rel_l2(got, exact) <= TOL
+    assert float(np.abs(got - exact).max()) < 0.02 * float(np.abs(exact).max())
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
 def test_many_small_workgroups_share_a_cu(hip, fmt):
     """Few activation rows against a wide matrix: small tiles, several workgroups resident on every
     CU (with room for more products the K walk is also split), so LDS traffic is at its densest.
