@@ -131,14 +131,18 @@ def bench_gemv(ln, hiprt, fmt, n, k, steps, warmup, n_buffers, seed=1, graph_rot
     # graph costs about 13 us on the device whatever it holds (measured with empty kernels: 14.4 us
     # for a graph of one, 1.58 us per kernel in a graph of 256, 1.53 us per kernel launched
     # directly), so a graph holds up to 16 rotations; exactly `steps` kernels run, all from graphs.
-    # A short run (fewer than 64 steps) is timed as the difference of two graphs: SHORT_RUN_PRIMING
-    # launches followed by the `steps` timed ones, and the SHORT_RUN_PRIMING launches alone, each
-    # between two events, the median of SHORT_RUN_REPEATS replays each.  The timed launches then
-    # follow others back to back on the device, as they do in a long run, and what every graph
-    # replay pays once (its start, the two events) cancels.  Other ways to time 20 launches, all
-    # measured: a graph of the 20 alone pays its start (8.3 us per launch where the long run gives
-    # 7.6); event nodes inside one graph of 64 + 20 launches cost about 5 us themselves (7.9 to 8.2);
-    # launched directly, one host call per kernel, the host is the limit (8.25).
+    # A short run (fewer than 64 steps) times a graph of exactly `steps` launches between two events
+    # in the middle of a busy queue: SHORT_RUN_PRIMING replays of a graph of 256 launches go first
+    # (about 16 ms: the card is then at the clocks it sustains, and the queue never runs dry), and
+    # nothing synchronises before the timed graph.  The region is taken SHORT_RUN_REPEATS times, with
+    # an untimed graph of 2 x `steps` launches between two takes, and the median is reported.
+    # Measured alternatives for 20 launches, on boxes where 3000 steps give 7.6 to 7.7 us: the graph
+    # of 20 alone after a synchronisation pays its start (8.3 us per launch); launched directly, one
+    # host call per kernel, the host is the limit (8.25); event nodes inside one graph cost about
+    # 5 us themselves (7.9 to 8.2); the difference of two graph replays (64 + 20 launches against
+    # 64), each after a synchronisation, read 6.6 us on one box and 7.5 to 7.75 on another, because
+    # the launches at the end of a replay run at clocks the card does not sustain.  This method:
+    # 7.82 to 7.88 where 3000 steps give 7.71.
     graph_len = min(steps, graph_rotations * n_buffers)
 
     def capture(count, first=0):
@@ -161,17 +165,22 @@ def bench_gemv(ln, hiprt, fmt, n, k, steps, warmup, n_buffers, seed=1, graph_rot
     short_run = steps < 64
     e0, e1 = hiprt.Event(), hiprt.Event()
     if short_run:
-        graphs = [capture(SHORT_RUN_PRIMING + steps), capture(SHORT_RUN_PRIMING)]
+        prime, timed_graph, filler = capture(256), capture(steps), capture(2 * steps)
+        graphs = [prime, timed_graph, filler]
+        marks = [hiprt.Event() for _ in range(2 * SHORT_RUN_REPEATS)]
         hiprt.device_synchronize()
         t0 = time.perf_counter()
-        both, priming = [], []
-        for _ in range(SHORT_RUN_REPEATS):  # alternating, so that a clock change touches both alike
-            both.append(timed(graphs[:1]))
-            priming.append(timed(graphs[1:]))
-        both, priming = float(np.median(both)), float(np.median(priming))
+        for _ in range(SHORT_RUN_PRIMING):
+            prime.launch(stream)
+        for r in range(SHORT_RUN_REPEATS):
+            marks[2 * r].record(stream)
+            timed_graph.launch(stream)
+            marks[2 * r + 1].record(stream)
+            filler.launch(stream)
+        stream.synchronize()
         hiprt.device_synchronize()
-        wall_launches = SHORT_RUN_REPEATS * (2 * SHORT_RUN_PRIMING + steps)
-        event_ms = both - priming
+        wall_launches = SHORT_RUN_PRIMING * 256 + SHORT_RUN_REPEATS * 3 * steps
+        event_ms = float(np.median([marks[2 * r].elapsed_ms(marks[2 * r + 1]) for r in range(SHORT_RUN_REPEATS)]))
     else:
         graphs = [capture(graph_len)] * (steps // graph_len)
         if steps % graph_len:
@@ -190,9 +199,9 @@ def bench_gemv(ln, hiprt, fmt, n, k, steps, warmup, n_buffers, seed=1, graph_rot
         w.free()
     stream.destroy()
     bench_gemv.last_mode = (f"graphs of {graph_len} launches replayed" if not short_run else
-                            f"a graph of {SHORT_RUN_PRIMING} + {steps} launches minus a graph of {SHORT_RUN_PRIMING} "
-                            f"launches, each between two events, the median of {SHORT_RUN_REPEATS} replays each "
-                            f"(the wall figure is over all of their launches, graph starts included)")
+                            f"a graph of {steps} launches between two events in a busy queue ({SHORT_RUN_PRIMING} replays of "
+                            f"a graph of 256 launches go first, nothing synchronises in between), median of "
+                            f"{SHORT_RUN_REPEATS} such regions (the wall figure is over all launches of the run)")
     return event_ms / steps, wall_ms / wall_launches
 
 
@@ -212,7 +221,7 @@ def traffic_probe(ln, launches=8, n_elems=16 * 1024 * 1024):
         f"{4 * n_elems} B written each")
 
 
-SHORT_RUN_PRIMING = 64  # launches that precede the timed ones in a short run
+SHORT_RUN_PRIMING = 8  # replays of a graph of 256 launches that precede the timed graph of a short run
 SHORT_RUN_REPEATS = 15
 
 
