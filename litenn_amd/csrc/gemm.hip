@@ -518,7 +518,7 @@ namespace litenn_hip
 			static constexpr int kChunkBytes = 176;
 			static constexpr int kFragValu = 27;
 			static constexpr bool kAligned16 = true;
-			static constexpr bool kWideTile = false;
+			static constexpr bool kWideTile = true;  // (185 VGPRs with two row groups: no spill)
 			// header (d, dmin, 12 scale bytes), the 32 fifth-bit bytes, the 32 nibble bytes of group g
 			struct Raw { u32x4 h; uint32_t qh[8]; uint32_t q[8]; };
 			struct Scale { float s0, m0, s1, m1; int shift; }; // as Q4_K; shift = 2g, the group's bit pair in qh

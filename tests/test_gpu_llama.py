@@ -143,7 +143,7 @@ def test_prompt_pass_with_a_q6_k_value_projection(hip, oracle, main_fmt, d_model
     dev.close()
 
 
-@pytest.mark.parametrize("fmt,ff,rows", [(Q4_K, 5120, 512), (Q4_0, 5024, 500)])
+@pytest.mark.parametrize("fmt,ff,rows", [(Q4_K, 5120, 512), (Q4_0, 5024, 500), (Q5_K, 5120, 400)])
 def test_prompt_pass_with_swiglu_in_the_gate_up_launch(hip, oracle, fmt, ff, rows):
     """With enough rows and a wide enough feed-forward block the gate and up projections of a prompt
     run as one matrix-core launch whose epilogue stores silu(gate) * up.  The second case has a
