@@ -221,7 +221,7 @@ namespace litenn_hip
 			static constexpr int kChunkBytes = 8 * 22;
 			static constexpr int kFragValu = 33;
 			static constexpr bool kAligned16 = true;
-			static constexpr bool kWideTile = false;
+			static constexpr bool kWideTile = true;  // (182 VGPRs with two row groups: no spill)
 			struct Raw { uint32_t w[11]; }; // blocks 2g and 2g+1: bytes 0..21 and 22..43
 			struct Scale { float d0, d1; };
 			static __device__ __forceinline__ Raw load(lds_bytes_t chunk, int g)
@@ -296,7 +296,7 @@ namespace litenn_hip
 			static constexpr int kChunkBytes = 84;
 			static constexpr int kFragValu = 24;
 			static constexpr bool kAligned16 = false; // 84-byte blocks: 4-byte aligned
-			static constexpr bool kWideTile = false;
+			static constexpr bool kWideTile = true;  // (206 VGPRs with two row groups: no spill)
 			struct Raw { uint32_t q[8]; uint32_t sc, dd; };
 			struct Scale { float s[4], b[4]; int shift; };
 			static __device__ __forceinline__ Raw load(lds_bytes_t chunk, int g)
