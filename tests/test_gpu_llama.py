@@ -7,7 +7,7 @@ import pytest
 
 from conftest import rel_l2
 from litenn_amd import synth
-from litenn_amd.formats import DT_F16, DT_F32, Q4_0, Q4_K, Q5_K, Q6_K, Q8_0
+from litenn_amd.formats import DT_F16, DT_F32, Q2_K, Q4_0, Q4_K, Q5_0, Q5_K, Q6_K, Q8_0
 from llama_util import hip_model, oracle_model, tiny_reference_archive
 
 pytestmark = pytest.mark.gpu
@@ -143,7 +143,8 @@ def test_prompt_pass_with_a_q6_k_value_projection(hip, oracle, main_fmt, d_model
     dev.close()
 
 
-@pytest.mark.parametrize("fmt,ff,rows", [(Q4_K, 5120, 512), (Q4_0, 5024, 500), (Q5_K, 5120, 400)])
+@pytest.mark.parametrize("fmt,ff,rows", [(Q4_K, 5120, 512), (Q4_0, 5024, 500), (Q5_K, 5120, 400), (Q5_0, 5088, 512),
+                                        (Q2_K, 5120, 450)])
 def test_prompt_pass_with_swiglu_in_the_gate_up_launch(hip, oracle, fmt, ff, rows):
     """With enough rows and a wide enough feed-forward block the gate and up projections of a prompt
     run as one matrix-core launch whose epilogue stores silu(gate) * up.  The second case has a
