@@ -75,6 +75,15 @@ def traffic_source():
                     "changed; not re-measured by this run"}
 
 
+def last_gemm_launch():
+    """The instance and grid of the matrix-core kernel this thread launched last, as the library reports it."""
+    import ctypes as C
+    from litenn_amd._lib import check, load
+    buf = C.create_string_buffer(256)
+    check(load().litenn_hip_gemm_last_launch(buf, len(buf)))
+    return buf.value.decode()
+
+
 def last_gemv_launch():
     """The instance and geometry of the streaming kernel this thread launched last, as the library reports it."""
     import ctypes as C
@@ -284,9 +293,9 @@ def bench_prefill_gemm(ln, hiprt, only=None):
             out.append({"format": name, "m": m, "n": n, "k": k, "us": round(ms * 1e3, 2),
                         "tflops": round(flops / (ms * 1e-3) / 1e12, 1),
                         "frac_of_fp16_mfma_peak": round(flops / (ms * 1e-3) / 1e12 / FP16_MFMA_PEAK_TFLOPS, 4),
-                        "gbps": round(bytes_ / (ms * 1e-3) / 1e9, 1)})
+                        "gbps": round(bytes_ / (ms * 1e-3) / 1e9, 1), "launch": last_gemm_launch()})
             log(f"[bench] GEMM {name} M={m} N={n} K={k}: {ms * 1e3:.1f} us, {out[-1]['tflops']} TFLOP/s, "
-                f"{out[-1]['gbps']} GB/s")
+                f"{out[-1]['gbps']} GB/s; {out[-1]['launch']}")
     return out
 
 

@@ -165,6 +165,12 @@ size_t litenn_hip_mul_mat_q_workspace_bytes(size_t m, size_t k);
  * "gemv_stream_kernel<Q4_KUnit, 2, true, 512> grid 256 x 512 threads, 83968 B LDS, runs of 8 and 6 rows"
  * ("none" before the first such launch).  The name is the one a kernel trace shows. */
 int litenn_hip_gemv_last_launch(char* out, size_t capacity);
+/* The same for the matrix cores: the calling thread's last launch for m >= 4 rows, e.g.
+ * "gemm_q_kernel<4, 1, 8, 2> grid 224 x 1 x 1, 512 threads, 118784 B LDS" (activation tiles and
+ * weight groups of a workgroup's tile, its wavefronts, the groups of them that split the tile's K
+ * range; grid z = K ranges walked by separate workgroups), "gemm_stream_kernel<1, 1, 16> ..." for
+ * the streaming form of few rows.  No reference counterpart. */
+int litenn_hip_gemm_last_launch(char* out, size_t capacity);
 int litenn_hip_mul_mat_q_ws(int dev, int fmt, const void* wq, size_t n, size_t k, const void* x, int x_dtype, size_t m,
                             void* y, const void* residual, unsigned flags, void* workspace, size_t workspace_bytes,
                             const litenn_hip_exec* opts);

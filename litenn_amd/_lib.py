@@ -69,6 +69,7 @@ SIGNATURES = {
     "litenn_hip_mul_mat_q": [_i, _i, _vp, _sz, _sz, _vp, _i, _sz, _vp, _vp, _u, _ex],
     "litenn_hip_mul_mat_q_workspace_bytes": [_sz, _sz],
     "litenn_hip_gemv_last_launch": [C.c_char_p, _sz],
+    "litenn_hip_gemm_last_launch": [C.c_char_p, _sz],
     "litenn_hip_mul_mat_q_ws": [_i, _i, _vp, _sz, _sz, _vp, _i, _sz, _vp, _vp, _u, _vp, _sz, _ex],
     "litenn_hip_linear_group": [_i, _i, _sz, C.POINTER(_vp), _szp, _sz, _vp, C.POINTER(_vp), _vp, _vp, _d, _u, _ex],
     "litenn_hip_dequantize": [_i, _i, _vp, _sz, _sz, _vp, _ex],

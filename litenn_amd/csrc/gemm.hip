@@ -23,6 +23,8 @@
 #include "fetch_model.hpp"
 
 #include <algorithm>
+#include <cstdio>
+#include <cstring>
 #include <type_traits>
 
 namespace litenn_hip
@@ -1693,6 +1695,16 @@ namespace litenn_hip
 
 #pragma clang diagnostic pop
 
+		// What the calling thread's last matrix-core launch was (litenn_hip_gemm_last_launch formats it)
+		struct GemmLaunchRecord
+		{
+			const char* kernel = nullptr; // gemm_q_kernel, gemm_q_pair_kernel, gemm_q_gated_kernel or gemm_stream_kernel
+			int a = 0, b = 0, c = 0, d = 0; // the instance's integer template arguments (d: K groups of a tile, 0 where there is none)
+			unsigned grid_x = 0, grid_y = 0, grid_z = 0, threads = 0;
+			size_t lds = 0;
+		};
+		thread_local GemmLaunchRecord t_last_gemm_launch;
+
 		struct GemmCall
 		{
 			int count;
@@ -1739,6 +1751,7 @@ namespace litenn_hip
 				blocks += i < c.count ? (c.n[i] + bn - 1) / bn : 0;
 			}
 			const dim3 grid(blocks, (c.m_tiles + MT - 1) / MT, c.k_splits);
+			t_last_gemm_launch = { "gemm_q_kernel", MT, NG, WAVES, KS, grid.x, grid.y, grid.z, 64u * WAVES, lds };
 			gemm_q_kernel<F, MT, NG, WAVES, KS><<<grid, dim3(64 * WAVES), lds, c.stream>>>(mats, c.xf, c.unscale, c.residual,
 			                                                                              c.k, c.m, c.m_tiles, c.row_bytes);
 		}
@@ -1764,6 +1777,7 @@ namespace litenn_hip
 				blocks += i < c.count ? (c.n[i] + bn - 1) / bn : 0;
 			}
 			const dim3 grid(blocks, (c.m_tiles + MT - 1) / MT, 1);
+			t_last_gemm_launch = { "gemm_q_pair_kernel", MT, 1, WAVES, 0, grid.x, grid.y, grid.z, 64u * WAVES, lds };
 			gemm_q_pair_kernel<F0, F1, MT, 1, WAVES><<<grid, dim3(64 * WAVES), lds, c.stream>>>(
 			    mats, mats.first_block[second], c.xf, xf1, c.unscale, unscale1, c.k, c.m, c.m_tiles, c.row_bytes, row_bytes1);
 		}
@@ -2020,6 +2034,8 @@ namespace litenn_hip
 				a.round_tiles = round;
 				const size_t lds = slots + round * per_round_tile;
 				allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_stream_kernel<F, MT, CPW, kStreamWaves>), kLdsLimit);
+				t_last_gemm_launch = { "gemm_stream_kernel", MT, CPW, kStreamWaves, 0, static_cast<unsigned>(blocks), 1u, 1u,
+					                   64u * kStreamWaves, lds };
 				gemm_stream_kernel<F, MT, CPW, kStreamWaves><<<dim3(blocks), dim3(64 * kStreamWaves), lds, c.stream>>>(a);
 				return true;
 			}
@@ -2135,6 +2151,7 @@ namespace litenn_hip
 				mats.y[0] = c.y[0];
 				mats.n[0] = c.n[0];
 				const dim3 grid((c.n[0] + 127) / 128, (c.m_tiles + 7) / 8, 1);
+				t_last_gemm_launch = { "gemm_q_gated_kernel", 8, 8, 0, 0, grid.x, grid.y, grid.z, 512u, lds };
 				gemm_q_gated_kernel<F, 8, 8><<<grid, dim3(512), lds, c.stream>>>(mats, c.xf, c.unscale, c.k, c.m, c.m_tiles,
 				                                                                c.row_bytes);
 				return true;
@@ -2427,3 +2444,38 @@ namespace litenn_hip
 		                         partial_floats, stream);
 	}
 } // namespace litenn_hip
+
+extern "C" int litenn_hip_gemm_last_launch(char* out, size_t capacity)
+{
+	using namespace litenn_hip;
+	if (!out || capacity == 0)
+	{
+		return fail("describe the last matrix-core launch", "destination is null or empty");
+	}
+	const GemmLaunchRecord& r = t_last_gemm_launch;
+	if (!r.kernel)
+	{
+		std::snprintf(out, capacity, "none");
+		return 0;
+	}
+	char args[64];
+	if (std::strcmp(r.kernel, "gemm_q_kernel") == 0)
+	{
+		std::snprintf(args, sizeof args, "%d, %d, %d, %d", r.a, r.b, r.c, r.d);
+	}
+	else if (std::strcmp(r.kernel, "gemm_q_gated_kernel") == 0)
+	{
+		std::snprintf(args, sizeof args, "%d, %d", r.a, r.b);
+	}
+	else if (std::strcmp(r.kernel, "gemm_q_pair_kernel") == 0)
+	{
+		std::snprintf(args, sizeof args, "%d, %d, %d", r.a, r.b, r.c);
+	}
+	else
+	{
+		std::snprintf(args, sizeof args, "%d, %d, %d", r.a, r.b, r.c);
+	}
+	std::snprintf(out, capacity, "%s<%s> grid %u x %u x %u, %u threads, %zu B LDS", r.kernel, args, r.grid_x, r.grid_y,
+	              r.grid_z, r.threads, r.lds);
+	return 0;
+}

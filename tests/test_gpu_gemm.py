@@ -19,6 +19,15 @@ TOL = 1e-3
 FORMATS = [Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K]
 
 
+def last_gemm_launch():
+    """The instance and grid of the calling thread's last matrix-core launch, as the library reports it."""
+    import ctypes as C
+    from litenn_amd._lib import check, load
+    buf = C.create_string_buffer(256)
+    check(load().litenn_hip_gemm_last_launch(buf, len(buf)))
+    return buf.value.decode()
+
+
 def run_case(hip, oracle, fmt, m, n, k, seed=0, residual=False, rows=None, flags=0):
     """rows: compare only these weight rows (they are independent), to bound the checker's time."""
     wq = synth.quant_weights(fmt, n, k, seed, 1)
@@ -165,6 +174,8 @@ def check_k_ranges(hip, oracle, fmt, m, n, k, products):
                                           C.byref(opts)))
         outs.append(y.numpy())
     plain, split = outs
+    import re
+    assert int(re.search(r"grid \d+ x \d+ x (\d+)", last_gemm_launch()).group(1)) > 1, last_gemm_launch()  # K in ranges
     assert rel_l2(split - res, plain - res) < 1e-5
     assert not np.array_equal(split, plain)  # the ranges ran
     y = hip.Tensor.from_numpy(res)
@@ -224,8 +235,13 @@ def test_two_groups_of_wavefronts_share_a_tile(hip, oracle, fmt, m, n, k):
     x = hip.Tensor.from_numpy(synth.activations(m, k, 7, 2))
     exact = hip.mul_mat_q(fmt, wq, n, k, x, flags=MATMUL_PRECISE).numpy()
     got = hip.mul_mat_q(fmt, wq, n, k, x).numpy()
+    launch = last_gemm_launch()
     assert rel_l2(got, exact) <= TOL
     assert float(np.abs(got - exact).max()) < 0.02 * float(np.abs(exact).max())
+    # the tile this test is about ran (on a card of 256 CUs; the rule counts tiles against CUs)
+    if "256 CUs" in hip.DeviceTraits.Info(hip.HIP(0)):
+        assert launch.startswith("gemm_q_kernel<4, 1, 8, 2>"), launch
+        assert ("x 2," in launch) == ((m, n, k) == (64, 5120, 4096)), launch  # two K ranges for that case only
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
