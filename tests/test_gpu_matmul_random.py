@@ -50,3 +50,38 @@ def test_random_matmul_matches_checker(hip, oracle, seed):
     # f32 operands (fewer than 4 rows, a K that is no whole number of 256-element chunks, or the flag):
     # summation order only; matrix cores: the stated bar for Float16 operands
     assert err <= (1e-5 if (m < 4 or precise) else 1e-3), what
+
+
+def draw_tile_case(seed):
+    """Shapes on both sides of the tile rules of the tiled matrix-core form: 64 and 128-row tiles, one or
+    two weight groups, two groups of wavefronts per tile, K walked in one, two or four ranges."""
+    rng = np.random.default_rng(5000 + seed)
+    fmt = FORMATS[seed % len(FORMATS)]
+    k = int(rng.choice([1024, 1536, 2048, 4096, 4352, 8192, 11008]))
+    m = int(rng.choice([49, 64, 65, 96, 128, 130, 192, 256, 300, 512, 600]))
+    n = int(rng.choice([1024, 2048, 4096, 5120, 8192, 12288, 14336, 22016, 4100, 13000]))
+    if m * n * k > 512 * 14336 * 4096:
+        n = 4096
+    return fmt, m, n, k, bool(rng.integers(2))
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_tiles_match_the_float32_path(hip, seed):
+    """The matrix-core product against the device's own Float32-operand path (held to the CPU checker by
+    the tests above), so that large shapes stay cheap: within the Float16-operand bar overall and with no
+    outlier element, with and without a residual."""
+    fmt, m, n, k, residual = draw_tile_case(seed)
+    what = f"seed {seed}: format {fmt} m {m} n {n} k {k} residual {residual}"
+    print(what, flush=True)
+    wq = hip.Tensor.from_numpy(synth.quant_weights(fmt, n, k, seed, 1))
+    x = hip.Tensor.from_numpy(synth.activations(m, k, seed, 2))
+    res = hip.Tensor.from_numpy(synth.activations(m, n, seed, 3)) if residual else None
+    exact = hip.mul_mat_q(fmt, wq, n, k, x, residual=res, flags=MATMUL_PRECISE).numpy()
+    got = hip.mul_mat_q(fmt, wq, n, k, x, residual=res).numpy()
+    import ctypes as C
+    from litenn_amd._lib import check, load
+    buf = C.create_string_buffer(256)
+    check(load().litenn_hip_gemm_last_launch(buf, len(buf)))
+    print("  " + buf.value.decode(), flush=True)
+    assert rel_l2(got, exact) <= 1e-3, what
+    assert float(np.abs(got - exact).max()) < 0.02 * float(np.abs(exact).max()), what
