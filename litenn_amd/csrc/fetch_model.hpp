@@ -178,6 +178,24 @@ namespace litenn_hip
 			return { q / seg_pieces, static_cast<uint32_t>(q % seg_pieces) * 16u, p < total };
 		}
 
+		// ---- tiled GEMM: the chunks of K a group of wavefronts walks ------------------------------
+		// K (in 256-element chunks) is cut into `parts` consecutive ranges: grid z x the K groups of a
+		// workgroup, part = blockIdx.z * groups + group
+		struct ChunkRange
+		{
+			int begin, end;
+		};
+		LITENN_FETCH_FN ChunkRange gemm_chunk_range(int part, int parts, int chunks)
+		{
+			return { part * chunks / parts, (part + 1) * chunks / parts };
+		}
+		// The K groups of one workgroup pass the same barriers, one set per chunk: a launch with more than
+		// one group per workgroup is only made when this holds (every range is then equally long)
+		LITENN_FETCH_FN bool gemm_ranges_equal(int chunks, int parts)
+		{
+			return parts > 0 && chunks >= parts && chunks % parts == 0;
+		}
+
 		// ---- tiled prompt attention: key / value rows of a 64-key tile -------------------------
 		// keys any query row of the 64-row tile starting at q_first may see
 		LITENN_FETCH_FN int attn_tile_kv_len(int past, int q_first, int q_tile, int m)

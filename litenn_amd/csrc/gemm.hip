@@ -981,8 +981,9 @@ namespace litenn_hip
 			// [c_begin, c_end)
 			const int k_part = static_cast<int>(blockIdx.z) * KS + kgroup;
 			const int k_parts = static_cast<int>(gridDim.z) * KS;
-			const int c_begin = k_part * chunks / k_parts;
-			const int c_end = (k_part + 1) * chunks / k_parts;
+			const fetch::ChunkRange my_chunks = fetch::gemm_chunk_range(k_part, k_parts, chunks);
+			const int c_begin = my_chunks.begin;
+			const int c_end = my_chunks.end;
 			constexpr int kXRegion = KS * 3 * kHalfBytes; // every group's three activation buffers
 			const int x_group = kgroup * 3 * kHalfBytes;  // this group's
 			const uint32_t lds_base =
@@ -1729,7 +1730,7 @@ namespace litenn_hip
 			if constexpr (KS > 1)
 			{
 				// the K groups of a workgroup pass the same barriers: their ranges must be equally long
-				if ((c.k / kChunk) % (c.k_splits * KS) != 0)
+				if (!fetch::gemm_ranges_equal(c.k / kChunk, c.k_splits * KS))
 				{
 					launch_variant<F, MT, NG, WAVES / KS, 1>(c);
 					return;

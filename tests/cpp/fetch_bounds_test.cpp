@@ -584,8 +584,54 @@ static void test_team_rows_and_segments()
 	std::printf("team rows and column segments: %ld rows and pieces walked\n", cases);
 }
 
+// The K ranges of the tiled GEMM: whatever the split, the ranges tile [0, chunks) in order; and
+// whenever the launcher's condition for several groups per workgroup holds, the groups of every
+// workgroup walk equally many chunks (they pass one set of barriers per chunk: an unequal walk would
+// leave a group waiting at a barrier the other never reaches).
+static void test_gemm_chunk_ranges()
+{
+	using namespace litenn_hip::fetch;
+	long walked = 0;
+	for (int chunks = 1; chunks <= 96; ++chunks)
+	{
+		for (int grid_z = 1; grid_z <= 4; grid_z *= 2)
+		{
+			for (int groups = 1; groups <= 2; ++groups)
+			{
+				const int parts = grid_z * groups;
+				int expect_begin = 0;
+				for (int part = 0; part < parts; ++part)
+				{
+					const ChunkRange r = gemm_chunk_range(part, parts, chunks);
+					CHECK(r.begin == expect_begin && r.end >= r.begin && r.end <= chunks, "chunks %d parts %d part %d: [%d, %d)",
+					      chunks, parts, part, r.begin, r.end);
+					expect_begin = r.end;
+					walked += r.end - r.begin;
+				}
+				CHECK(expect_begin == chunks, "chunks %d parts %d: ranges end at %d", chunks, parts, expect_begin);
+				if (groups > 1 && gemm_ranges_equal(chunks, parts))
+				{
+					for (int z = 0; z < grid_z; ++z)
+					{
+						const ChunkRange g0 = gemm_chunk_range(z * groups, parts, chunks);
+						const ChunkRange g1 = gemm_chunk_range(z * groups + 1, parts, chunks);
+						CHECK(g0.end - g0.begin == g1.end - g1.begin && g0.end > g0.begin,
+						      "chunks %d grid z %d: groups of workgroup %d walk %d and %d chunks", chunks, grid_z, z,
+						      g0.end - g0.begin, g1.end - g1.begin);
+					}
+				}
+			}
+		}
+	}
+	// an odd chunk count must not pass the launcher's condition
+	CHECK(!gemm_ranges_equal(43, 2) && !gemm_ranges_equal(6, 4) && gemm_ranges_equal(16, 4) && !gemm_ranges_equal(1, 2),
+	      "the condition for several groups per workgroup");
+	std::printf("tiled GEMM K ranges: %ld chunks walked\n", walked);
+}
+
 int main()
 {
+	test_gemm_chunk_ranges();
 	test_gemm_weight_pieces();
 	test_gemm_stream_pieces();
 	test_stream_rows_and_pieces();
