@@ -1865,7 +1865,13 @@ namespace litenn_hip
 				// (the wide tile, too, from 5/8 of the CUs on: 22016 x 4096 at M = 256, 172 workgroups,
 				// 74.9 against 84.7 us; 12288 x 4096 at M = 512, 192: 78.9 against 86.2; 5120 x 4096 at
 				// M = 1024, 160: 77.7 against 87.9; at half the CUs and below the narrower tiles win)
-				if (m_tiles >= 8 && F::kWideTile && 8 * blocks(8, 256) >= 5 * cus)
+				// (and where the 128 x 128 tiles would need a second round of workgroups that the wide ones,
+				// on at least half of the CUs, do not: 12288 x 4096 at M = 384, 144 wide workgroups against 288,
+				// 72.3 against 81.8 us; 14336 x 4096 at M = 384: 73.6 against 85.5)
+				const auto rounds = [&](long workgroups) { return (workgroups + cus - 1) / cus; };
+				if (m_tiles >= 8 && F::kWideTile &&
+				    (8 * blocks(8, 256) >= 5 * cus ||
+				     (2 * blocks(8, 256) >= cus && 10 * rounds(blocks(8, 256)) <= 7 * rounds(blocks(8, 128)))))
 				{
 					pick = 828;
 				}
